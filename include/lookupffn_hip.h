@@ -1,0 +1,172 @@
+/*
+ * lookupffn_hip.h -- C ABI of the MI355X (gfx950) LookupFFN kernel library.
+ *
+ * One shared library (liblookupffn_hip.so), plain C linkage, raw device
+ * pointers, sizes as int64_t, a hipStream_t passed as void*.  No C++ types and
+ * no torch types cross this boundary.  The entry points are what the reference's
+ * three pybind modules bind for this path (paths relative to the reference
+ * checkout, PL/ = src/roberta/models/prenorm_lookup/):
+ *
+ *   fast_hadamard_transform_kernel  PL/bh4/fast_hadamard_transform/extension/torch_extension.cpp:30-32
+ *   gather_add                      PL/gather/cuda/extension/torch_extension.cpp:91-96
+ *   ccs_cpu                         PL/compute_code_score/torch_extension.cc:45
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer to a contiguous row-major array that the
+ *     caller owns.  The library allocates nothing, frees nothing and keeps no
+ *     state between calls.
+ *   - Forward outputs are fully overwritten (no zero-initialisation needed).
+ *     Only lffn_scatter_add_f32 accumulates into its output.
+ *   - Calls are asynchronous on `stream` (NULL = the legacy default stream) and
+ *     may be issued from any host thread.
+ *   - Return value: LFFN_OK, or a negative LFFN_ERR_* code.  Nothing throws or
+ *     aborts.  lffn_error_string() names a code.
+ *   - Indices are never trusted: a row index outside [0, source_size) is clamped
+ *     into range inside the kernels, so a bad index gives a wrong value, not a
+ *     memory fault.
+ */
+#ifndef LOOKUPFFN_HIP_H
+#define LOOKUPFFN_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LFFN_OK               0
+#define LFFN_ERR_BAD_ARG     -1   /* null pointer, negative size, misaligned pointer */
+#define LFFN_ERR_UNSUPPORTED -2   /* a shape outside what the kernels are built for */
+#define LFFN_ERR_LAUNCH      -3   /* hipGetLastError() after the launch was not hipSuccess */
+
+#define LFFN_ABI_VERSION 1
+
+/* ABI version of the loaded library (LFFN_ABI_VERSION at build time). */
+int lffn_version(void);
+
+/* Static, human-readable name of a return code. */
+const char *lffn_error_string(int code);
+
+/* ---------------------------------------------------------------- projection */
+
+/*
+ * out[b,:] = in[b,:] . H_D, unnormalised Sylvester (natural) order, fp32.
+ * in, out: [B, D]; D a power of two, 4 <= D <= 1024.  in == out is allowed.
+ * Replaces fast_hadamard_transform (fast_hadamard_transform/extension/cuda_launch.cu:56-78,
+ * kernel cuda_kernel.cu:219-257); the transform is its own transpose, so the
+ * same call is the backward (fast_hadamard_transform/kernel.py:47-54).
+ */
+int lffn_fht_f32(const float *in, float *out, int64_t B, int64_t D, void *stream);
+
+/*
+ * BH4 mixing with block size 1 (a diagonal scale before every transform):
+ *   for r < R:  y = pad(x);  for j < J:  y = FHT(diag[r,j,:] * y);  out[b, r*D:(r+1)*D] = y
+ * x: [B, H] with H <= D (zero-padded on load, PL/lookup.py:32-34); diag: [R, J, D];
+ * out: [B, R*D].  Replaces bh4_cuda (PL/bh4/kernel.py:23-36) for weight
+ * [R, J, D, 1, 1], where the einsum "bni,noi->bno" (":32") is an element-wise product.
+ */
+int lffn_bh4_diag_f32(const float *x, const float *diag, float *out,
+                      int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, void *stream);
+
+/*
+ * The whole hashing front-end of the layer in one pass over x, for block size 1
+ * and 8-bit codes (PL/lookup.py:29-39,64-77 + PL/compute_code_score/kernel.py:43-55):
+ *   y      = bh4_diag(x)                                   (as above)
+ *   z      = decay * y + residual * tile(pad(x), R)        (PL/lookup.py:36)
+ *   z      = z[:, :T*8] + proj_bias                        (PL/lookup.py:37)
+ *   code   = sum_d (z[b,t,d] > 0) << (7-d)   int32         (compute_code_score/kernel.py:32-34,47-48)
+ *   score  = sum_d |z| / prod_d (1 + exp(-2|z|))           (compute_code_score/kernel.py:51-53)
+ * x: [B, H]; diag: [R, J, D]; proj_bias: [T*8] or NULL; z_out: [B, T*8] or NULL
+ * (written only when non-NULL: the backward of the score needs it);
+ * codes: [B, T] int32; scores: [B, T].  Requires T*8 <= R*D and D >= 8.
+ * `residual` is passed separately from `decay` so that the caller decides how
+ * 1 - decay is rounded (torch rounds the python double to fp32).
+ */
+int lffn_project_hash_f32(const float *x, const float *diag, const float *proj_bias,
+                          float *z_out, int32_t *codes, float *scores,
+                          int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
+                          float decay, float residual, void *stream);
+
+/* ---------------------------------------------------------------- code + score */
+
+/*
+ * Per (token, table) n < N = B*T, over k consecutive values of z (1 <= k <= 24):
+ *   codes[n]  = sum_d (z[n,d] > 0) << (k-1-d)      (MSB first, strict >)
+ *   scores[n] = sum_d |z[n,d]| / prod_d (1 + exp(-2 |z[n,d]|))   (d ascending)
+ * Replaces ccs_cpu.compute_code_score (PL/compute_code_score/torch_extension.cc:14-42)
+ * and the eight torch ops of compute_code_score_torch (PL/compute_code_score/kernel.py:43-55).
+ */
+int lffn_code_score_f32(const float *z, int32_t *codes, float *scores,
+                        int64_t N, int64_t k, void *stream);
+
+/*
+ * g_z[n,j] = g_score[n] * d score[n] / d z[n,j]
+ *          = g_score[n] * sgn(z_j) * (1 + S * 2 e_j / (1 + e_j)) / P,
+ *   e_j = exp(-2|z_j|), S = sum|z|, P = prod(1 + e).   sgn(0) = 0 as in torch.
+ * The reference leaves this to autograd over PL/compute_code_score/kernel.py:51-53
+ * (its ComputeCodeScore.backward raises NotImplementedError, kernel.py:63-65).
+ */
+int lffn_code_score_bwd_f32(const float *z, const float *g_score, float *g_z,
+                            int64_t N, int64_t k, void *stream);
+
+/* ---------------------------------------------------------------- gather-add */
+
+/*
+ * out[b,:] = sum_i w[b,i] * src[idx[b,i],:], fp32 accumulation, i ascending.
+ * idx: [B, I] int32; src: [source_size, Dv]; w: [B, I]; out: [B, Dv]; Dv % 64 == 0.
+ * Replaces gather_add.weighted_vector_gather_add_fp32
+ * (PL/gather/cuda/extension/gather_fp32.cu:6-36, kernel gather_kernel_fp32.cu:3-47).
+ */
+int lffn_gather_add_f32(const int32_t *idx, const float *src, const float *w, float *out,
+                        int64_t B, int64_t I, int64_t source_size, int64_t Dv, void *stream);
+
+/*
+ * Same with rows stored as bfloat16 (raw 16-bit patterns) and fp32 weights,
+ * accumulation and output.  Takes the place of the reference's fp16 variant
+ * (gather_fp16.cu:9-39), which stores and accumulates in fp16.
+ */
+int lffn_gather_add_bf16(const int32_t *idx, const uint16_t *src, const float *w, float *out,
+                         int64_t B, int64_t I, int64_t source_size, int64_t Dv, void *stream);
+
+/*
+ * The gather as LookupFFN.gather issues it (PL/lookup.py:120-130): one index per
+ * table, idx[b,t] = code[b,t] + t*S folded in, optional bias (PL/lookup.py:108):
+ *   out[b,:] = bias + sum_t score[b,t] * tables[t, code[b,t] & (S-1), :]
+ * code: [B, T] int32; score: [B, T]; tables: [T, S, Do]; bias: [Do] or NULL;
+ * out: [B, Do].  S a power of two, Do % 64 == 0.  Table-major: a slice of each
+ * table is staged in LDS and consumed by a block of tokens.
+ */
+int lffn_lookup_gather_f32(const int32_t *code, const float *score, const float *tables,
+                           const float *bias, float *out,
+                           int64_t B, int64_t T, int64_t S, int64_t Do, void *stream);
+
+/* bfloat16 tables, fp32 accumulate; otherwise as lffn_lookup_gather_f32. */
+int lffn_lookup_gather_bf16(const int32_t *code, const float *score, const uint16_t *tables,
+                            const float *bias, float *out,
+                            int64_t B, int64_t T, int64_t S, int64_t Do, void *stream);
+
+/*
+ * out[b,i] = <g[b,:], src[idx[b,i],:]>   (gradient w.r.t. the weights).
+ * g: [B, Dv]; src: [source_size, Dv]; out: [B, I].
+ * Replaces gather_add.indexed_inner_product_fp32 (gather_fp32.cu:69-98,
+ * kernel gather_kernel_fp32.cu:94-157).
+ */
+int lffn_indexed_inner_product_f32(const int32_t *idx, const float *g, const float *src, float *out,
+                                   int64_t B, int64_t I, int64_t source_size, int64_t Dv, void *stream);
+
+/*
+ * out[idx[b,i],:] += w[b,i] * g[b,:]     (gradient w.r.t. the table rows).
+ * g: [B, Dv]; w: [B, I]; out: [out_size, Dv], ACCUMULATED INTO: zero it first
+ * for a plain gradient (the reference pre-zeroes it in Python,
+ * PL/gather/cuda/kernel.py:162).  fp32 atomics: the order of additions, and so the
+ * last bits of the result, vary from run to run, as in the reference
+ * (gather_kernel_fp32.cu:88).
+ * Replaces gather_add.weighted_vector_scatter_add_fp32 (gather_fp32.cu:38-67).
+ */
+int lffn_scatter_add_f32(const int32_t *idx, const float *g, const float *w, float *out,
+                         int64_t B, int64_t I, int64_t out_size, int64_t Dv, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LOOKUPFFN_HIP_H */

@@ -1,0 +1,303 @@
+// Projection kernels of the LookupFFN layer for gfx950: fast Hadamard transform,
+// BH4 mixing with block size 1 (diagonal scale + transform, repeated), and the
+// fused projection -> mix -> bias -> 8-bit code + score front-end.
+//
+// One row (or, for D < 256, 256/D rows) lives in the registers of one 64-lane
+// wavefront for the whole computation: nothing is staged in LDS and nothing
+// round-trips through memory between the transforms.
+//
+// Register layout.  A lane holds NJ float4; value c of float4 j of row-lane lr is
+// element  e = 256*j + 4*lr + c.  So bits 0-1 of e are in-register (c), bits 2..
+// are the lane, and bits 8-9 are in-register again (j).  Every global access is a
+// fully coalesced 16-byte-per-lane access.  A butterfly over an in-register bit is
+// two plain adds; over a lane bit it is one cross-lane move (DPP for lane xor
+// 1,2,4,8; ds_swizzle for 16; ds_bpermute for 32) plus one fma with +-1.
+//
+// Stage order is stride D/2 first, stride 1 last, each stage a single rounded
+// add/subtract: the same operations in the same order as the reference kernel
+// (fast_hadamard_transform/extension/cuda_kernel.cu:235-251), so results agree
+// bit for bit with a scalar butterfly in that order.
+#include "lffn_common.h"
+
+#include <type_traits>
+
+// Keep mul and add separate where the reference computes them separately (the
+// diagonal scale, the decay/residual mix): explicit fmaf calls below stay fused.
+#pragma clang fp contract(off)
+
+namespace {
+
+template <int LOGD>
+struct FhtCfg {
+    static constexpr int D = 1 << LOGD;
+    static constexpr int LPR = D >= 256 ? 64 : D / 4;   // lanes per row
+    static constexpr int NJ = D >= 256 ? D / 256 : 1;   // float4 per lane
+    static constexpr int RPW = 64 / LPR;                // rows per wavefront
+    static_assert(LOGD >= 2 && LOGD <= 10, "FHT dims 4..1024");
+};
+
+template <int M, int LPR, int NJ>
+__device__ __forceinline__ void lane_stage(float (&v)[NJ][4], int lr) {
+    if constexpr (M >= 1 && M < LPR) {
+        const float sgn = (lr & M) ? -1.0f : 1.0f;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) v[j][c] = butterfly_xor<M>(v[j][c], sgn);
+    }
+}
+
+template <int LOGD>
+__device__ __forceinline__ void fht_rows(float (&v)[FhtCfg<LOGD>::NJ][4], int lr) {
+    using C = FhtCfg<LOGD>;
+    constexpr int NJ = C::NJ;
+    // strides 512 and 256: across the float4s of a lane
+    if constexpr (NJ == 4) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                float a = v[j][c], b = v[j + 2][c];
+                v[j][c] = a + b;
+                v[j + 2][c] = a - b;
+            }
+    }
+    if constexpr (NJ >= 2) {
+#pragma unroll
+        for (int j = 0; j < NJ; j += 2)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                float a = v[j][c], b = v[j + 1][c];
+                v[j][c] = a + b;
+                v[j + 1][c] = a - b;
+            }
+    }
+    // strides 4*32 .. 4*1: across lanes
+    lane_stage<32, C::LPR, NJ>(v, lr);
+    lane_stage<16, C::LPR, NJ>(v, lr);
+    lane_stage<8, C::LPR, NJ>(v, lr);
+    lane_stage<4, C::LPR, NJ>(v, lr);
+    lane_stage<2, C::LPR, NJ>(v, lr);
+    lane_stage<1, C::LPR, NJ>(v, lr);
+    // strides 2 and 1: inside a float4
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        float a0 = v[j][0], a1 = v[j][1], a2 = v[j][2], a3 = v[j][3];
+        float b0 = a0 + a2, b2 = a0 - a2, b1 = a1 + a3, b3 = a1 - a3;
+        v[j][0] = b0 + b1;
+        v[j][1] = b0 - b1;
+        v[j][2] = b2 + b3;
+        v[j][3] = b2 - b3;
+    }
+}
+
+struct ProjectArgs {
+    const float *x;       // [B, H]
+    const float *diag;    // [R, J, D] or null (no scale)
+    const float *pbias;   // [out_cols] or null
+    float *out;           // [B, out_stride] or null
+    int32_t *codes;       // [B, T] (HASH only)
+    float *scores;        // [B, T] (HASH only)
+    int64_t B;
+    int H;                // valid input columns (<= D)
+    int R, J;
+    int out_stride;       // row stride of out
+    int out_cols;         // columns of the R*D-wide result that exist (T*8 when hashing)
+    int T;
+    float decay, residual;
+    int mix;              // 1: out = decay*y + residual*x (+ bias); 0: out = y
+    int vec_in;           // x rows are 16-byte aligned and H % 4 == 0
+};
+
+// Local part of the score recurrence over the four values of one float4:
+// s <- s + |z_c|, p <- p * (1 + exp(-2|z_c|)), c ascending.
+__device__ __forceinline__ void score_chain(const float (&z)[4], float &s, float &p) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const float a = fabsf(z[c]);
+        s = s + a;
+        p = p * (1.0f + expf(-2.0f * a));
+    }
+}
+
+template <int LOGD, bool HASH>
+__global__ __launch_bounds__(256) void project_kernel(ProjectArgs a) {
+    using C = FhtCfg<LOGD>;
+    constexpr int D = C::D, NJ = C::NJ, LPR = C::LPR, RPW = C::RPW;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int lr = lane % LPR;
+    const int64_t row = (int64_t(blockIdx.x) * 4 + wave) * RPW + lane / LPR;
+    const bool live = row < a.B;
+
+    float orig[NJ][4];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        const int e0 = 256 * j + 4 * lr;
+        float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (live) {
+            if (a.vec_in) {
+                if (e0 < a.H) t = *reinterpret_cast<const float4 *>(a.x + row * a.H + e0);
+            } else {
+                const float *p = a.x + row * a.H;
+                if (e0 + 0 < a.H) t.x = p[e0 + 0];
+                if (e0 + 1 < a.H) t.y = p[e0 + 1];
+                if (e0 + 2 < a.H) t.z = p[e0 + 2];
+                if (e0 + 3 < a.H) t.w = p[e0 + 3];
+            }
+        }
+        orig[j][0] = t.x; orig[j][1] = t.y; orig[j][2] = t.z; orig[j][3] = t.w;
+    }
+
+    for (int r = 0; r < a.R; ++r) {
+        float v[NJ][4];
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) v[j][c] = orig[j][c];
+
+        for (int s = 0; s < a.J; ++s) {
+            if (a.diag) {
+                const float *dg = a.diag + (int64_t(r) * a.J + s) * D;
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    const float4 w = *reinterpret_cast<const float4 *>(dg + 256 * j + 4 * lr);
+                    v[j][0] = v[j][0] * w.x;
+                    v[j][1] = v[j][1] * w.y;
+                    v[j][2] = v[j][2] * w.z;
+                    v[j][3] = v[j][3] * w.w;
+                }
+            }
+            fht_rows<LOGD>(v, lr);
+        }
+
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const int e0 = 256 * j + 4 * lr;
+            const int col = r * D + e0;            // column in the R*D-wide result
+            const bool in_cols = col < a.out_cols; // out_cols % 4 == 0: all four or none
+            float z[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) z[c] = v[j][c];
+            if (a.mix) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const float m0 = a.decay * z[c];
+                    const float m1 = a.residual * orig[j][c];
+                    z[c] = m0 + m1;
+                }
+                if (a.pbias && in_cols) {
+                    const float4 bb = *reinterpret_cast<const float4 *>(a.pbias + col);
+                    z[0] = z[0] + bb.x; z[1] = z[1] + bb.y; z[2] = z[2] + bb.z; z[3] = z[3] + bb.w;
+                }
+            }
+            if (a.out && live && in_cols)
+                *reinterpret_cast<float4 *>(a.out + row * a.out_stride + col) =
+                    make_float4(z[0], z[1], z[2], z[3]);
+
+            if constexpr (HASH) {
+                // An 8-value group is split over a lane pair: the even lane has
+                // d = 0..3 (the high nibble), the odd lane d = 4..7.  The odd lane
+                // continues the even lane's running sum and product so that the
+                // order of operations is d = 0..7, as in
+                // compute_code_score/torch_extension.cc:31-37.
+                const int nib = (z[0] > 0.f ? 8 : 0) | (z[1] > 0.f ? 4 : 0) |
+                                (z[2] > 0.f ? 2 : 0) | (z[3] > 0.f ? 1 : 0);
+                float s_loc = 0.f, p_loc = 1.f;
+                score_chain(z, s_loc, p_loc);
+                float s_run = lane_xor<1>(s_loc);
+                float p_run = lane_xor<1>(p_loc);
+                const int nib_hi = __float_as_int(lane_xor<1>(__int_as_float(nib)));
+                score_chain(z, s_run, p_run);
+                const int t = col >> 3;
+                if (live && (lr & 1) && t < a.T) {
+                    a.codes[row * a.T + t] = (nib_hi << 4) | nib;
+                    a.scores[row * a.T + t] = s_run / p_run;
+                }
+            }
+        }
+    }
+}
+
+template <bool HASH>
+int launch_project(const ProjectArgs &a, int logd, hipStream_t stream) {
+    if (a.B == 0) return LFFN_OK;
+    auto go = [&](auto tag) {
+        constexpr int L = decltype(tag)::value;
+        const int64_t rows_per_block = 4 * FhtCfg<L>::RPW;
+        const int64_t blocks = (a.B + rows_per_block - 1) / rows_per_block;
+        hipLaunchKernelGGL((project_kernel<L, HASH>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+    };
+    switch (logd) {
+        case 2: if constexpr (!HASH) { go(std::integral_constant<int, 2>{}); break; } else return LFFN_ERR_UNSUPPORTED;
+        case 3: go(std::integral_constant<int, 3>{}); break;
+        case 4: go(std::integral_constant<int, 4>{}); break;
+        case 5: go(std::integral_constant<int, 5>{}); break;
+        case 6: go(std::integral_constant<int, 6>{}); break;
+        case 7: go(std::integral_constant<int, 7>{}); break;
+        case 8: go(std::integral_constant<int, 8>{}); break;
+        case 9: go(std::integral_constant<int, 9>{}); break;
+        case 10: go(std::integral_constant<int, 10>{}); break;
+        default: return LFFN_ERR_UNSUPPORTED;
+    }
+    return lffn_launch_status();
+}
+
+int check_dims(int64_t B, int64_t H, int64_t D, int64_t R, int64_t J) {
+    LFFN_REQUIRE(B >= 0 && H >= 1 && R >= 1 && J >= 0, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_is_pow2(D) && D >= 4 && D <= 1024, LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(H <= D, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(B * 1 <= (int64_t(1) << 31) - 1, LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(R * D <= (int64_t(1) << 24) && J <= 64, LFFN_ERR_UNSUPPORTED);
+    return LFFN_OK;
+}
+
+}  // namespace
+
+extern "C" int lffn_fht_f32(const float *in, float *out, int64_t B, int64_t D, void *stream) {
+    LFFN_REQUIRE(in && out, LFFN_ERR_BAD_ARG);
+    int rc = check_dims(B, D, D, 1, 1);
+    if (rc != LFFN_OK) return rc;
+    LFFN_REQUIRE(lffn_aligned16(out), LFFN_ERR_BAD_ARG);
+    ProjectArgs a{};
+    a.x = in; a.diag = nullptr; a.pbias = nullptr; a.out = out; a.codes = nullptr; a.scores = nullptr;
+    a.B = B; a.H = (int)D; a.R = 1; a.J = 1; a.out_stride = (int)D; a.out_cols = (int)D; a.T = 0;
+    a.decay = 1.f; a.residual = 0.f; a.mix = 0; a.vec_in = lffn_aligned16(in) ? 1 : 0;
+    return launch_project<false>(a, lffn_log2(D), static_cast<hipStream_t>(stream));
+}
+
+extern "C" int lffn_bh4_diag_f32(const float *x, const float *diag, float *out,
+                                 int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, void *stream) {
+    LFFN_REQUIRE(x && diag && out, LFFN_ERR_BAD_ARG);
+    int rc = check_dims(B, H, D, R, J);
+    if (rc != LFFN_OK) return rc;
+    LFFN_REQUIRE(lffn_aligned16(out) && lffn_aligned16(diag), LFFN_ERR_BAD_ARG);
+    ProjectArgs a{};
+    a.x = x; a.diag = diag; a.pbias = nullptr; a.out = out; a.codes = nullptr; a.scores = nullptr;
+    a.B = B; a.H = (int)H; a.R = (int)R; a.J = (int)J;
+    a.out_stride = (int)(R * D); a.out_cols = (int)(R * D); a.T = 0;
+    a.decay = 1.f; a.residual = 0.f; a.mix = 0;
+    a.vec_in = (lffn_aligned16(x) && H % 4 == 0) ? 1 : 0;
+    return launch_project<false>(a, lffn_log2(D), static_cast<hipStream_t>(stream));
+}
+
+extern "C" int lffn_project_hash_f32(const float *x, const float *diag, const float *proj_bias,
+                                     float *z_out, int32_t *codes, float *scores,
+                                     int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
+                                     float decay, float residual, void *stream) {
+    LFFN_REQUIRE(x && diag && codes && scores, LFFN_ERR_BAD_ARG);
+    int rc = check_dims(B, H, D, R, J);
+    if (rc != LFFN_OK) return rc;
+    LFFN_REQUIRE(D >= 8, LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(T >= 1 && T * 8 <= R * D, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_aligned16(diag) && (!proj_bias || lffn_aligned16(proj_bias)) &&
+                     (!z_out || lffn_aligned16(z_out)),
+                 LFFN_ERR_BAD_ARG);
+    ProjectArgs a{};
+    a.x = x; a.diag = diag; a.pbias = proj_bias; a.out = z_out; a.codes = codes; a.scores = scores;
+    a.B = B; a.H = (int)H; a.R = (int)R; a.J = (int)J;
+    a.out_stride = (int)(T * 8); a.out_cols = (int)(T * 8); a.T = (int)T;
+    a.decay = decay; a.residual = residual; a.mix = 1;
+    a.vec_in = (lffn_aligned16(x) && H % 4 == 0) ? 1 : 0;
+    return launch_project<true>(a, lffn_log2(D), static_cast<hipStream_t>(stream));
+}

@@ -1,0 +1,433 @@
+// Weighted gather-add and its backward for gfx950, token-major form.
+//
+//   gather_add              out[b,:]  = sum_i w[b,i] * src[idx[b,i],:]
+//   indexed_inner_product   out[b,i]  = <g[b,:], src[idx[b,i],:]>
+//   scatter_add             out[idx[b,i],:] += w[b,i] * g[b,:]
+//
+// A token is owned by a group of LPT lanes (64, 32, 16 or 8, the largest that
+// divides the row's 16-byte vectors); lane l of the group owns vectors
+// l, l+LPT, ... of a column chunk of LPT*NV vectors (blockIdx.y selects the
+// chunk).  Every row access is a 16-byte load per lane, LPT lanes side by side:
+// whole 128-byte lines.  The (index, weight) pairs of a block's tokens are staged
+// in LDS 64 at a time; the row loop is unrolled so that eight rows' loads are in
+// flight per lane before the first is consumed.  Accumulation is fp32, index
+// ascending: the order of the reference loop (gather_kernel_fp32.cu:41-43).
+//
+// All blocks walk the index dimension from 0 upwards at the same pace, so when
+// the indices are per-table (idx[b,t] in table t, as LookupFFN issues them) the
+// rows in use at any moment belong to a few tables and stay in the L2 of each XCD.
+#include "lffn_common.h"
+
+#include <hip/amd_detail/amd_hip_unsafe_atomics.h>
+
+namespace {
+
+constexpr int IC = 64;      // (index, weight) pairs staged per token per pass
+constexpr int UNROLL = 8;   // rows in flight per lane group
+
+template <bool BF16>
+struct Row {
+    static constexpr int EPV = BF16 ? 8 : 4;   // elements per 16-byte vector
+    static constexpr int ESZ = BF16 ? 2 : 4;
+};
+
+template <bool BF16>
+__device__ __forceinline__ void axpy_vec(float (&acc)[Row<BF16>::EPV], const uint4 &r, float w) {
+    if constexpr (BF16) {
+        acc[0] = fmaf(bf16_lo(r.x), w, acc[0]);
+        acc[1] = fmaf(bf16_hi(r.x), w, acc[1]);
+        acc[2] = fmaf(bf16_lo(r.y), w, acc[2]);
+        acc[3] = fmaf(bf16_hi(r.y), w, acc[3]);
+        acc[4] = fmaf(bf16_lo(r.z), w, acc[4]);
+        acc[5] = fmaf(bf16_hi(r.z), w, acc[5]);
+        acc[6] = fmaf(bf16_lo(r.w), w, acc[6]);
+        acc[7] = fmaf(bf16_hi(r.w), w, acc[7]);
+    } else {
+        acc[0] = fmaf(__uint_as_float(r.x), w, acc[0]);
+        acc[1] = fmaf(__uint_as_float(r.y), w, acc[1]);
+        acc[2] = fmaf(__uint_as_float(r.z), w, acc[2]);
+        acc[3] = fmaf(__uint_as_float(r.w), w, acc[3]);
+    }
+}
+
+struct GatherArgs {
+    const int32_t *idx;   // [B, I]  (codes when structured)
+    const void *src;      // [source_size, Dv]
+    const float *w;       // [B, I]
+    const float *g;       // [B, Dv]   (backward kernels)
+    const float *bias;    // [Dv] or null (structured forward)
+    float *out;
+    int64_t B;
+    int I;
+    int64_t source_size;  // rows of src / out
+    int Dv;
+    int S;                // structured: table size (power of two); 0 = flat indices
+};
+
+// Stage the block's (index, weight) pairs [i0, i0+IC) in LDS, resolving the row
+// number: flat indices are clamped into [0, source_size); codes are masked into
+// their table and offset by i*S (PL/lookup.py:126).
+template <int TPB, bool WITH_W>
+__device__ __forceinline__ void stage_pairs(const GatherArgs &a, int64_t tok0, int i0,
+                                            int (*s_row)[IC], float (*s_w)[IC]) {
+    for (int e = threadIdx.x; e < TPB * IC; e += 256) {
+        const int tl = e / IC, ii = e % IC;
+        const int64_t tok = tok0 + tl;
+        const int i = i0 + ii;
+        int row = 0;
+        float wt = 0.f;
+        if (tok < a.B && i < a.I) {
+            const int raw = a.idx[tok * a.I + i];
+            if (a.S > 0) {
+                row = (raw & (a.S - 1)) + i * a.S;
+            } else {
+                const int64_t hi = a.source_size - 1;
+                row = (int)(raw < 0 ? 0 : (raw > hi ? hi : raw));
+            }
+            if constexpr (WITH_W) wt = a.w[tok * a.I + i];
+        }
+        s_row[tl][ii] = row;
+        if constexpr (WITH_W) s_w[tl][ii] = wt;
+    }
+}
+
+template <bool BF16, int LPT, int NV>
+__global__ __launch_bounds__(256) void gather_add_kernel(GatherArgs a) {
+    constexpr int TPB = 256 / LPT;
+    constexpr int EPV = Row<BF16>::EPV;
+    __shared__ int s_row[TPB][IC];
+    __shared__ float s_w[TPB][IC];
+
+    const int tl = threadIdx.x / LPT;
+    const int ll = threadIdx.x % LPT;
+    const int64_t tok0 = int64_t(blockIdx.x) * TPB;
+    const int64_t tok = tok0 + tl;
+    const int vec0 = blockIdx.y * (LPT * NV) + ll;            // first 16-byte vector of this lane
+    const size_t row_bytes = size_t(a.Dv) * Row<BF16>::ESZ;
+    const char *base = static_cast<const char *>(a.src) + size_t(vec0) * 16;
+
+    float acc[NV][EPV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        if (a.bias) {
+#pragma unroll
+            for (int q = 0; q < EPV / 4; ++q) {
+                const float4 bb = *reinterpret_cast<const float4 *>(a.bias + (size_t)(vec0 + v * LPT) * EPV + 4 * q);
+                acc[v][4 * q + 0] = bb.x; acc[v][4 * q + 1] = bb.y;
+                acc[v][4 * q + 2] = bb.z; acc[v][4 * q + 3] = bb.w;
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) acc[v][e] = 0.f;
+        }
+    }
+
+    for (int i0 = 0; i0 < a.I; i0 += IC) {
+        __syncthreads();
+        stage_pairs<TPB, true>(a, tok0, i0, s_row, s_w);
+        __syncthreads();
+        const int n = min(IC, a.I - i0);
+        int ii = 0;
+        for (; ii + UNROLL <= n; ii += UNROLL) {
+            uint4 r[UNROLL][NV];
+            float wt[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                int row = s_row[tl][ii + u];
+                wt[u] = s_w[tl][ii + u];
+                if constexpr (LPT == 64) {   // one token per wavefront: the row address is uniform
+                    row = __builtin_amdgcn_readfirstlane(row);
+                    wt[u] = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(wt[u])));
+                }
+                const uint4 *p = reinterpret_cast<const uint4 *>(base + size_t(row) * row_bytes);
+#pragma unroll
+                for (int v = 0; v < NV; ++v) r[u][v] = p[v * LPT];
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+                for (int v = 0; v < NV; ++v) axpy_vec<BF16>(acc[v], r[u][v], wt[u]);
+        }
+        for (; ii < n; ++ii) {
+            const int row = s_row[tl][ii];
+            const float wt = s_w[tl][ii];
+            const uint4 *p = reinterpret_cast<const uint4 *>(base + size_t(row) * row_bytes);
+#pragma unroll
+            for (int v = 0; v < NV; ++v) axpy_vec<BF16>(acc[v], p[v * LPT], wt);
+        }
+    }
+
+    if (tok < a.B) {
+        float *o = a.out + tok * a.Dv;
+#pragma unroll
+        for (int v = 0; v < NV; ++v)
+#pragma unroll
+            for (int q = 0; q < EPV / 4; ++q)
+                *reinterpret_cast<float4 *>(o + (size_t)(vec0 + v * LPT) * EPV + 4 * q) =
+                    make_float4(acc[v][4 * q + 0], acc[v][4 * q + 1], acc[v][4 * q + 2], acc[v][4 * q + 3]);
+    }
+}
+
+// Sum over the LPT lanes of a token group (LPT a power of two, groups aligned).
+template <int LPT>
+__device__ __forceinline__ float group_sum(float v) {
+    if constexpr (LPT > 1) v += lane_xor<1>(v);
+    if constexpr (LPT > 2) v += lane_xor<2>(v);
+    if constexpr (LPT > 4) v += lane_xor<4>(v);
+    if constexpr (LPT > 8) v += lane_xor<8>(v);
+    if constexpr (LPT > 16) v += lane_xor<16>(v);
+    if constexpr (LPT > 32) v += lane_xor<32>(v);
+    return v;
+}
+
+// out[b,i] = <g[b,:], src[idx[b,i],:]>.  Column chunks are walked inside the
+// block; the per-chunk partial dot products are summed in LDS in chunk order.
+template <int LPT, int NV>
+__global__ __launch_bounds__(256) void inner_product_kernel(GatherArgs a, int chunks) {
+    constexpr int TPB = 256 / LPT;
+    __shared__ int s_row[TPB][IC];
+    __shared__ float s_dot[TPB][IC];
+
+    const int tl = threadIdx.x / LPT;
+    const int ll = threadIdx.x % LPT;
+    const int64_t tok0 = int64_t(blockIdx.x) * TPB;
+    const int64_t tok = tok0 + tl;
+    const size_t row_bytes = size_t(a.Dv) * 4;
+
+    for (int i0 = 0; i0 < a.I; i0 += IC) {
+        __syncthreads();
+        stage_pairs<TPB, false>(a, tok0, i0, s_row, s_dot);
+        for (int e = threadIdx.x; e < TPB * IC; e += 256) s_dot[e / IC][e % IC] = 0.f;
+        __syncthreads();
+        const int n = min(IC, a.I - i0);
+        for (int ch = 0; ch < chunks; ++ch) {
+            const int vec0 = ch * (LPT * NV) + ll;
+            float4 gv[NV];
+#pragma unroll
+            for (int v = 0; v < NV; ++v)
+                gv[v] = tok < a.B ? *reinterpret_cast<const float4 *>(a.g + tok * a.Dv + (size_t)(vec0 + v * LPT) * 4)
+                                  : make_float4(0.f, 0.f, 0.f, 0.f);
+            const char *base = static_cast<const char *>(a.src) + size_t(vec0) * 16;
+            int ii = 0;
+            for (; ii + 4 <= n; ii += 4) {
+                float4 r[4][NV];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const float4 *p = reinterpret_cast<const float4 *>(base + size_t(s_row[tl][ii + u]) * row_bytes);
+#pragma unroll
+                    for (int v = 0; v < NV; ++v) r[u][v] = p[v * LPT];
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    float d = 0.f;
+#pragma unroll
+                    for (int v = 0; v < NV; ++v) {
+                        d = fmaf(gv[v].x, r[u][v].x, d);
+                        d = fmaf(gv[v].y, r[u][v].y, d);
+                        d = fmaf(gv[v].z, r[u][v].z, d);
+                        d = fmaf(gv[v].w, r[u][v].w, d);
+                    }
+                    d = group_sum<LPT>(d);
+                    if (ll == 0) s_dot[tl][ii + u] += d;
+                }
+            }
+            for (; ii < n; ++ii) {
+                const float4 *p = reinterpret_cast<const float4 *>(base + size_t(s_row[tl][ii]) * row_bytes);
+                float d = 0.f;
+#pragma unroll
+                for (int v = 0; v < NV; ++v) {
+                    const float4 r = p[v * LPT];
+                    d = fmaf(gv[v].x, r.x, d);
+                    d = fmaf(gv[v].y, r.y, d);
+                    d = fmaf(gv[v].z, r.z, d);
+                    d = fmaf(gv[v].w, r.w, d);
+                }
+                d = group_sum<LPT>(d);
+                if (ll == 0) s_dot[tl][ii] += d;
+            }
+        }
+        __syncthreads();
+        for (int e = threadIdx.x; e < TPB * IC; e += 256) {
+            const int t2 = e / IC, ii2 = e % IC;
+            if (tok0 + t2 < a.B && i0 + ii2 < a.I) a.out[(tok0 + t2) * a.I + i0 + ii2] = s_dot[t2][ii2];
+        }
+    }
+}
+
+// out[idx[b,i],:] += w[b,i] * g[b,:] with hardware fp32 atomics.
+template <int LPT, int NV>
+__global__ __launch_bounds__(256) void scatter_add_kernel(GatherArgs a) {
+    constexpr int TPB = 256 / LPT;
+    __shared__ int s_row[TPB][IC];
+    __shared__ float s_w[TPB][IC];
+
+    const int tl = threadIdx.x / LPT;
+    const int ll = threadIdx.x % LPT;
+    const int64_t tok0 = int64_t(blockIdx.x) * TPB;
+    const int64_t tok = tok0 + tl;
+    const int vec0 = blockIdx.y * (LPT * NV) + ll;
+
+    float4 gv[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v)
+        gv[v] = tok < a.B ? *reinterpret_cast<const float4 *>(a.g + tok * a.Dv + (size_t)(vec0 + v * LPT) * 4)
+                          : make_float4(0.f, 0.f, 0.f, 0.f);
+
+    for (int i0 = 0; i0 < a.I; i0 += IC) {
+        __syncthreads();
+        stage_pairs<TPB, true>(a, tok0, i0, s_row, s_w);
+        __syncthreads();
+        if (tok >= a.B) continue;
+        const int n = min(IC, a.I - i0);
+        for (int ii = 0; ii < n; ++ii) {
+            const float wt = s_w[tl][ii];
+            float *o = a.out + size_t(s_row[tl][ii]) * a.Dv + size_t(vec0) * 4;
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                unsafeAtomicAdd(o + v * LPT * 4 + 0, wt * gv[v].x);
+                unsafeAtomicAdd(o + v * LPT * 4 + 1, wt * gv[v].y);
+                unsafeAtomicAdd(o + v * LPT * 4 + 2, wt * gv[v].z);
+                unsafeAtomicAdd(o + v * LPT * 4 + 3, wt * gv[v].w);
+            }
+        }
+    }
+}
+
+// Split a row of `nvec` 16-byte vectors into lanes-per-token, vectors per lane and
+// column chunks.  nvec is a multiple of 8 (bf16) or 16 (f32) by the Dv % 64 rule.
+struct Tiling {
+    int lpt, nv, chunks;
+};
+
+Tiling pick_tiling(int nvec) {
+    Tiling t{};
+    t.lpt = (nvec % 64 == 0) ? 64 : (nvec % 32 == 0) ? 32 : (nvec % 16 == 0) ? 16 : 8;
+    const int m = nvec / t.lpt;
+    t.nv = (m % 4 == 0) ? 4 : (m % 3 == 0) ? 3 : (m % 2 == 0) ? 2 : 1;
+    t.chunks = m / t.nv;
+    return t;
+}
+
+enum class Op { Gather, Inner, Scatter };
+
+template <bool BF16, Op OP, int LPT, int NV>
+void launch_one(const GatherArgs &a, const Tiling &t, hipStream_t s) {
+    constexpr int TPB = 256 / LPT;
+    const unsigned gx = (unsigned)((a.B + TPB - 1) / TPB);
+    if constexpr (OP == Op::Gather)
+        hipLaunchKernelGGL((gather_add_kernel<BF16, LPT, NV>), dim3(gx, t.chunks), dim3(256), 0, s, a);
+    else if constexpr (OP == Op::Inner)
+        hipLaunchKernelGGL((inner_product_kernel<LPT, NV>), dim3(gx), dim3(256), 0, s, a, t.chunks);
+    else
+        hipLaunchKernelGGL((scatter_add_kernel<LPT, NV>), dim3(gx, t.chunks), dim3(256), 0, s, a);
+}
+
+template <bool BF16, Op OP, int LPT>
+void launch_nv(const GatherArgs &a, const Tiling &t, hipStream_t s) {
+    switch (t.nv) {
+        case 1: launch_one<BF16, OP, LPT, 1>(a, t, s); break;
+        case 2: launch_one<BF16, OP, LPT, 2>(a, t, s); break;
+        case 3: launch_one<BF16, OP, LPT, 3>(a, t, s); break;
+        default: launch_one<BF16, OP, LPT, 4>(a, t, s); break;
+    }
+}
+
+template <bool BF16, Op OP>
+int launch(const GatherArgs &a, hipStream_t s) {
+    if (a.B == 0 || (a.I == 0 && OP != Op::Gather)) return LFFN_OK;
+    const Tiling t = pick_tiling(a.Dv / Row<BF16>::EPV);
+    switch (t.lpt) {
+        case 64: launch_nv<BF16, OP, 64>(a, t, s); break;
+        case 32: launch_nv<BF16, OP, 32>(a, t, s); break;
+        case 16: launch_nv<BF16, OP, 16>(a, t, s); break;
+        default:
+            if constexpr (BF16) { launch_nv<BF16, OP, 8>(a, t, s); break; }
+            else return LFFN_ERR_UNSUPPORTED;
+    }
+    return lffn_launch_status();
+}
+
+int check_common(const void *idx, int64_t B, int64_t I, int64_t rows, int64_t Dv) {
+    LFFN_REQUIRE(B >= 0 && I >= 0 && rows >= 1 && Dv >= 1, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(idx || B * I == 0, LFFN_ERR_BAD_ARG);   // an empty index array may be null
+    LFFN_REQUIRE(Dv % 64 == 0, LFFN_ERR_UNSUPPORTED);            // PL/gather/cuda/kernel.py:43
+    LFFN_REQUIRE(Dv <= (1 << 20) && I <= (1 << 24), LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(rows <= 0x7fffffff, LFFN_ERR_UNSUPPORTED);      // int32 indices
+    LFFN_REQUIRE(B <= (int64_t(1) << 31) - 1, LFFN_ERR_UNSUPPORTED);
+    return LFFN_OK;
+}
+
+template <bool BF16>
+int gather_entry(const int32_t *idx, const void *src, const float *w, const float *bias, float *out,
+                 int64_t B, int64_t I, int64_t rows, int64_t Dv, int64_t S, void *stream) {
+    int rc = check_common(idx, B, I, rows, Dv);
+    if (rc != LFFN_OK) return rc;
+    LFFN_REQUIRE(src && out && (w || B * I == 0), LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_aligned16(src) && lffn_aligned16(out) && (!bias || lffn_aligned16(bias)), LFFN_ERR_BAD_ARG);
+    GatherArgs a{};
+    a.idx = idx; a.src = src; a.w = w; a.g = nullptr; a.bias = bias; a.out = out;
+    a.B = B; a.I = (int)I; a.source_size = rows; a.Dv = (int)Dv; a.S = (int)S;
+    return launch<BF16, Op::Gather>(a, static_cast<hipStream_t>(stream));
+}
+
+}  // namespace
+
+extern "C" int lffn_gather_add_f32(const int32_t *idx, const float *src, const float *w, float *out,
+                                   int64_t B, int64_t I, int64_t source_size, int64_t Dv, void *stream) {
+    return gather_entry<false>(idx, src, w, nullptr, out, B, I, source_size, Dv, 0, stream);
+}
+
+extern "C" int lffn_gather_add_bf16(const int32_t *idx, const uint16_t *src, const float *w, float *out,
+                                    int64_t B, int64_t I, int64_t source_size, int64_t Dv, void *stream) {
+    return gather_entry<true>(idx, src, w, nullptr, out, B, I, source_size, Dv, 0, stream);
+}
+
+extern "C" int lffn_lookup_gather_f32(const int32_t *code, const float *score, const float *tables,
+                                      const float *bias, float *out,
+                                      int64_t B, int64_t T, int64_t S, int64_t Do, void *stream) {
+    LFFN_REQUIRE(lffn_is_pow2(S) && S <= (1 << 24) && T >= 0 && T * S <= 0x7fffffff, LFFN_ERR_UNSUPPORTED);
+    return gather_entry<false>(code, tables, score, bias, out, B, T, T * S > 0 ? T * S : 1, Do, S, stream);
+}
+
+extern "C" int lffn_lookup_gather_bf16(const int32_t *code, const float *score, const uint16_t *tables,
+                                       const float *bias, float *out,
+                                       int64_t B, int64_t T, int64_t S, int64_t Do, void *stream) {
+    LFFN_REQUIRE(lffn_is_pow2(S) && S <= (1 << 24) && T >= 0 && T * S <= 0x7fffffff, LFFN_ERR_UNSUPPORTED);
+    return gather_entry<true>(code, tables, score, bias, out, B, T, T * S > 0 ? T * S : 1, Do, S, stream);
+}
+
+extern "C" int lffn_indexed_inner_product_f32(const int32_t *idx, const float *g, const float *src, float *out,
+                                              int64_t B, int64_t I, int64_t source_size, int64_t Dv, void *stream) {
+    int rc = check_common(idx, B, I, source_size, Dv);
+    if (rc != LFFN_OK) return rc;
+    LFFN_REQUIRE(g && src && (out || B * I == 0), LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_aligned16(src) && lffn_aligned16(g), LFFN_ERR_BAD_ARG);
+    GatherArgs a{};
+    a.idx = idx; a.src = src; a.w = nullptr; a.g = g; a.bias = nullptr; a.out = out;
+    a.B = B; a.I = (int)I; a.source_size = source_size; a.Dv = (int)Dv; a.S = 0;
+    return launch<false, Op::Inner>(a, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int lffn_scatter_add_f32(const int32_t *idx, const float *g, const float *w, float *out,
+                                    int64_t B, int64_t I, int64_t out_size, int64_t Dv, void *stream) {
+    int rc = check_common(idx, B, I, out_size, Dv);
+    if (rc != LFFN_OK) return rc;
+    LFFN_REQUIRE(g && out && (w || B * I == 0), LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_aligned16(g) && lffn_aligned16(out), LFFN_ERR_BAD_ARG);
+    GatherArgs a{};
+    a.idx = idx; a.src = nullptr; a.w = w; a.g = g; a.bias = nullptr; a.out = out;
+    a.B = B; a.I = (int)I; a.source_size = out_size; a.Dv = (int)Dv; a.S = 0;
+    return launch<false, Op::Scatter>(a, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int lffn_version(void) { return LFFN_ABI_VERSION; }
+
+extern "C" const char *lffn_error_string(int code) {
+    switch (code) {
+        case LFFN_OK: return "ok";
+        case LFFN_ERR_BAD_ARG: return "bad argument (null or misaligned pointer, negative or inconsistent size)";
+        case LFFN_ERR_UNSUPPORTED: return "shape not supported by the gfx950 kernels";
+        case LFFN_ERR_LAUNCH: return "kernel launch failed";
+        default: return "unknown error code";
+    }
+}

@@ -1,0 +1,84 @@
+// Shared device helpers and host-side argument checks for the gfx950 LookupFFN kernels.
+// wave64 is assumed everywhere: this code is built for gfx950 only.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/lookupffn_hip.h"
+
+#define LFFN_WAVE 64
+
+#define LFFN_REQUIRE(cond, code) \
+    do {                         \
+        if (!(cond)) return (code); \
+    } while (0)
+
+static inline bool lffn_aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+static inline bool lffn_is_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
+static inline int lffn_log2(int64_t v) {
+    int l = 0;
+    while ((int64_t(1) << l) < v) ++l;
+    return l;
+}
+
+static inline int lffn_launch_status() {
+    return hipGetLastError() == hipSuccess ? LFFN_OK : LFFN_ERR_LAUNCH;
+}
+
+// ---------------------------------------------------------------------------
+// Cross-lane moves.  dpp_mov<CTRL>: lanes whose source is outside the row, or
+// that the bank mask switches off, keep `old`.
+// ---------------------------------------------------------------------------
+template <int CTRL, int ROW_MASK = 0xF, int BANK_MASK = 0xF>
+__device__ __forceinline__ float dpp_mov(float old, float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(old), __float_as_int(v), CTRL,
+                                                      ROW_MASK, BANK_MASK, false));
+}
+
+constexpr int DPP_QUAD_XOR1 = 0xB1;   // quad_perm [1,0,3,2]
+constexpr int DPP_QUAD_XOR2 = 0x4E;   // quad_perm [2,3,0,1]
+constexpr int DPP_ROW_SHL4 = 0x104;   // lane i <- lane i+4
+constexpr int DPP_ROW_SHR4 = 0x114;   // lane i <- lane i-4
+constexpr int DPP_ROW_ROR8 = 0x128;   // lane i <- lane (i-8) mod 16 == i xor 8
+
+// Value held by lane (lane ^ M), for M a power of two below 64.
+template <int M>
+__device__ __forceinline__ float lane_xor(float v) {
+    if constexpr (M == 1) {
+        return dpp_mov<DPP_QUAD_XOR1>(v, v);
+    } else if constexpr (M == 2) {
+        return dpp_mov<DPP_QUAD_XOR2>(v, v);
+    } else if constexpr (M == 4) {
+        float r = dpp_mov<DPP_ROW_SHL4, 0xF, 0x5>(v, v);   // banks 0,2 take lane+4
+        return dpp_mov<DPP_ROW_SHR4, 0xF, 0xA>(r, v);      // banks 1,3 take lane-4
+    } else if constexpr (M == 8) {
+        return dpp_mov<DPP_ROW_ROR8>(v, v);
+    } else if constexpr (M == 16) {
+        // ds_swizzle, bit-mask mode inside 32 lanes: and 0x1F, or 0, xor 0x10
+        return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401F));
+    } else {
+        static_assert(M == 32, "lane_xor: M must be a power of two below 64");
+        return __shfl_xor(v, 32, 64);
+    }
+}
+
+// One butterfly across lanes: the lane whose M bit is clear gets own + partner,
+// the other gets partner - own.  `sgn` is +1 / -1 for the two cases.
+template <int M>
+__device__ __forceinline__ float butterfly_xor(float v, float sgn) {
+    return fmaf(v, sgn, lane_xor<M>(v));   // (+-1)*v is exact: one rounding, like a plain add
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+    v += lane_xor<1>(v);
+    v += lane_xor<2>(v);
+    v += lane_xor<4>(v);
+    v += lane_xor<8>(v);
+    v += lane_xor<16>(v);
+    v += lane_xor<32>(v);
+    return v;
+}
+
+__device__ __forceinline__ float bf16_lo(uint32_t packed) { return __uint_as_float(packed << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t packed) { return __uint_as_float(packed & 0xFFFF0000u); }

@@ -1,0 +1,155 @@
+"""``BH4``, ``Hashing`` and ``LookupFFN``: the module surface of the reference's
+PL/lookup.py (PL/ = src/roberta/models/prenorm_lookup/), with the same
+constructor arguments, ``config`` attribute names, parameter names and shapes
+(so a reference state_dict loads unchanged), on the gfx950 kernels.
+
+Inference (no gradient needed) with ``block_size == 1`` and 8-bit codes runs as
+LayerNorm -> one fused projection+hash kernel -> one gather kernel.  Every other
+case runs the same operator sequence as the reference, each operator on its
+kernel and differentiable.
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import torch
+import torch.nn as nn
+
+from . import ops
+from .bh4 import bh4
+from .compute_code_score import compute_code_score
+from .gather import gather, lookup_gather
+
+
+class BH4(nn.Module):
+    """PL/lookup.py:10-47."""
+
+    def __init__(self, in_dim, out_dim, block_size, decay_coeff=0.7):
+        super().__init__()
+        self.in_dim = in_dim
+        self.out_dim = out_dim
+        self.block_size = block_size
+        self.decay_coeff = decay_coeff
+
+        self.padded_in_dim = int(2 ** math.ceil(math.log2(in_dim)))
+        self.num_repeat = max(1, int(math.ceil(self.out_dim / self.padded_in_dim)))
+        self.num_block = self.padded_in_dim // self.block_size
+
+        coeff = math.sqrt(self.block_size * self.padded_in_dim)
+        self.weight = nn.Parameter(
+            torch.randn(self.num_repeat, 4, self.num_block, self.block_size, self.block_size) / coeff)
+        self.bias = nn.Parameter(torch.zeros(self.out_dim))
+
+    def extra_repr(self):
+        return (f"in_dim={self.in_dim}, out_dim={self.out_dim}, block_size={self.block_size}, "
+                f"decay_coeff={self.decay_coeff}")
+
+    def _forward(self, x):
+        batch_size, dim = x.shape
+        if dim < self.padded_in_dim:
+            padding_dim = self.padded_in_dim - dim
+            x = torch.cat([x, torch.zeros(batch_size, padding_dim, dtype=x.dtype, device=x.device)],
+                          dim=-1).contiguous()
+        x = (self.decay_coeff * bh4(x, self.weight, training=self.training)
+             + (1 - self.decay_coeff) * x.repeat(1, self.num_repeat))
+        x = x[:, :self.out_dim].contiguous() + self.bias
+        return x
+
+    def forward(self, xs):
+        shape = xs.shape[:-1]
+        dim = xs.shape[-1]
+        xs = xs.reshape(int(np.prod(shape)), dim)
+        outputs = self._forward(xs)
+        return outputs.reshape(*shape, self.out_dim)
+
+
+class Hashing(nn.Module):
+    """PL/lookup.py:49-77."""
+
+    def __init__(self, config):
+        super().__init__()
+        self.hidden_size = config.hidden_size
+        self.num_table = config.ffn_num_table
+        self.table_size = config.ffn_table_size
+        self.code_length = int(math.log2(self.table_size))
+        self.total_dim = self.num_table * self.code_length
+        if config.projection_type == "bh4":
+            self.projection = BH4(self.hidden_size, self.total_dim, block_size=config.block_size)
+        elif config.projection_type == "dense":
+            self.projection = nn.Linear(self.hidden_size, self.total_dim)
+        else:
+            raise NotImplementedError
+
+    def can_fuse(self, x):
+        """One-kernel projection+hash: diagonal BH4, 8-bit codes, fp32, no gradient."""
+        p = self.projection
+        needs_grad = torch.is_grad_enabled() and (
+            x.requires_grad or any(q.requires_grad for q in self.parameters()))
+        return (isinstance(p, BH4) and p.block_size == 1 and self.code_length == 8
+                and p.padded_in_dim <= 1024 and p.padded_in_dim >= 8
+                and x.dtype == torch.float32 and x.is_cuda and not needs_grad)
+
+    def forward_fused(self, x):
+        p = self.projection
+        diag = p.weight.reshape(p.num_repeat, p.weight.shape[1], p.padded_in_dim)
+        code, score, _ = ops.project_hash(
+            x.contiguous(), diag.contiguous(), p.bias, self.num_table,
+            float(p.decay_coeff), float(1 - p.decay_coeff), False)
+        return code, score
+
+    def forward(self, x):
+        B, D = x.shape
+        if self.can_fuse(x):
+            return self.forward_fused(x)
+        z = self.projection(x)
+        z = z.reshape(B, self.num_table, self.code_length)
+        code, score = compute_code_score(z, training=self.training)
+        return code, score
+
+
+class LookupFFN(nn.Module):
+    """PL/lookup.py:79-130."""
+
+    def __init__(self, config, output_size):
+        super().__init__()
+        self.hidden_size = config.hidden_size
+        self.output_size = output_size
+        self.LayerNorm = nn.LayerNorm(self.hidden_size, eps=config.layer_norm_eps)
+
+        self.num_table = config.ffn_num_table
+        self.table_size = config.ffn_table_size
+        assert (2 ** int(math.log2(self.table_size))) == self.table_size
+        self.hash = Hashing(config)
+        self.tables = nn.Parameter(0.02 * torch.randn(self.num_table, self.table_size, self.output_size))
+        self.bias = nn.Parameter(0.001 * torch.randn(self.output_size))
+
+    def extra_repr(self):
+        return (f"hidden_size={self.hidden_size}, num_table={self.num_table}, "
+                f"table_size={self.table_size}, output_size={self.output_size}")
+
+    def _forward(self, hidden_states):
+        hidden_states = self.LayerNorm(hidden_states)
+        code, score = self.hash(hidden_states)
+        if self.output_size % 64 == 0 and self.tables.dtype in (torch.float32, torch.bfloat16):
+            # table-local codes, offset and bias folded into the gather kernel
+            return lookup_gather(code, score.float(), self.tables, self.bias.float())
+        outputs = self.gather(code, score, self.tables)
+        return outputs + self.bias
+
+    def forward(self, hidden_states):
+        shape = hidden_states.shape[:-1]
+        dim = hidden_states.shape[-1]
+        hidden_states = hidden_states.reshape(int(np.prod(shape)), dim)
+        outputs = self._forward(hidden_states)
+        return outputs.reshape(*shape, self.output_size)
+
+    def gather(self, indexes, weights, tables):
+        """PL/lookup.py:120-130: flat row numbers, then the general gather."""
+        B, N = indexes.shape
+        num_table, table_size, vector_dim = tables.shape
+        assert weights.shape[0] == B
+        assert weights.shape[1] == N
+        indexes = indexes + torch.arange(num_table, device=indexes.device, dtype=indexes.dtype)[None] * table_size
+        tables = tables.reshape(num_table * table_size, vector_dim)
+        return gather(indexes, weights, tables, training=self.training)

@@ -1,0 +1,316 @@
+"""torch custom ops (namespace ``lookupffn``) over the C ABI of liblookupffn_hip.so.
+
+Each op checks shapes and dtypes on the host, allocates its outputs with
+``torch.empty`` on the inputs' device, and launches on torch's current stream.
+Only a GPU ("CUDA" dispatch key, which is HIP on ROCm) implementation is
+registered: calling an op with CPU tensors fails in the dispatcher.  Fake
+(meta) implementations let the ops be traced.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+_L = torch.library.Library("lookupffn", "DEF")
+
+
+def _is_pow2(v: int) -> bool:
+    return v > 0 and (v & (v - 1)) == 0
+
+
+def _dev_guard(t: torch.Tensor):
+    return torch.cuda.device(t.device)
+
+
+# ----------------------------------------------------------------------------- fht
+
+_L.define("fht(Tensor x) -> Tensor")
+
+
+def _fht_impl(x: torch.Tensor) -> torch.Tensor:
+    _lib.require_gpu(x)
+    assert x.dim() == 2 and x.dtype == torch.float32 and x.is_contiguous()
+    B, D = x.shape
+    out = torch.empty_like(x)
+    with _dev_guard(x):
+        rc = _lib.load().lffn_fht_f32(_lib.ptr(x), _lib.ptr(out), B, D, _lib.stream_of(x))
+    _lib.check(rc, f"lffn_fht_f32(B={B}, D={D})")
+    return out
+
+
+_L.impl("fht", _fht_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::fht")
+def _(x):
+    return torch.empty_like(x)
+
+
+# ----------------------------------------------------------------------------- bh4_diag
+
+_L.define("bh4_diag(Tensor x, Tensor diag) -> Tensor")
+
+
+def _bh4_diag_impl(x: torch.Tensor, diag: torch.Tensor) -> torch.Tensor:
+    _lib.require_gpu(x, diag)
+    assert x.dim() == 2 and diag.dim() == 3
+    assert x.dtype == torch.float32 and diag.dtype == torch.float32
+    assert x.is_contiguous() and diag.is_contiguous()
+    B, H = x.shape
+    R, J, D = diag.shape
+    assert H <= D
+    out = torch.empty(B, R * D, dtype=torch.float32, device=x.device)
+    with _dev_guard(x):
+        rc = _lib.load().lffn_bh4_diag_f32(_lib.ptr(x), _lib.ptr(diag), _lib.ptr(out), B, H, D, R, J,
+                                           _lib.stream_of(x))
+    _lib.check(rc, f"lffn_bh4_diag_f32(B={B}, H={H}, D={D}, R={R}, J={J})")
+    return out
+
+
+_L.impl("bh4_diag", _bh4_diag_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::bh4_diag")
+def _(x, diag):
+    return x.new_empty(x.shape[0], diag.shape[0] * diag.shape[2])
+
+
+# ----------------------------------------------------------------------------- project_hash
+
+_L.define("project_hash(Tensor x, Tensor diag, Tensor? bias, int T, float decay, float residual, bool keep_z)"
+          " -> (Tensor, Tensor, Tensor)")
+
+
+def _project_hash_impl(x, diag, bias, T, decay, residual, keep_z):
+    _lib.require_gpu(x, diag, bias)
+    assert x.dim() == 2 and diag.dim() == 3
+    assert x.dtype == torch.float32 and diag.dtype == torch.float32
+    assert x.is_contiguous() and diag.is_contiguous()
+    B, H = x.shape
+    R, J, D = diag.shape
+    assert H <= D and T * 8 <= R * D
+    if bias is not None:
+        assert bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == T * 8
+    codes = torch.empty(B, T, dtype=torch.int32, device=x.device)
+    scores = torch.empty(B, T, dtype=torch.float32, device=x.device)
+    z = torch.empty((B, T * 8) if keep_z else (0,), dtype=torch.float32, device=x.device)
+    with _dev_guard(x):
+        rc = _lib.load().lffn_project_hash_f32(
+            _lib.ptr(x), _lib.ptr(diag), _lib.ptr(bias), _lib.ptr(z) if keep_z else None,
+            _lib.ptr(codes), _lib.ptr(scores), B, H, D, R, J, T, decay, residual, _lib.stream_of(x))
+    _lib.check(rc, f"lffn_project_hash_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T})")
+    return codes, scores, z
+
+
+_L.impl("project_hash", _project_hash_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::project_hash")
+def _(x, diag, bias, T, decay, residual, keep_z):
+    B = x.shape[0]
+    return (x.new_empty(B, T, dtype=torch.int32), x.new_empty(B, T),
+            x.new_empty((B, T * 8) if keep_z else (0,)))
+
+
+# ----------------------------------------------------------------------------- code_score
+
+_L.define("code_score(Tensor z) -> (Tensor, Tensor)")
+
+
+def _code_score_impl(z: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    _lib.require_gpu(z)
+    assert z.dim() >= 1 and z.dtype == torch.float32 and z.is_contiguous()
+    k = z.shape[-1]
+    N = z.numel() // max(k, 1)
+    codes = torch.empty(z.shape[:-1], dtype=torch.int32, device=z.device)
+    scores = torch.empty(z.shape[:-1], dtype=torch.float32, device=z.device)
+    with _dev_guard(z):
+        rc = _lib.load().lffn_code_score_f32(_lib.ptr(z), _lib.ptr(codes), _lib.ptr(scores), N, k,
+                                             _lib.stream_of(z))
+    _lib.check(rc, f"lffn_code_score_f32(N={N}, k={k})")
+    return codes, scores
+
+
+_L.impl("code_score", _code_score_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::code_score")
+def _(z):
+    return z.new_empty(z.shape[:-1], dtype=torch.int32), z.new_empty(z.shape[:-1])
+
+
+_L.define("code_score_bwd(Tensor z, Tensor g_score) -> Tensor")
+
+
+def _code_score_bwd_impl(z: torch.Tensor, g_score: torch.Tensor) -> torch.Tensor:
+    _lib.require_gpu(z, g_score)
+    assert z.dtype == torch.float32 and g_score.dtype == torch.float32
+    assert z.is_contiguous() and g_score.is_contiguous()
+    assert tuple(g_score.shape) == tuple(z.shape[:-1])
+    k = z.shape[-1]
+    N = z.numel() // max(k, 1)
+    g_z = torch.empty_like(z)
+    with _dev_guard(z):
+        rc = _lib.load().lffn_code_score_bwd_f32(_lib.ptr(z), _lib.ptr(g_score), _lib.ptr(g_z), N, k,
+                                                 _lib.stream_of(z))
+    _lib.check(rc, f"lffn_code_score_bwd_f32(N={N}, k={k})")
+    return g_z
+
+
+_L.impl("code_score_bwd", _code_score_bwd_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::code_score_bwd")
+def _(z, g_score):
+    return torch.empty_like(z)
+
+
+# ----------------------------------------------------------------------------- gather-add family
+
+def _check_gather_args(indexes, rows, vector_dim):
+    assert indexes.dim() == 2 and indexes.dtype == torch.int32 and indexes.is_contiguous()
+    assert vector_dim % 64 == 0, vector_dim
+    assert rows >= 1
+
+
+_L.define("gather_add(Tensor indexes, Tensor source, Tensor weights) -> Tensor")
+
+
+def _gather_add_impl(indexes, source, weights):
+    _lib.require_gpu(indexes, source, weights)
+    assert source.dim() == 2 and source.is_contiguous()
+    assert weights.dtype == torch.float32 and weights.is_contiguous()
+    assert tuple(weights.shape) == tuple(indexes.shape)
+    B, I = indexes.shape
+    S, Dv = source.shape
+    _check_gather_args(indexes, S, Dv)
+    out = torch.empty(B, Dv, dtype=torch.float32, device=source.device)
+    lib = _lib.load()
+    if source.dtype == torch.float32:
+        fn, name = lib.lffn_gather_add_f32, "lffn_gather_add_f32"
+    elif source.dtype == torch.bfloat16:
+        fn, name = lib.lffn_gather_add_bf16, "lffn_gather_add_bf16"
+    else:
+        raise NotImplementedError(f"gather_add: source dtype {source.dtype} (float32 and bfloat16 rows are built)")
+    with _dev_guard(source):
+        rc = fn(_lib.ptr(indexes), _lib.ptr(source), _lib.ptr(weights), _lib.ptr(out), B, I, S, Dv,
+                _lib.stream_of(source))
+    _lib.check(rc, f"{name}(B={B}, I={I}, S={S}, Dv={Dv})")
+    return out
+
+
+_L.impl("gather_add", _gather_add_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::gather_add")
+def _(indexes, source, weights):
+    return weights.new_empty(indexes.shape[0], source.shape[1])
+
+
+_L.define("lookup_gather(Tensor code, Tensor score, Tensor tables, Tensor? bias) -> Tensor")
+
+
+def _lookup_gather_impl(code, score, tables, bias):
+    _lib.require_gpu(code, score, tables, bias)
+    assert tables.dim() == 3 and tables.is_contiguous()
+    assert score.dtype == torch.float32 and score.is_contiguous()
+    assert tuple(score.shape) == tuple(code.shape)
+    B, T = code.shape
+    T2, S, Do = tables.shape
+    assert T2 == T and _is_pow2(S)
+    _check_gather_args(code, T * S, Do)
+    if bias is not None:
+        assert bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == Do
+    out = torch.empty(B, Do, dtype=torch.float32, device=tables.device)
+    lib = _lib.load()
+    if tables.dtype == torch.float32:
+        fn, name = lib.lffn_lookup_gather_f32, "lffn_lookup_gather_f32"
+    elif tables.dtype == torch.bfloat16:
+        fn, name = lib.lffn_lookup_gather_bf16, "lffn_lookup_gather_bf16"
+    else:
+        raise NotImplementedError(f"lookup_gather: table dtype {tables.dtype} (float32 and bfloat16 are built)")
+    with _dev_guard(tables):
+        rc = fn(_lib.ptr(code), _lib.ptr(score), _lib.ptr(tables), _lib.ptr(bias), _lib.ptr(out),
+                B, T, S, Do, _lib.stream_of(tables))
+    _lib.check(rc, f"{name}(B={B}, T={T}, S={S}, Do={Do})")
+    return out
+
+
+_L.impl("lookup_gather", _lookup_gather_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::lookup_gather")
+def _(code, score, tables, bias):
+    return score.new_empty(code.shape[0], tables.shape[2])
+
+
+_L.define("indexed_inner_product(Tensor indexes, Tensor source_1, Tensor source_2) -> Tensor")
+
+
+def _inner_impl(indexes, source_1, source_2):
+    _lib.require_gpu(indexes, source_1, source_2)
+    assert source_1.dim() == 2 and source_2.dim() == 2
+    assert source_1.dtype == torch.float32 and source_2.dtype == torch.float32
+    assert source_1.is_contiguous() and source_2.is_contiguous()
+    B, I = indexes.shape
+    S, Dv = source_2.shape
+    assert source_1.shape[0] == B and source_1.shape[1] == Dv
+    _check_gather_args(indexes, S, Dv)
+    out = torch.empty(B, I, dtype=torch.float32, device=source_2.device)
+    with _dev_guard(source_2):
+        rc = _lib.load().lffn_indexed_inner_product_f32(
+            _lib.ptr(indexes), _lib.ptr(source_1), _lib.ptr(source_2), _lib.ptr(out), B, I, S, Dv,
+            _lib.stream_of(source_2))
+    _lib.check(rc, f"lffn_indexed_inner_product_f32(B={B}, I={I}, S={S}, Dv={Dv})")
+    return out
+
+
+_L.impl("indexed_inner_product", _inner_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::indexed_inner_product")
+def _(indexes, source_1, source_2):
+    return source_1.new_empty(indexes.shape)
+
+
+_L.define("scatter_add(Tensor indexes, Tensor source, Tensor weights, int output_size) -> Tensor")
+
+
+def _scatter_impl(indexes, source, weights, output_size):
+    _lib.require_gpu(indexes, source, weights)
+    assert source.dim() == 2 and source.dtype == torch.float32 and source.is_contiguous()
+    assert weights.dtype == torch.float32 and weights.is_contiguous()
+    assert tuple(weights.shape) == tuple(indexes.shape)
+    B, I = indexes.shape
+    Dv = source.shape[1]
+    assert source.shape[0] == B
+    _check_gather_args(indexes, output_size, Dv)
+    out = torch.zeros(output_size, Dv, dtype=torch.float32, device=source.device)
+    with _dev_guard(source):
+        rc = _lib.load().lffn_scatter_add_f32(
+            _lib.ptr(indexes), _lib.ptr(source), _lib.ptr(weights), _lib.ptr(out), B, I, output_size, Dv,
+            _lib.stream_of(source))
+    _lib.check(rc, f"lffn_scatter_add_f32(B={B}, I={I}, out={output_size}, Dv={Dv})")
+    return out
+
+
+_L.impl("scatter_add", _scatter_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::scatter_add")
+def _(indexes, source, weights, output_size):
+    return source.new_empty(output_size, source.shape[1])
+
+
+fht = torch.ops.lookupffn.fht
+bh4_diag = torch.ops.lookupffn.bh4_diag
+project_hash = torch.ops.lookupffn.project_hash
+code_score = torch.ops.lookupffn.code_score
+code_score_bwd = torch.ops.lookupffn.code_score_bwd
+gather_add = torch.ops.lookupffn.gather_add
+lookup_gather = torch.ops.lookupffn.lookup_gather
+indexed_inner_product = torch.ops.lookupffn.indexed_inner_product
+scatter_add = torch.ops.lookupffn.scatter_add

@@ -39,6 +39,10 @@ def lib() -> ctypes.CDLL:
     return _lib
 
 
+def num_threads() -> int:
+    return int(lib().orc_num_threads())
+
+
 def _sfx(dtype) -> str:
     dtype = np.dtype(dtype)
     if dtype == np.float32:

@@ -60,3 +60,11 @@
 #undef SQRT
 
 int orc_version(void) { return 1; }
+
+/* Threads the parallel loops above use (for reporting the CPU baseline). */
+#ifdef _OPENMP
+#include <omp.h>
+int orc_num_threads(void) { return omp_get_max_threads(); }
+#else
+int orc_num_threads(void) { return 1; }
+#endif

@@ -1,0 +1,122 @@
+"""Test helper: call the C ABI of liblookupffn_hip.so directly (ctypes), with
+torch tensors used only as device memory.  Inputs are numpy arrays, outputs come
+back as numpy arrays, so a parity test reads: oracle(numpy) vs cabi(numpy)."""
+import numpy as np
+import torch
+
+from lookupffn_amd import _lib
+
+DEV = "cuda:0"
+
+
+def dev(a):
+    if a is None:
+        return None
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.uint16:    # bfloat16 bit patterns
+        return torch.from_numpy(a.view(np.int16)).to(DEV)
+    return torch.from_numpy(a).to(DEV)
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def _call(name, *args):
+    stream = torch.cuda.current_stream().cuda_stream
+    rc = getattr(_lib.load(), name)(*args, stream)
+    assert rc == 0, f"{name} returned {rc}: {_lib.load().lffn_error_string(rc).decode()}"
+
+
+def p(t):
+    return None if t is None else t.data_ptr()
+
+
+def fht(x):
+    xd = dev(x)
+    out = torch.empty_like(xd)
+    _call("lffn_fht_f32", p(xd), p(out), x.shape[0], x.shape[1])
+    return host(out)
+
+
+def fht_inplace(x):
+    xd = dev(x)
+    _call("lffn_fht_f32", p(xd), p(xd), x.shape[0], x.shape[1])
+    return host(xd)
+
+
+def bh4_diag(x, diag):
+    xd, dd = dev(x), dev(diag)
+    B, H = x.shape
+    R, J, D = diag.shape
+    out = torch.empty(B, R * D, dtype=torch.float32, device=DEV)
+    _call("lffn_bh4_diag_f32", p(xd), p(dd), p(out), B, H, D, R, J)
+    return host(out)
+
+
+def project_hash(x, diag, bias, T, decay=0.7, keep_z=True):
+    xd, dd, bd = dev(x), dev(diag), dev(bias)
+    B, H = x.shape
+    R, J, D = diag.shape
+    codes = torch.full((B, T), -1, dtype=torch.int32, device=DEV)
+    scores = torch.full((B, T), float("nan"), dtype=torch.float32, device=DEV)
+    z = torch.full((B, T * 8), float("nan"), dtype=torch.float32, device=DEV) if keep_z else None
+    _call("lffn_project_hash_f32", p(xd), p(dd), p(bd), p(z), p(codes), p(scores), B, H, D, R, J, T,
+          float(np.float32(decay)), float(np.float32(1 - decay)))
+    return host(codes), host(scores), (host(z) if keep_z else None)
+
+
+def code_score(z):
+    zd = dev(z)
+    k = z.shape[-1]
+    N = z.size // k
+    codes = torch.full(z.shape[:-1], -1, dtype=torch.int32, device=DEV)
+    scores = torch.full(z.shape[:-1], float("nan"), dtype=torch.float32, device=DEV)
+    _call("lffn_code_score_f32", p(zd), p(codes), p(scores), N, k)
+    return host(codes), host(scores)
+
+
+def code_score_bwd(z, g):
+    zd, gd = dev(z), dev(g)
+    k = z.shape[-1]
+    out = torch.full(z.shape, float("nan"), dtype=torch.float32, device=DEV)
+    _call("lffn_code_score_bwd_f32", p(zd), p(gd), p(out), z.size // k, k)
+    return host(out)
+
+
+def gather_add(idx, src, w, bf16=False):
+    idd, sd, wd = dev(idx), dev(src), dev(w)
+    B, I = idx.shape
+    S, Dv = src.shape
+    out = torch.full((B, Dv), float("nan"), dtype=torch.float32, device=DEV)
+    _call("lffn_gather_add_bf16" if bf16 else "lffn_gather_add_f32", p(idd), p(sd), p(wd), p(out), B, I, S, Dv)
+    return host(out)
+
+
+def lookup_gather(code, score, tables, bias=None, bf16=False):
+    cd, sd, td, bd = dev(code), dev(score), dev(tables), dev(bias)
+    B, T = code.shape
+    _, S, Do = tables.shape
+    out = torch.full((B, Do), float("nan"), dtype=torch.float32, device=DEV)
+    _call("lffn_lookup_gather_bf16" if bf16 else "lffn_lookup_gather_f32",
+          p(cd), p(sd), p(td), p(bd), p(out), B, T, S, Do)
+    return host(out)
+
+
+def indexed_inner_product(idx, g, src):
+    idd, gd, sd = dev(idx), dev(g), dev(src)
+    B, I = idx.shape
+    S, Dv = src.shape
+    out = torch.full((B, I), float("nan"), dtype=torch.float32, device=DEV)
+    _call("lffn_indexed_inner_product_f32", p(idd), p(gd), p(sd), p(out), B, I, S, Dv)
+    return host(out)
+
+
+def scatter_add(idx, g, w, out_size, init=None):
+    idd, gd, wd = dev(idx), dev(g), dev(w)
+    B, I = idx.shape
+    Dv = g.shape[1]
+    out = torch.zeros(out_size, Dv, dtype=torch.float32, device=DEV) if init is None else dev(init)
+    _call("lffn_scatter_add_f32", p(idd), p(gd), p(wd), p(out), B, I, out_size, Dv)
+    return host(out)

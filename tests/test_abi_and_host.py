@@ -1,0 +1,136 @@
+"""CPU-only checks of the boundary and host logic: the C-ABI library loads and
+exports every symbol include/lookupffn_hip.h declares, argument validation
+returns error codes without touching a GPU, and the module surface keeps the
+reference's parameter names, shapes and config attributes (PL/lookup.py:10-130).
+No kernel is launched here.
+"""
+import ctypes
+import math
+import os
+import re
+from argparse import Namespace
+
+import pytest
+import torch
+
+import lookupffn_amd
+from lookupffn_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    hdr = open(os.path.join(ROOT, "include", "lookupffn_hip.h")).read()
+    hdr = re.sub(r"/\*.*?\*/", "", hdr, flags=re.S)
+    return sorted(set(re.findall(r"\b(lffn_\w+)\s*\(", hdr)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    names = _declared()
+    assert len(names) >= 12
+    for n in names:
+        assert hasattr(lib, n), n
+    assert names == sorted(_lib.exported_symbols())
+
+
+def test_version_and_error_strings():
+    lib = _lib.load()
+    assert lib.lffn_version() == _lib.ABI_VERSION
+    for code in (0, -1, -2, -3, -99):
+        assert len(lib.lffn_error_string(code)) > 0
+
+
+def test_argument_validation_needs_no_gpu():
+    lib = _lib.load()
+    # null pointers
+    assert lib.lffn_fht_f32(None, None, 4, 8, None) == _lib.LFFN_ERR_BAD_ARG
+    assert lib.lffn_gather_add_f32(None, None, None, None, 4, 2, 8, 64, None) == _lib.LFFN_ERR_BAD_ARG
+    # unsupported shapes (pointers are never dereferenced on the host)
+    assert lib.lffn_fht_f32(256, 256, 4, 2048, None) == _lib.LFFN_ERR_UNSUPPORTED
+    assert lib.lffn_fht_f32(256, 256, 4, 48, None) == _lib.LFFN_ERR_UNSUPPORTED      # not a power of two
+    assert lib.lffn_gather_add_f32(256, 256, 256, 256, 4, 2, 8, 96, None) == _lib.LFFN_ERR_UNSUPPORTED  # Dv % 64
+    assert lib.lffn_code_score_f32(256, 256, 256, 4, 0, None) == _lib.LFFN_ERR_UNSUPPORTED
+    assert lib.lffn_code_score_f32(256, 256, 256, 4, 25, None) == _lib.LFFN_ERR_UNSUPPORTED
+    assert lib.lffn_lookup_gather_f32(256, 256, 256, None, 256, 4, 2, 100, 64, None) == _lib.LFFN_ERR_UNSUPPORTED  # S
+    # misaligned output
+    assert lib.lffn_fht_f32(256, 260, 4, 8, None) == _lib.LFFN_ERR_BAD_ARG
+    # T*8 > R*D
+    assert lib.lffn_project_hash_f32(256, 256, None, None, 256, 256, 4, 16, 16, 1, 4, 3, 0.7, 0.3, None) \
+        == _lib.LFFN_ERR_BAD_ARG
+    # empty batches succeed without a launch
+    assert lib.lffn_fht_f32(256, 256, 0, 8, None) == _lib.LFFN_OK
+    assert lib.lffn_gather_add_f32(256, 256, 256, 256, 0, 2, 8, 64, None) == _lib.LFFN_OK
+    assert lib.lffn_code_score_f32(256, 256, 256, 0, 8, None) == _lib.LFFN_OK
+
+
+def _config(**kw):
+    base = dict(hidden_size=48, ffn_num_table=8, ffn_table_size=256, layer_norm_eps=1e-5,
+                projection_type="bh4", block_size=1)
+    base.update(kw)
+    return Namespace(**base)
+
+
+def test_module_surface_matches_reference_names_and_shapes():
+    m = lookupffn_amd.LookupFFN(_config(hidden_size=768, ffn_num_table=128, block_size=64), 768)
+    sd = m.state_dict()
+    assert set(sd) == {"LayerNorm.weight", "LayerNorm.bias", "hash.projection.weight",
+                       "hash.projection.bias", "tables", "bias"}
+    assert tuple(sd["tables"].shape) == (128, 256, 768)
+    assert tuple(sd["bias"].shape) == (768,)
+    # D = 1024, R = ceil(128*8/1024) = 1, 4 stages, 16 blocks of 64x64  (PL/lookup.py:18-23)
+    assert tuple(sd["hash.projection.weight"].shape) == (1, 4, 16, 64, 64)
+    assert tuple(sd["hash.projection.bias"].shape) == (1024,)
+    assert m.hash.code_length == 8 and m.hash.total_dim == 1024
+    p = m.hash.projection
+    assert (p.padded_in_dim, p.num_repeat, p.num_block, p.decay_coeff) == (1024, 1, 16, 0.7)
+    big = lookupffn_amd.BH4(1024, 4096, 1)
+    assert big.num_repeat == 4 and tuple(big.weight.shape) == (4, 4, 1024, 1, 1)
+
+
+def test_dense_projection_and_bad_projection_type():
+    m = lookupffn_amd.Hashing(_config(projection_type="dense"))
+    assert isinstance(m.projection, torch.nn.Linear)
+    with pytest.raises(NotImplementedError):
+        lookupffn_amd.Hashing(_config(projection_type="other"))
+    with pytest.raises(AssertionError):
+        lookupffn_amd.LookupFFN(_config(ffn_table_size=100), 64)       # PL/lookup.py:88
+
+
+def test_cpu_tensors_fail_loudly():
+    m = lookupffn_amd.LookupFFN(_config(), 64).eval()
+    with pytest.raises(RuntimeError, match="GPU only"):
+        m(torch.randn(3, 48))
+    with pytest.raises(RuntimeError, match="GPU only"):
+        lookupffn_amd.gather(torch.zeros(2, 2, dtype=torch.int32), torch.ones(2, 2), torch.ones(4, 64), False)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        lookupffn_amd.compute_code_score(torch.randn(2, 3, 8), False)
+    with pytest.raises((RuntimeError, NotImplementedError)):
+        lookupffn_amd.hadamard(torch.randn(2, 8))       # no CPU kernel registered for the op
+
+
+def test_slow_torch_hooks_match_closed_forms():
+    # use_torch=True keeps the reference's slow formulas; they run on any device
+    import scipy.linalg
+    x = torch.randn(3, 16, dtype=torch.float64)
+    want = x @ torch.tensor(scipy.linalg.hadamard(16), dtype=torch.float64)
+    assert torch.allclose(lookupffn_amd.hadamard(x, use_torch=True), want)
+    z = torch.tensor([[[1.0, -1, 1, -1, 0, 2, -3, 4]]])
+    code, score = lookupffn_amd.compute_code_score_torch(z)
+    assert code.item() == 0b10100101
+    idx = torch.tensor([[0, 3], [2, 2]], dtype=torch.int32)
+    src = torch.arange(4 * 64, dtype=torch.float32).reshape(4, 64)
+    w = torch.tensor([[1.0, 2.0], [0.5, 0.5]])
+    out = lookupffn_amd.weighted_gather_add(idx, src, w, use_torch=True)
+    assert torch.equal(out[0], src[0] + 2 * src[3]) and torch.equal(out[1], src[2])
+
+
+def test_ops_have_fake_implementations():
+    # shape inference without a device (meta tensors)
+    x = torch.empty(5, 48, device="meta")
+    diag = torch.empty(1, 4, 64, device="meta")
+    c, s, z = torch.ops.lookupffn.project_hash(x, diag, None, 8, 0.7, 0.3, True)
+    assert c.shape == (5, 8) and c.dtype == torch.int32 and s.shape == (5, 8) and z.shape == (5, 64)
+    t = torch.empty(8, 256, 64, device="meta")
+    assert torch.ops.lookupffn.lookup_gather(c, s, t, None).shape == (5, 64)
+    assert torch.ops.lookupffn.fht(torch.empty(3, 64, device="meta")).shape == (3, 64)

@@ -1,0 +1,335 @@
+"""GPU parity: every C-ABI entry point against the CPU oracle on the same seeded
+inputs (sizes the oracle finishes in seconds), against the committed golden
+fixtures, and at the BASELINE.json shapes through size-independent properties.
+
+Tolerances (stated once, used below):
+  * FHT / BH4 mixing: <= 1e-5 of the largest reference magnitude; in fact the
+    kernel runs the reference's butterfly order with one rounding per stage, so
+    the float32 oracle is matched bit for bit and the tests assert that.
+  * codes: bit-exact given identical z.
+  * scores and their gradient: <= 2e-6 relative (exp differs by <= 1 ulp).
+  * gather-add fp32 and inner product: <= 1e-5 of the largest reference magnitude
+    (fused multiply-add vs multiply-then-add).
+  * bf16 tables: <= 1e-5 against the oracle on the same bf16 table, <= 1e-2
+    against the fp32-table result.
+  * scatter-add: <= 1e-5 of the largest magnitude (atomic order is free).
+"""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+from tests import _cabi as cabi
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _need_gpu():
+    assert torch.cuda.is_available(), "GPU tests need an MI355X"
+    yield
+
+
+@pytest.fixture(scope="module")
+def golden(golden_dir):
+    with open(os.path.join(golden_dir, "lookupffn_golden.json")) as f:
+        return json.load(f)
+
+
+def relmax(got, want):
+    want = np.asarray(want, dtype=np.float64)
+    scale = max(np.abs(want).max(), 1e-30)
+    return float(np.abs(np.asarray(got, dtype=np.float64) - want).max() / scale)
+
+
+# ----------------------------------------------------------------------------- FHT
+
+def test_fht_golden(golden):
+    for D, g in golden["hadamard"].items():
+        x = np.array(g["x"], dtype=np.float32)
+        assert np.array_equal(cabi.fht(x), np.array(g["xH"], dtype=np.float32))
+
+
+@pytest.mark.parametrize("D", [4, 8, 16, 32, 64, 128, 256, 512, 1024])
+@pytest.mark.parametrize("B", [1, 7, 300])
+def test_fht_matches_oracle(B, D):
+    rng = np.random.RandomState(B * 10007 + D)
+    x = rng.randn(B, D).astype(np.float32)
+    want64 = oracle.fht(x.astype(np.float64))
+    got = cabi.fht(x)
+    assert relmax(got, want64) <= 1e-5
+    assert np.array_equal(got, oracle.fht(x))           # same order, one rounding per stage
+    assert np.array_equal(cabi.fht_inplace(x), got)
+
+
+def test_fht_integer_inputs_exact_and_involution():
+    rng = np.random.RandomState(5)
+    D = 1024
+    x = rng.randint(-8, 9, size=(64, D)).astype(np.float32)
+    y = cabi.fht(x)
+    import scipy.linalg
+    assert np.array_equal(y.astype(np.float64), x.astype(np.float64) @ scipy.linalg.hadamard(D))
+    assert np.array_equal(cabi.fht(y), D * x)            # H.H = D.I, exact on integers
+    e = np.zeros((1, D), np.float32); e[0, 0] = 1
+    assert np.array_equal(cabi.fht(e), np.ones((1, D), np.float32))
+
+
+def test_fht_full_size_properties():
+    # BASELINE config 2 shape: 16384 x 1024; linearity + Parseval + involution
+    rng = np.random.RandomState(6)
+    B, D = 16384, 1024
+    x = rng.randn(B, D).astype(np.float32)
+    y = cabi.fht(x)
+    n_in = (x.astype(np.float64) ** 2).sum(1)
+    n_out = (y.astype(np.float64) ** 2).sum(1)
+    assert np.abs(n_out / (D * n_in) - 1).max() < 1e-5
+    assert relmax(cabi.fht(y), D * x.astype(np.float64)) <= 1e-5
+    sub = rng.choice(B, 64, replace=False)
+    assert np.array_equal(y[sub], oracle.fht(x[sub]))
+
+
+# ----------------------------------------------------------------------------- BH4 diag / projection + hash
+
+@pytest.mark.parametrize("H,D,R,J", [(256, 256, 1, 4), (768, 1024, 1, 4), (1024, 1024, 4, 4), (48, 64, 2, 1),
+                                      (100, 128, 1, 3), (6, 8, 1, 2), (511, 512, 2, 4)])
+def test_bh4_diag_matches_oracle(H, D, R, J):
+    rng = np.random.RandomState(H + D + R)
+    B = 37
+    x = rng.randn(B, H).astype(np.float32)
+    diag = (rng.randn(R, J, D) / math.sqrt(D)).astype(np.float32)
+    xp = np.concatenate([x, np.zeros((B, D - H), np.float32)], axis=1)
+    want = oracle.bh4(xp, diag.reshape(R, J, D, 1, 1))
+    got = cabi.bh4_diag(x, diag)
+    assert np.array_equal(got, want)
+    want64 = oracle.bh4(xp.astype(np.float64), diag.reshape(R, J, D, 1, 1).astype(np.float64))
+    assert relmax(got, want64) <= 1e-5
+
+
+def test_sign_diagonal_fht_exact():
+    # the BASELINE "random +-1 sign diagonal from seed": one round, exact on integers
+    rng = np.random.RandomState(8)
+    B, D = 33, 1024
+    x = rng.randint(-8, 9, size=(B, D)).astype(np.float32)
+    s = (2 * rng.randint(0, 2, size=(1, 1, D)) - 1).astype(np.float32)
+    import scipy.linalg
+    want = (x * s[0, 0]).astype(np.float64) @ scipy.linalg.hadamard(D)
+    assert np.array_equal(cabi.bh4_diag(x, s).astype(np.float64), want)
+
+
+@pytest.mark.parametrize("H,D,R,T", [(256, 256, 1, 32), (768, 1024, 1, 128), (1024, 1024, 4, 512),
+                                      (48, 64, 1, 5), (100, 128, 2, 30), (8, 8, 1, 1)])
+def test_project_hash_matches_oracle(H, D, R, T):
+    rng = np.random.RandomState(H * 3 + T)
+    B, J = 41, 4
+    x = rng.randn(B, H).astype(np.float32)
+    diag = (rng.randn(R, J, D) / math.sqrt(D)).astype(np.float32)
+    bias = (0.1 * rng.randn(T * 8)).astype(np.float32)
+    z_want = oracle.projection(x, diag.reshape(R, J, D, 1, 1), bias, T * 8, np.float32(0.7))
+    code_want, score_want = oracle.code_score(z_want.reshape(B, T, 8))
+    codes, scores, z = cabi.project_hash(x, diag, bias, T)
+    assert np.array_equal(z, z_want)                      # identical operations in identical order
+    assert np.array_equal(codes, code_want)               # so the codes are bit-exact end to end
+    np.testing.assert_allclose(scores, score_want, rtol=2e-6, atol=0)
+    codes2, scores2, _ = cabi.project_hash(x, diag, bias, T, keep_z=False)
+    assert np.array_equal(codes2, codes) and np.array_equal(scores2, scores)
+    codes3, _, z3 = cabi.project_hash(x, diag, None, T)
+    z_nb = oracle.projection(x, diag.reshape(R, J, D, 1, 1), None, T * 8, np.float32(0.7))
+    assert np.array_equal(z3, z_nb) and np.array_equal(codes3, oracle.code_score(z_nb.reshape(B, T, 8))[0])
+
+
+def test_project_hash_near_zero_flip_count():
+    # end to end against the float64 truth: flips may only happen where |z| is tiny
+    rng = np.random.RandomState(9)
+    B, H, D, R, J, T = 2048, 768, 1024, 1, 4, 128
+    x = rng.randn(B, H).astype(np.float32)
+    diag = ((2 * rng.randint(0, 2, size=(R, J, D)) - 1) / math.sqrt(D)).astype(np.float32)
+    codes, _, z = cabi.project_hash(x, diag, None, T)
+    z64 = oracle.projection(x.astype(np.float64), diag.reshape(R, J, D, 1, 1).astype(np.float64), None, T * 8, 0.7)
+    code64, _ = oracle.code_score(z64.reshape(B, T, 8))
+    bits = (z.reshape(B, T, 8) > 0) != (z64.reshape(B, T, 8) > 0)
+    flips = int(bits.sum())
+    tiny = int((np.abs(z64) < 1e-6).sum())
+    print(f"sign flips vs float64 truth: {flips} of {bits.size} (|z| < 1e-6: {tiny})")
+    assert np.all(np.abs(z64.reshape(B, T, 8)[bits]) < 1e-5)
+    assert (codes != code64).sum() <= flips
+
+
+# ----------------------------------------------------------------------------- code + score
+
+def test_code_golden(golden):
+    z = np.array(golden["codes"]["z"], dtype=np.float32)
+    codes, _ = cabi.code_score(z)
+    assert np.array_equal(codes, np.array(golden["codes"]["code"], dtype=np.int32))
+    for zz, want in zip(golden["score"]["z"], golden["score"]["score"]):
+        _, s = cabi.code_score(np.array([zz], dtype=np.float32))
+        assert abs(float(s[0]) - want) <= 2e-6 * max(1.0, abs(want))
+
+
+@pytest.mark.parametrize("k", [1, 2, 3, 4, 7, 8, 11, 12, 16, 24])
+def test_code_score_matches_oracle(k):
+    rng = np.random.RandomState(k)
+    z = rng.randn(257, 13, k).astype(np.float32)
+    z[0, 0, : min(k, 3)] = [0.0, -0.0, np.nan][: min(k, 3)]
+    code_want, score_want = oracle.code_score(z)
+    codes, scores = cabi.code_score(z)
+    assert np.array_equal(codes, code_want)
+    ok = ~np.isnan(score_want)
+    np.testing.assert_allclose(scores[ok], score_want[ok], rtol=2e-6, atol=0)
+    assert np.array_equal(np.isnan(scores), np.isnan(score_want))
+
+
+def test_code_score_bwd_matches_oracle():
+    rng = np.random.RandomState(12)
+    for k in (3, 8):
+        z = rng.randn(300, 9, k).astype(np.float32)
+        z[0, 0, 0] = 0.0
+        g = rng.randn(300, 9).astype(np.float32)
+        want = oracle.code_score_bwd(z.astype(np.float64), g.astype(np.float64))
+        got = cabi.code_score_bwd(z, g)
+        np.testing.assert_allclose(got, want, rtol=2e-5, atol=1e-6)
+
+
+# ----------------------------------------------------------------------------- gather-add
+
+def _rand_gather(rng, B, T, S, Do):
+    tables = (0.02 * rng.randn(T, S, Do)).astype(np.float32)
+    code = rng.randint(0, S, size=(B, T)).astype(np.int32)
+    idx = code + (np.arange(T, dtype=np.int32) * S)[None]
+    w = (1.0 - rng.rand(B, T)).astype(np.float32)
+    return tables, code, idx, w
+
+
+def test_gather_golden(golden):
+    g = golden["gather"]
+    tables = np.array(g["tables"], dtype=np.float32)
+    T, S, Do = tables.shape
+    code = np.array(g["code"], dtype=np.int32)
+    idx = code + (np.arange(T, dtype=np.int32) * S)[None]
+    w = np.array(g["w"], dtype=np.float32)
+    flat = tables.reshape(T * S, Do)
+    want = np.array(g["out"], dtype=np.float32)
+    assert np.array_equal(cabi.gather_add(idx, flat, w), want)
+    assert np.array_equal(cabi.gather_add(idx, oracle.bf16_round(flat), w, bf16=True), want)
+    gout = np.array(g["g_out"], dtype=np.float32)
+    assert np.array_equal(cabi.indexed_inner_product(idx, gout, flat), np.array(g["g_w"], dtype=np.float32))
+    assert np.array_equal(cabi.scatter_add(idx, gout, w, T * S).reshape(T, S, Do),
+                          np.array(g["g_tables"], dtype=np.float32))
+
+
+# (B, T, S, Do): config 1, ragged token counts, every lanes-per-token / vectors-per-lane tiling,
+# index counts that are not multiples of the staging chunk or the unroll
+GATHER_CASES = [(256, 32, 256, 256), (1, 2, 4, 64), (5, 6, 16, 128), (67, 10, 8, 192), (33, 130, 4, 768),
+                (19, 64, 256, 1024), (9, 4, 8, 320), (130, 66, 16, 512), (3, 2, 2, 1920), (40, 128, 256, 768)]
+
+
+@pytest.mark.parametrize("B,T,S,Do", GATHER_CASES)
+def test_gather_add_matches_oracle(B, T, S, Do):
+    rng = np.random.RandomState(B + T + Do)
+    tables, code, idx, w = _rand_gather(rng, B, T, S, Do)
+    flat = tables.reshape(T * S, Do)
+    want64 = oracle.gather_add(idx, flat.astype(np.float64), w.astype(np.float64))
+    want32 = oracle.gather_add(idx, flat, w)
+    got = cabi.gather_add(idx, flat, w)
+    assert relmax(got, want64) <= 1e-5
+    assert relmax(got, want32) <= 1e-5
+    # arbitrary (not per-table) indices, as the reference's own unit test draws them
+    idx_any = rng.randint(0, T * S, size=(B, T)).astype(np.int32)
+    assert relmax(cabi.gather_add(idx_any, flat, w), oracle.gather_add(idx_any, flat.astype(np.float64), w.astype(np.float64))) <= 1e-5
+    # the layer's form: table-local codes, offset and bias folded in
+    bias = (0.001 * rng.randn(Do)).astype(np.float32)
+    if S & (S - 1) == 0:
+        assert relmax(cabi.lookup_gather(code, w, tables, None), want64) <= 1e-5
+        assert relmax(cabi.lookup_gather(code, w, tables, bias), want64 + bias) <= 1e-5
+
+
+@pytest.mark.parametrize("B,T,S,Do", GATHER_CASES)
+def test_gather_add_bf16_matches_oracle(B, T, S, Do):
+    rng = np.random.RandomState(B + T + Do + 1)
+    tables, code, idx, w = _rand_gather(rng, B, T, S, Do)
+    flat = tables.reshape(T * S, Do)
+    bits = oracle.bf16_round(flat)
+    want_bf = oracle.gather_add_bf16(idx, bits, w.astype(np.float64))
+    want_f32 = oracle.gather_add(idx, flat.astype(np.float64), w.astype(np.float64))
+    got = cabi.gather_add(idx, bits, w, bf16=True)
+    assert relmax(got, want_bf) <= 1e-5
+    assert relmax(got, want_f32) <= 1e-2
+    if S & (S - 1) == 0:
+        assert relmax(cabi.lookup_gather(code, w, bits.reshape(T, S, Do), None, bf16=True), want_bf) <= 1e-5
+
+
+def test_gather_special_cases():
+    rng = np.random.RandomState(30)
+    tables, code, idx, w = _rand_gather(rng, 16, 8, 16, 128)
+    flat = tables.reshape(-1, 128)
+    onehot = np.zeros_like(w); onehot[:, 3] = 1.0
+    assert np.array_equal(cabi.gather_add(idx, flat, onehot), flat[idx[:, 3]])
+    np.testing.assert_allclose(cabi.gather_add(idx, np.ones_like(flat), w)[:, 5], w.astype(np.float64).sum(1), rtol=1e-6)
+    # out-of-range indices are clamped, never dereferenced
+    bad = idx.copy(); bad[0, 0] = -5; bad[1, 1] = 10 ** 6
+    ref = idx.copy(); ref[0, 0] = 0; ref[1, 1] = flat.shape[0] - 1
+    assert np.array_equal(cabi.gather_add(bad, flat, w), cabi.gather_add(ref, flat, w))
+    # index count 0: zeros (or the bias)
+    empty = cabi.gather_add(np.zeros((4, 0), np.int32), flat, np.zeros((4, 0), np.float32))
+    assert np.array_equal(empty, np.zeros((4, 128), np.float32))
+
+
+def test_gather_full_size_properties():
+    # BASELINE config 2: 16384 tokens, 128 tables x 256 x 768 fp32
+    rng = np.random.RandomState(31)
+    B, T, S, Do = 16384, 128, 256, 768
+    tables, code, idx, w = _rand_gather(rng, B, T, S, Do)
+    flat = tables.reshape(T * S, Do)
+    out = cabi.lookup_gather(code, w, tables, None)
+    out_flat = cabi.gather_add(idx, flat, w)
+    assert relmax(out_flat, out) <= 1e-6
+    sub = rng.choice(B, 48, replace=False)
+    want = oracle.gather_add(idx[sub], flat.astype(np.float64), w[sub].astype(np.float64))
+    assert relmax(out[sub], want) <= 1e-5
+    # linearity in the weights: G(a*w1 + w2) = a*G(w1) + G(w2)
+    w2 = rng.rand(B, T).astype(np.float32)
+    lhs = cabi.lookup_gather(code, (2 * w + w2).astype(np.float32), tables, None)
+    rhs = 2 * out.astype(np.float64) + cabi.lookup_gather(code, w2, tables, None)
+    assert relmax(lhs, rhs) <= 1e-5
+    # checksum: sum_b out[b] = sum_{t,s} (sum_{b: code=s} w) * tables[t,s]
+    cnt = np.zeros((T, S), np.float64)
+    np.add.at(cnt, (np.broadcast_to(np.arange(T), (B, T)), code), w.astype(np.float64))
+    want_sum = np.einsum("ts,tsd->d", cnt, tables.astype(np.float64))
+    assert relmax(out.astype(np.float64).sum(0), want_sum) <= 1e-5
+
+
+# ----------------------------------------------------------------------------- backward
+
+@pytest.mark.parametrize("B,T,S,Do", [(256, 32, 256, 256), (5, 6, 16, 128), (67, 10, 8, 192), (33, 130, 4, 768),
+                                      (9, 4, 8, 320), (3, 2, 2, 1920), (19, 64, 256, 1024)])
+def test_backward_matches_oracle(B, T, S, Do):
+    rng = np.random.RandomState(B + T + Do + 2)
+    tables, code, idx, w = _rand_gather(rng, B, T, S, Do)
+    flat = tables.reshape(T * S, Do)
+    g = rng.randn(B, Do).astype(np.float32)
+    want_w = oracle.indexed_inner_product(idx, g.astype(np.float64), flat.astype(np.float64))
+    assert relmax(cabi.indexed_inner_product(idx, g, flat), want_w) <= 1e-5
+    want_t = oracle.scatter_add(idx, g.astype(np.float64), w.astype(np.float64), T * S)
+    got_t = cabi.scatter_add(idx, g, w, T * S)
+    assert relmax(got_t, want_t) <= 1e-5
+    # accumulates into what is already there
+    init = rng.randn(T * S, Do).astype(np.float32)
+    assert relmax(cabi.scatter_add(idx, g, w, T * S, init=init), want_t + init) <= 1e-5
+
+
+def test_scatter_duplicates_zipf():
+    # heavy duplication of rows (BASELINE config 5 draws codes Zipf(1.1))
+    rng = np.random.RandomState(40)
+    B, T, S, Do = 2048, 16, 256, 256
+    p = 1.0 / np.arange(1, S + 1) ** 1.1
+    p /= p.sum()
+    code = rng.choice(S, size=(B, T), p=p).astype(np.int32)
+    idx = code + (np.arange(T, dtype=np.int32) * S)[None]
+    w = (1.0 - rng.rand(B, T)).astype(np.float32)
+    g = rng.randn(B, Do).astype(np.float32)
+    want = oracle.scatter_add(idx, g.astype(np.float64), w.astype(np.float64), T * S)
+    assert relmax(cabi.scatter_add(idx, g, w, T * S), want) <= 1e-5
