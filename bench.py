@@ -1,0 +1,227 @@
+"""Benchmark of the LookupFFN hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg1|cfg3|cfg3bf16]
+
+A step is one forward pass of the layer over one batch of synthetic tokens that
+is already resident in HBM: LayerNorm (PyTorch-ROCm) -> fused projection+hash
+kernel -> gather-add kernel (+bias).  Prints ONE JSON line:
+
+  value        whole-layer forward tokens/s (BASELINE.json's metric, config 2 by default)
+  roofline     the gather-add kernel: algorithmic ("logical") bytes per launch
+               = B*T*Do*e + B*T*8 + B*Do*4, divided by the kernel's average
+               duration measured with HIP events on the launch stream inside the
+               timed region, against the 8 TB/s HBM peak
+  cpu_baseline the CPU oracle (OpenMP C restatement of the reference's layer) on a
+               bounded sample of the same workload, on the host cores of this box
+
+One GPU only: this path has no multi-GPU form in this build.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+from argparse import Namespace
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (B, H, T, S, Do, table dtype)          BASELINE.json configs[0..2]
+    "cfg1": dict(B=256, H=256, T=32, S=256, Do=256, bf16=False,
+                 desc="config 1: 2x128 tokens, d=256, 32 tables x 256 x 256 fp32"),
+    "cfg2": dict(B=16384, H=768, T=128, S=256, Do=768, bf16=False,
+                 desc="config 2 (RoBERTa-base): 32x512 tokens, d=768 padded to 1024, 128 tables x 256 x 768 fp32"),
+    "cfg3": dict(B=16384, H=1024, T=512, S=256, Do=1024, bf16=False,
+                 desc="config 3: 16384 tokens, d=1024, 512 tables x 256 x 1024 fp32"),
+    "cfg3bf16": dict(B=16384, H=1024, T=512, S=256, Do=1024, bf16=True,
+                     desc="config 3: 16384 tokens, d=1024, 512 tables x 256 x 1024 bf16 rows, fp32 accumulate"),
+}
+
+# HBM bytes per launch of the gather kernel measured with rocprofv3 --pmc
+# (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); the summaries
+# are kept under profiles/.  None until measured for that workload.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def build_layer(wl, device):
+    import torch
+
+    import lookupffn_amd
+
+    cfg = Namespace(hidden_size=wl["H"], ffn_num_table=wl["T"], ffn_table_size=wl["S"],
+                    layer_norm_eps=1e-5, projection_type="bh4", block_size=1)
+    g = torch.Generator().manual_seed(1234)
+    layer = lookupffn_amd.LookupFFN(cfg, wl["Do"]).eval()
+    p = layer.hash.projection
+    with torch.no_grad():
+        # seeded +-1 sign diagonals, scaled by 1/sqrt(D) so that each of the four
+        # (diagonal, Hadamard) stages is orthonormal
+        sign = 2.0 * torch.randint(0, 2, p.weight.shape, generator=g).float() - 1.0
+        p.weight.copy_(sign / math.sqrt(p.padded_in_dim))
+        layer.tables.copy_(0.02 * torch.randn(layer.tables.shape, generator=g))
+        layer.bias.copy_(0.001 * torch.randn(layer.bias.shape, generator=g))
+    x = torch.randn(wl["B"], wl["H"], generator=g)
+    layer = layer.to(device)
+    if wl["bf16"]:
+        layer.tables.data = layer.tables.data.to(torch.bfloat16)
+    return layer, x
+
+
+def cpu_baseline(layer, x, wl, budget_s=12.0):
+    """The oracle's whole-layer forward on a slice of the same tokens, all host cores."""
+    import numpy as np
+
+    import oracle
+
+    npf = lambda t: t.detach().float().cpu().numpy()
+    p = layer.hash.projection
+    args = (npf(layer.LayerNorm.weight), npf(layer.LayerNorm.bias), np.float32(layer.LayerNorm.eps),
+            npf(p.weight), npf(p.bias), npf(layer.tables), npf(layer.bias))
+    n = min(wl["B"], 2048)
+    xs = np.ascontiguousarray(npf(x)[:n])
+    oracle.lookup_ffn(xs, *args, decay=np.float32(p.decay_coeff))          # warm-up (page-in)
+    reps, t_total = 0, 0.0
+    while reps < 3 or (t_total < budget_s and reps < 5000):
+        t0 = time.perf_counter()
+        oracle.lookup_ffn(xs, *args, decay=np.float32(p.decay_coeff))
+        t_total += time.perf_counter() - t0
+        reps += 1
+    out = {"value": n * reps / t_total, "unit": "tokens/s", "cores": oracle.num_threads(), "kind": "port",
+           "sample": f"first {n} of {wl['B']} tokens, full tables, {reps} passes of the OpenMP C oracle "
+                     f"(whole layer, fp32{' on bf16-rounded tables' if wl['bf16'] else ''}), {t_total:.1f} s"}
+    # the reference's own x86 kernels (compiled from its sources), gather + code/score legs only
+    try:
+        import torch
+        ga = oracle.load_ref("gather_add_cpu")
+        if ga is not None and wl["S"] == 256 and n % 64 == 0:
+            torch.set_num_threads(oracle.num_threads())
+            T, S = wl["T"], wl["S"]
+            idx = torch.randint(0, S, (n, T), dtype=torch.int32) + torch.arange(T, dtype=torch.int32)[None] * S
+            w = torch.rand(n, T)
+            flat = layer.tables.detach().float().cpu().reshape(T * S, wl["Do"])
+            ga.weighted_vector_gather_add_avx2_par(idx, flat, w)
+            t0 = time.perf_counter()
+            r = 0
+            while r < 3 or time.perf_counter() - t0 < 3.0:
+                ga.weighted_vector_gather_add_avx2_par(idx, flat, w)
+                r += 1
+            out["reference_gather_tokens_per_s"] = n * r / (time.perf_counter() - t0)
+    except Exception as e:   # the reference build is optional
+        out["reference_gather_error"] = repr(e)
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 1 GiB device-to-device copy, so that a rocprofv3 --pmc run of "
+                         "this command holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs the LookupFFN hot path on ONE GPU only "
+              "(no multi-GPU form exists); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from lookupffn_amd import _lib, ops
+    _lib.load()                       # fail here, loudly, if the HIP library is missing
+    assert torch.cuda.is_available(), "bench.py needs an MI355X"
+    dev = torch.device("cuda:0")
+    wl = WORKLOADS[args.workload]
+    B, H, T, S, Do = wl["B"], wl["H"], wl["T"], wl["S"], wl["Do"]
+    layer, x_cpu = build_layer(wl, dev)
+    x = x_cpu.to(dev)
+    esz = 2 if wl["bf16"] else 4
+    gather_bytes = B * T * Do * esz + B * T * 8 + B * Do * 4
+
+    def step(events=None):
+        with torch.no_grad():
+            h = layer.LayerNorm(x)
+            code, score = layer.hash(h)
+            if events is not None:
+                events[0].record()
+            out = ops.lookup_gather(code, score, layer.tables, layer.bias)
+            if events is not None:
+                events[1].record()
+        return out
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)                 # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        out = step(evs[i])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    sec = t1 - t0
+    gather_ms = sum(a.elapsed_time(b) for a, b in evs) / args.steps
+    achieved = gather_bytes / (gather_ms * 1e-3) / 1e9
+
+    # stage breakdown (outside the timed region)
+    def timed(fn, n=20):
+        fn(); torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(n):
+            fn()
+        b.record(); torch.cuda.synchronize()
+        return a.elapsed_time(b) / n
+    with torch.no_grad():
+        h = layer.LayerNorm(x)
+        code, score = layer.hash(h)
+        ln_ms = timed(lambda: layer.LayerNorm(x))
+        hash_ms = timed(lambda: layer.hash(h))
+
+    res = {
+        "metric": "LookupFFN fwd tokens/s + gather-add GB/s as % of HBM peak, RoBERTa-base",
+        "value": B * args.steps / sec,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": sec / args.steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16 rows, f32 accumulate" if wl["bf16"] else "f32",
+        "data": "synthetic (seeded N(0,1) tokens, seeded +-1/sqrt(D) sign diagonals, N(0,0.02) tables)",
+        "config": {"workload": wl["desc"], "tokens": B, "d_model": H, "fht_dim": layer.hash.projection.padded_in_dim,
+                   "tables": T, "table_size": S, "d_out": Do, "step": "LayerNorm + fused BH4(block 1)x4 + hash + gather-add + bias"},
+        "roofline": {"bound": "hbm", "kernel": "lookup_gather", "achieved": achieved, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "algorithmic_bytes": gather_bytes, "avg_kernel_ms": gather_ms},
+        "stages_ms": {"layernorm": ln_ms, "project_hash": hash_ms, "gather_add": gather_ms},
+        "gather_tokens_per_s": B / (gather_ms * 1e-3),
+    }
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline(layer, x_cpu, wl)
+    else:
+        res["cpu_baseline"] = None
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()
