@@ -146,6 +146,15 @@ int lffn_lookup_gather_bf16(const int32_t *code, const float *score, const uint1
                             int64_t B, int64_t T, int64_t S, int64_t Do, void *stream);
 
 /*
+ * Which kernel lffn_lookup_gather_{f32,bf16} runs for a shape: the number of
+ * tokens whose accumulators one workgroup keeps in registers while it walks the
+ * tables through LDS, or 0 when the token-major kernel is used (small batches,
+ * S > 256).  Pure host function, no GPU work; negative on bad arguments.
+ * No counterpart in the reference (its gather has one kernel, gather_fp32.cu:6-36).
+ */
+int lffn_lookup_gather_plan(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t bf16);
+
+/*
  * out[b,i] = <g[b,:], src[idx[b,i],:]>   (gradient w.r.t. the weights).
  * g: [B, Dv]; src: [source_size, Dv]; out: [B, I].
  * Replaces gather_add.indexed_inner_product_fp32 (gather_fp32.cu:69-98,

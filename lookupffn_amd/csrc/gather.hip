@@ -382,18 +382,15 @@ extern "C" int lffn_gather_add_bf16(const int32_t *idx, const uint16_t *src, con
     return gather_entry<true>(idx, src, w, nullptr, out, B, I, source_size, Dv, 0, stream);
 }
 
-extern "C" int lffn_lookup_gather_f32(const int32_t *code, const float *score, const float *tables,
-                                      const float *bias, float *out,
-                                      int64_t B, int64_t T, int64_t S, int64_t Do, void *stream) {
-    LFFN_REQUIRE(lffn_is_pow2(S) && S <= (1 << 24) && T >= 0 && T * S <= 0x7fffffff, LFFN_ERR_UNSUPPORTED);
-    return gather_entry<false>(code, tables, score, bias, out, B, T, T * S > 0 ? T * S : 1, Do, S, stream);
-}
-
-extern "C" int lffn_lookup_gather_bf16(const int32_t *code, const float *score, const uint16_t *tables,
-                                       const float *bias, float *out,
-                                       int64_t B, int64_t T, int64_t S, int64_t Do, void *stream) {
-    LFFN_REQUIRE(lffn_is_pow2(S) && S <= (1 << 24) && T >= 0 && T * S <= 0x7fffffff, LFFN_ERR_UNSUPPORTED);
-    return gather_entry<true>(code, tables, score, bias, out, B, T, T * S > 0 ? T * S : 1, Do, S, stream);
+// Token-major kernel on table-local codes (offset i*S and bias folded in): the
+// form lookup_gather.hip falls back to for shapes its LDS-tiled kernel is not
+// built for.
+int lffn_internal_lookup_gather_token_major(const int32_t *code, const float *score, const void *tables,
+                                            const float *bias, float *out, int64_t B, int64_t T, int64_t S,
+                                            int64_t Do, bool bf16, void *stream) {
+    const int64_t rows = T * S > 0 ? T * S : 1;
+    return bf16 ? gather_entry<true>(code, tables, score, bias, out, B, T, rows, Do, S, stream)
+                : gather_entry<false>(code, tables, score, bias, out, B, T, rows, Do, S, stream);
 }
 
 extern "C" int lffn_indexed_inner_product_f32(const int32_t *idx, const float *g, const float *src, float *out,

@@ -1,0 +1,325 @@
+// The weighted gather-add as the LookupFFN layer issues it, table-major with the
+// table staged in LDS:
+//
+//   out[b,:] = bias + sum_t score[b,t] * tables[t, code[b,t] & (S-1), :]
+//
+// (PL/lookup.py:120-130 with the index offset of ":126" and the bias of ":108" folded
+// in; the accumulation runs t = 0..T-1 as in gather_kernel_fp32.cu:41-43.)
+//
+// Work decomposition.  A workgroup of 1024 lanes owns a column slice of 256 bytes
+// per row (64 fp32 or 128 bf16 columns) and a tile of 64*NP tokens, whose
+// accumulators live in registers for the whole kernel (NP float4 per lane: 16
+// lanes side by side cover the 256-byte row segment of one token, a wavefront
+// covers 4 tokens at a time, NP passes cover the tile).  For every table the
+// workgroup copies that table's slice (S rows x 256 bytes, 64 KiB for S = 256)
+// into LDS once and all of its tokens read their rows from there: 16 lanes read
+// 256 contiguous bytes, one conflict-free ds_read_b128.  The slices are
+// double-buffered: the global loads of table t+1 are issued before the LDS reads
+// of table t and land in the other buffer, one barrier per table.
+//
+// So each table slice is fetched once per 64*NP tokens instead of once per
+// token, and the per-token row reads are LDS reads.  The (code, score) pairs are
+// read 16 tables at a time, one table per lane of the 16-lane token group, and
+// handed to the group's lanes with ds_bpermute when their table comes up.
+//
+// blockIdx -> (slice, token tile) is XCD-aware: workgroups are dealt round-robin
+// to the 8 XCDs, so block b runs on XCD b % 8; units are numbered so that the
+// workgroups of one XCD share as few slices as possible and the slice they
+// stream stays in that XCD's L2.
+#include "lffn_common.h"
+
+namespace {
+
+constexpr int WG = 1024;
+constexpr int SEG_VECS = 16;          // 16-byte vectors per row segment (256 bytes)
+constexpr int CHUNK = 16;             // tables whose (code, score) a lane group holds at once
+constexpr int MAX_S = 256;            // rows per table the LDS buffers are sized for
+constexpr int XCDS = 8;
+
+struct LdsGatherArgs {
+    const int32_t *code;   // [B, T]
+    const float *score;    // [B, T]
+    const char *tables;    // [T, S, Do] fp32 or bf16
+    const float *bias;     // [Do] or null
+    float *out;            // [B, Do]
+    int64_t B;
+    int T, S, Do;
+    int ntiles, nslices, per_xcd;
+    int row_bytes;         // Do * element size
+};
+
+// One lane's share of a table slice: four 16-byte vectors, q = tid + 1024*i,
+// row q/16, vector q%16 of the 256-byte row segment.  Plain members (not an
+// array) so that they stay in registers across the table loop.
+struct SliceRegs {
+    uint4 v0, v1, v2, v3;
+};
+
+// FULL: the table has exactly MAX_S rows, so every lane moves all four vectors.
+template <bool FULL>
+__device__ __forceinline__ SliceRegs fetch_slice(const char *tb, int row_bytes, int tid, int buf_vecs) {
+    SliceRegs r;
+    const char *p = tb + (size_t)(tid >> 4) * row_bytes + (tid & 15) * 16;
+    const size_t step = (size_t)(WG / SEG_VECS) * row_bytes;   // 64 rows further down
+    if constexpr (FULL) {
+        r.v0 = *reinterpret_cast<const uint4 *>(p);
+        r.v1 = *reinterpret_cast<const uint4 *>(p + step);
+        r.v2 = *reinterpret_cast<const uint4 *>(p + 2 * step);
+        r.v3 = *reinterpret_cast<const uint4 *>(p + 3 * step);
+    } else {
+        // rows past the table's end re-read this lane's first row (always in range when
+        // tid < buf_vecs; lanes beyond read row 0) and are never written to LDS
+        const char *p0 = tid < buf_vecs ? p : tb + (tid & 15) * 16;
+        r.v0 = *reinterpret_cast<const uint4 *>(p0);
+        r.v1 = *reinterpret_cast<const uint4 *>(tid + WG < buf_vecs ? p + step : p0);
+        r.v2 = *reinterpret_cast<const uint4 *>(tid + 2 * WG < buf_vecs ? p + 2 * step : p0);
+        r.v3 = *reinterpret_cast<const uint4 *>(tid + 3 * WG < buf_vecs ? p + 3 * step : p0);
+    }
+    return r;
+}
+
+template <bool FULL>
+__device__ __forceinline__ void stash_slice(const SliceRegs &r, uint4 *dst, int tid, int buf_vecs) {
+    if (FULL || tid < buf_vecs) dst[tid] = r.v0;
+    if (FULL || tid + WG < buf_vecs) dst[tid + WG] = r.v1;
+    if (FULL || tid + 2 * WG < buf_vecs) dst[tid + 2 * WG] = r.v2;
+    if (FULL || tid + 3 * WG < buf_vecs) dst[tid + 3 * WG] = r.v3;
+}
+
+template <bool BF16, int NP, bool FULL>
+__global__ __launch_bounds__(WG) void lookup_gather_lds_kernel(LdsGatherArgs a) {
+    constexpr int EPV = BF16 ? 8 : 4;
+    static_assert(MAX_S * SEG_VECS == 4 * WG, "SliceRegs holds four vectors per lane");
+    extern __shared__ uint4 lds[];                // 2 buffers of S * SEG_VECS vectors
+
+    const int xcd = blockIdx.x % XCDS;
+    const int unit = xcd * a.per_xcd + blockIdx.x / XCDS;
+    if (unit >= a.ntiles * a.nslices) return;     // uniform over the workgroup
+    const int slice = unit / a.ntiles;
+    const int tile = unit % a.ntiles;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int grp = lane >> 4;        // token within the wavefront's four
+    const int j = lane & 15;          // 16-byte vector within the row segment
+    const int64_t tok0 = int64_t(tile) * (64 * NP) + wave * 4 + grp;
+
+    float acc[NP][EPV];
+    {
+        float b[EPV];
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) b[e] = 0.f;
+        if (a.bias) {
+            const float *bp = a.bias + (size_t)slice * (SEG_VECS * EPV) + j * EPV;
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) b[e] = bp[e];
+        }
+#pragma unroll
+        for (int p = 0; p < NP; ++p)
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) acc[p][e] = b[e];
+    }
+
+    const int buf_vecs = a.S * SEG_VECS;
+    const char *slice_base = a.tables + (size_t)slice * (SEG_VECS * 16);
+    const size_t table_bytes = (size_t)a.S * a.row_bytes;
+
+    {
+        const SliceRegs first = fetch_slice<FULL>(slice_base, a.row_bytes, tid, buf_vecs);
+        stash_slice<FULL>(first, lds, tid, buf_vecs);
+    }
+    __syncthreads();
+
+    constexpr int NQ = (NP + 3) / 4;     // codes are 8 bits (S <= 256): four passes' codes per register
+    for (int t0 = 0; t0 < a.T; t0 += CHUNK) {
+        // Lane j of a token group holds (code, score) of table t0 + j for each of
+        // its NP tokens.  Addresses are clamped into range and the loads are
+        // unconditional, so that all 2*NP of them are in flight together; what was
+        // loaded from a clamped address is then zeroed.
+        unsigned cd[NQ];
+        float sc[NP];
+        {
+            const int tt = t0 + j;
+            const int ttc = min(tt, a.T - 1);
+            int craw[NP];
+#pragma unroll
+            for (int p = 0; p < NP; ++p) {
+                const int64_t tok = min(tok0 + p * 64, a.B - 1);
+                craw[p] = a.code[tok * a.T + ttc];
+                sc[p] = a.score[tok * a.T + ttc];
+            }
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) cd[q] = 0u;
+#pragma unroll
+            for (int p = 0; p < NP; ++p) {
+                const bool ok = (tok0 + p * 64 < a.B) && (tt < a.T);
+                cd[p / 4] |= unsigned(craw[p] & (a.S - 1)) << (8 * (p % 4));
+                sc[p] = ok ? sc[p] : 0.f;
+            }
+        }
+        // The pairs must have landed before the table loop starts: inside it the
+        // only loads in flight are the next table's slice, which is not waited
+        // for until it is written to LDS at the end of an iteration.
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) asm volatile("" : "+v"(cd[q]));
+#pragma unroll
+        for (int p = 0; p < NP; ++p) asm volatile("" : "+v"(sc[p]));
+
+        const int nt = min(CHUNK, a.T - t0);
+        for (int tt = 0; tt < nt; ++tt) {
+            const int t = t0 + tt;
+            // next table's slice (the last iteration re-reads the last table: harmless)
+            const SliceRegs nxt = fetch_slice<FULL>(slice_base + (size_t)min(t + 1, a.T - 1) * table_bytes,
+                                                    a.row_bytes, tid, buf_vecs);
+            const uint4 *buf = lds + (t & 1) * buf_vecs + j;
+            const int src_lane = ((lane & 48) | tt) << 2;      // byte address of lane (grp*16 + tt)
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+                const unsigned packed = (unsigned)__builtin_amdgcn_ds_bpermute(src_lane, (int)cd[q]);
+#pragma unroll
+                for (int pp = 0; pp < 4; ++pp) {
+                    const int p = 4 * q + pp;
+                    if (p < NP) {
+                        const float w = __int_as_float(__builtin_amdgcn_ds_bpermute(src_lane, __float_as_int(sc[p])));
+                        const unsigned row = (packed >> (8 * pp)) & 0xFFu;
+                        const uint4 r = buf[row * SEG_VECS];
+                        if constexpr (BF16) {
+                            acc[p][0] = fmaf(bf16_lo(r.x), w, acc[p][0]);
+                            acc[p][1] = fmaf(bf16_hi(r.x), w, acc[p][1]);
+                            acc[p][2] = fmaf(bf16_lo(r.y), w, acc[p][2]);
+                            acc[p][3] = fmaf(bf16_hi(r.y), w, acc[p][3]);
+                            acc[p][4] = fmaf(bf16_lo(r.z), w, acc[p][4]);
+                            acc[p][5] = fmaf(bf16_hi(r.z), w, acc[p][5]);
+                            acc[p][6] = fmaf(bf16_lo(r.w), w, acc[p][6]);
+                            acc[p][7] = fmaf(bf16_hi(r.w), w, acc[p][7]);
+                        } else {
+                            acc[p][0] = fmaf(__uint_as_float(r.x), w, acc[p][0]);
+                            acc[p][1] = fmaf(__uint_as_float(r.y), w, acc[p][1]);
+                            acc[p][2] = fmaf(__uint_as_float(r.z), w, acc[p][2]);
+                            acc[p][3] = fmaf(__uint_as_float(r.w), w, acc[p][3]);
+                        }
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);   // bound the loads in flight to one group of four passes
+            }
+            // the other buffer was last read one table ago, before the previous barrier
+            stash_slice<FULL>(nxt, lds + ((t + 1) & 1) * buf_vecs, tid, buf_vecs);
+            __syncthreads();
+        }
+    }
+
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+        const int64_t tok = tok0 + p * 64;
+        if (tok < a.B) {
+            float *o = a.out + tok * a.Do + (size_t)slice * (SEG_VECS * EPV) + j * EPV;
+#pragma unroll
+            for (int q = 0; q < EPV / 4; ++q)
+                *reinterpret_cast<float4 *>(o + 4 * q) =
+                    make_float4(acc[p][4 * q], acc[p][4 * q + 1], acc[p][4 * q + 2], acc[p][4 * q + 3]);
+        }
+    }
+}
+
+template <bool BF16, int NP, bool FULL>
+int launch_lds_full(LdsGatherArgs a, hipStream_t stream) {
+    a.ntiles = (int)((a.B + 64 * NP - 1) / (64 * NP));
+    const int units = a.ntiles * a.nslices;
+    a.per_xcd = (units + XCDS - 1) / XCDS;
+    const size_t lds_bytes = size_t(2) * a.S * SEG_VECS * 16;
+    auto kern = lookup_gather_lds_kernel<BF16, NP, FULL>;
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds_bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        return LFFN_ERR_LAUNCH;
+    }
+    hipLaunchKernelGGL(kern, dim3(a.per_xcd * XCDS), dim3(WG), lds_bytes, stream, a);
+    return lffn_launch_status();
+}
+
+template <bool BF16, int NP>
+int launch_lds(const LdsGatherArgs &a, hipStream_t stream) {
+    return a.S == MAX_S ? launch_lds_full<BF16, NP, true>(a, stream) : launch_lds_full<BF16, NP, false>(a, stream);
+}
+
+// Plan for a shape: 0 = token-major kernel (gather.hip), otherwise NP of the
+// LDS-tiled kernel (64*NP tokens per workgroup).
+//
+// The LDS-tiled form needs the table to fit the buffers (S <= 256), rows that
+// split into whole 256-byte segments, and enough (token tile, slice) units to
+// occupy most of the 256 CUs even at the smallest tile.  Among the NP that are
+// built, the measured time per workgroup per table is close to (7 + NP) * 0.1 us
+// (staging a slice costs as much as seven passes), and workgroups run in
+// ceil(units / 256) rounds, one workgroup per CU.
+template <bool BF16>
+int plan_np(int64_t B, int64_t T, int64_t S, int64_t Do) {
+    const int cols = BF16 ? 128 : 64;
+    if (S > MAX_S || Do % cols != 0 || T < 4) return 0;
+    const int64_t nslices = Do / cols;
+    if (((B + 255) / 256) * nslices < 192) return 0;
+    if (B * nslices > (int64_t(1) << 30)) return 0;
+    constexpr int NPS_F32[] = {16, 13, 8, 4};
+    constexpr int NPS_BF16[] = {8, 4, 4, 4};
+    double best_cost = 1e300;
+    int best = 0;
+    for (int k = 0; k < 4; ++k) {
+        const int np = BF16 ? NPS_BF16[k] : NPS_F32[k];
+        if (S != MAX_S && np > (BF16 ? 4 : 8)) continue;   // the partial-table variants have fewer free registers
+        const int64_t tiles = (B + 64 * np - 1) / (64 * np);
+        const int64_t rounds = (tiles * nslices + 255) / 256;
+        const double cost = double(rounds) * (7.0 + np);
+        if (cost < best_cost) { best_cost = cost; best = np; }
+    }
+    return best;
+}
+
+template <bool BF16>
+int lookup_gather_entry(const int32_t *code, const float *score, const void *tables, const float *bias,
+                        float *out, int64_t B, int64_t T, int64_t S, int64_t Do, void *stream) {
+    LFFN_REQUIRE(B >= 0 && T >= 0 && Do >= 1, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_is_pow2(S) && S <= (1 << 24) && T * S <= 0x7fffffff, LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(Do % 64 == 0 && Do <= (1 << 20) && T <= (1 << 24), LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(B <= (int64_t(1) << 31) - 1, LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(tables && out && ((code && score) || B * T == 0), LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_aligned16(tables) && lffn_aligned16(out) && (!bias || lffn_aligned16(bias)), LFFN_ERR_BAD_ARG);
+    if (B == 0) return LFFN_OK;
+    const int np = plan_np<BF16>(B, T, S, Do);
+    if (np == 0)
+        return lffn_internal_lookup_gather_token_major(code, score, tables, bias, out, B, T, S, Do, BF16, stream);
+    LdsGatherArgs a{};
+    a.code = code; a.score = score; a.tables = static_cast<const char *>(tables); a.bias = bias; a.out = out;
+    a.B = B; a.T = (int)T; a.S = (int)S; a.Do = (int)Do;
+    a.nslices = (int)(Do / (BF16 ? 128 : 64));
+    a.row_bytes = (int)(Do * (BF16 ? 2 : 4));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if constexpr (BF16) {
+        return np == 8 ? launch_lds<true, 8>(a, st) : launch_lds<true, 4>(a, st);
+    } else {
+        switch (np) {
+            case 16: return launch_lds<false, 16>(a, st);
+            case 13: return launch_lds<false, 13>(a, st);
+            case 8: return launch_lds<false, 8>(a, st);
+            default: return launch_lds<false, 4>(a, st);
+        }
+    }
+}
+
+}  // namespace
+
+extern "C" int lffn_lookup_gather_f32(const int32_t *code, const float *score, const float *tables,
+                                      const float *bias, float *out,
+                                      int64_t B, int64_t T, int64_t S, int64_t Do, void *stream) {
+    return lookup_gather_entry<false>(code, score, tables, bias, out, B, T, S, Do, stream);
+}
+
+extern "C" int lffn_lookup_gather_bf16(const int32_t *code, const float *score, const uint16_t *tables,
+                                       const float *bias, float *out,
+                                       int64_t B, int64_t T, int64_t S, int64_t Do, void *stream) {
+    return lookup_gather_entry<true>(code, score, tables, bias, out, B, T, S, Do, stream);
+}
+
+extern "C" int lffn_lookup_gather_plan(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t bf16) {
+    if (B < 0 || T < 0 || Do < 1 || !lffn_is_pow2(S) || Do % 64 != 0) return LFFN_ERR_BAD_ARG;
+    return 64 * (bf16 ? plan_np<true>(B, T, S, Do) : plan_np<false>(B, T, S, Do));
+}

@@ -262,6 +262,44 @@ def test_gather_add_bf16_matches_oracle(B, T, S, Do):
         assert relmax(cabi.lookup_gather(code, w, bits.reshape(T, S, Do), None, bf16=True), want_bf) <= 1e-5
 
 
+# shapes that take the LDS-tiled kernel, with the tokens per workgroup the plan must pick:
+# every tile size that is built (256/512/832/1024 tokens), ragged token counts, table
+# counts that are not multiples of the 16-table chunk, tables smaller than the LDS buffer
+LDS_CASES = [(3000, 20, 256, 1024, False, 256), (16384, 6, 256, 512, False, 512), (16384, 5, 256, 768, False, 832),
+             (16384, 7, 256, 1024, False, 1024), (16301, 33, 256, 768, False, 832), (3001, 17, 64, 1024, False, 256),
+             (16384, 35, 128, 512, False, 512), (16384, 6, 256, 1024, True, 512), (5003, 19, 256, 2048, True, 512),
+             (3000, 18, 32, 2048, True, 256), (16384, 4, 256, 256, False, 256)]
+
+
+@pytest.mark.parametrize("B,T,S,Do,bf16,tokens_per_wg", LDS_CASES)
+def test_lookup_gather_lds_tiled_matches_oracle(B, T, S, Do, bf16, tokens_per_wg):
+    from lookupffn_amd import _lib
+    assert _lib.load().lffn_lookup_gather_plan(B, T, S, Do, int(bf16)) == tokens_per_wg
+    rng = np.random.RandomState(B + T + S + Do)
+    tables, code, idx, w = _rand_gather(rng, B, T, S, Do)
+    bias = (0.001 * rng.randn(Do)).astype(np.float32)
+    flat = tables.reshape(T * S, Do)
+    src = oracle.bf16_round(flat) if bf16 else flat
+    got = cabi.lookup_gather(code, w, src.reshape(T, S, Do), bias, bf16=bf16)
+    assert not np.isnan(got).any()
+    # a random sample of tokens plus the whole ragged tail
+    sub = np.unique(np.concatenate([rng.choice(B, 96, replace=False), np.arange(B - 80, B), np.arange(0, 8)]))
+    w64 = w[sub].astype(np.float64)
+    if bf16:
+        want = oracle.gather_add_bf16(idx[sub], src, w64) + bias
+    else:
+        want = oracle.gather_add(idx[sub], flat.astype(np.float64), w64) + bias
+    assert relmax(got[sub], want) <= 1e-5
+    # the two kernels (LDS-tiled, token-major) agree on every token
+    assert relmax(got, cabi.gather_add(idx, src, w, bf16=bf16).astype(np.float64) + bias) <= 1e-6
+    # codes are masked into their table: bits above log2(S) are ignored
+    dirty = (code + S * rng.randint(0, 5, size=code.shape)).astype(np.int32)
+    assert np.array_equal(cabi.lookup_gather(dirty, w, src.reshape(T, S, Do), bias, bf16=bf16), got)
+    # no bias
+    got_nb = cabi.lookup_gather(code, w, src.reshape(T, S, Do), None, bf16=bf16)
+    assert relmax(got_nb[sub], want - bias) <= 1e-5
+
+
 def test_gather_special_cases():
     rng = np.random.RandomState(30)
     tables, code, idx, w = _rand_gather(rng, 16, 8, 16, 128)
