@@ -47,7 +47,7 @@ WORKLOADS = {
 # HBM bytes per launch of the gather kernel measured with rocprofv3 --pmc
 # (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); the summaries
 # are kept under profiles/.  None until measured for that workload.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {"cfg2": 454936243, "cfg3": 2865333908, "cfg3bf16": 1397976562}
 
 
 def build_layer(wl, device):
