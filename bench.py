@@ -42,6 +42,9 @@ WORKLOADS = {
                  desc="config 3: 16384 tokens, d=1024, 512 tables x 256 x 1024 fp32"),
     "cfg3bf16": dict(B=16384, H=1024, T=512, S=256, Do=1024, bf16=True,
                      desc="config 3: 16384 tokens, d=1024, 512 tables x 256 x 1024 bf16 rows, fp32 accumulate"),
+    # BASELINE.json configs[4]: the backward at the config-2 shape, codes drawn Zipf(1.1)
+    "cfg5": dict(B=16384, H=768, T=128, S=256, Do=768, bf16=False,
+                 desc="config 5: backward at the config-2 shape, codes Zipf(s=1.1) over 256 entries"),
 }
 
 # HBM bytes per launch of the gather kernel measured with rocprofv3 --pmc
@@ -118,6 +121,118 @@ def cpu_baseline(layer, x, wl, budget_s=12.0):
     return out
 
 
+def zipf_codes(B, T, S, gen, s=1.1):
+    """Per (token, table) a rank drawn with p_r ~ r^-s, mapped to a table entry by a
+    fixed seeded permutation per table."""
+    import torch
+    p = 1.0 / torch.arange(1, S + 1, dtype=torch.float64) ** s
+    rank = torch.multinomial(p / p.sum(), B * T, replacement=True, generator=gen).reshape(B, T)
+    perm = torch.stack([torch.randperm(S, generator=gen) for _ in range(T)], dim=0)      # [T, S]
+    return torch.gather(perm.t().contiguous(), 0, rank).to(torch.int32)                  # perm[t][rank[b,t]]
+
+
+def main_backward(args):
+    """Backward of the layer's operators at the config-2 shape: gradient w.r.t. the
+    scores (indexed inner product), the tables (atomic scatter-add into a zeroed
+    buffer), z (closed-form score derivative) and the projection input (the four
+    diagonal x Hadamard stages transposed)."""
+    import numpy as np
+    import torch
+
+    from lookupffn_amd import _lib, ops
+    _lib.load()
+    assert torch.cuda.is_available(), "bench.py needs an MI355X"
+    dev = torch.device("cuda:0")
+    wl = WORKLOADS["cfg5"]
+    B, H, T, S, Do = wl["B"], wl["H"], wl["T"], wl["S"], wl["Do"]
+    layer, x_cpu = build_layer(wl, dev)
+    g = torch.Generator().manual_seed(4321)
+    code_cpu = zipf_codes(B, T, S, g)
+    z_cpu = torch.randn(B, T, 8, generator=g)
+    g_out_cpu = torch.randn(B, Do, generator=g)
+    score_cpu = 1.0 - torch.rand(B, T, generator=g)
+    code, z, g_out, score = code_cpu.to(dev), z_cpu.to(dev), g_out_cpu.to(dev), score_cpu.to(dev)
+    idx = code + torch.arange(T, device=dev, dtype=torch.int32)[None] * S
+    flat = layer.tables.detach().reshape(T * S, Do)
+    p = layer.hash.projection
+    D = p.padded_in_dim
+    diag = p.weight.detach().reshape(1, 4, D)
+    # transpose of x -> FHT(d3*FHT(d2*FHT(d1*FHT(d0*x)))) is g -> d0*FHT(d1*FHT(d2*FHT(d3*FHT(g))))
+    diag_t = torch.stack([torch.ones(D, device=dev), diag[0, 3], diag[0, 2], diag[0, 1]]).reshape(1, 4, D).contiguous()
+    d0 = diag[0, 0].contiguous()
+
+    def step(events=None):
+        g_score = ops.indexed_inner_product(idx, g_out, flat)
+        if events is not None:
+            events[0].record()
+        g_tables = ops.lookup_scatter(code, score, g_out, S)
+        if events is not None:
+            events[1].record()
+        g_z = ops.code_score_bwd(z, g_score).reshape(B, T * 8)
+        g_h = (ops.bh4_diag((p.decay_coeff * g_z).contiguous(), diag_t) * d0 + (1 - p.decay_coeff) * g_z)[:, :H]
+        return g_score, g_tables, g_z, g_h
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(evs[i])
+    torch.cuda.synchronize()
+    sec = time.perf_counter() - t0
+    scatter_ms = sum(a.elapsed_time(b) for a, b in evs) / args.steps
+    scatter_bytes = B * T * Do * 4 * 2 + B * T * 8 + B * Do * 4
+    achieved = scatter_bytes / (scatter_ms * 1e-3) / 1e9
+
+    def timed(fn, n=10):
+        fn(); torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(n):
+            fn()
+        b.record(); torch.cuda.synchronize()
+        return a.elapsed_time(b) / n
+    inner_ms = timed(lambda: ops.indexed_inner_product(idx, g_out, flat))
+    g_score = ops.indexed_inner_product(idx, g_out, flat)
+    bwd_score_ms = timed(lambda: ops.code_score_bwd(z, g_score))
+
+    res = {
+        "metric": "LookupFFN bwd tokens/s + scatter-add GB/s as % of HBM peak, RoBERTa-base shape, Zipf(1.1) codes",
+        "value": B * args.steps / sec, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": sec / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic (seeded; codes Zipf(1.1) through a seeded permutation per table)",
+        "config": {"workload": wl["desc"], "tokens": B, "tables": T, "table_size": S, "d_out": Do,
+                   "step": "inner product (grad score) + scatter-add (grad tables) + score "
+                           "derivative + transposed BH4(block 1)x4"},
+        "roofline": {"bound": "hbm", "kernel": "lookup_scatter", "achieved": achieved,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes": scatter_bytes, "avg_kernel_ms": scatter_ms},
+        "stages_ms": {"indexed_inner_product": inner_ms, "scatter_add": scatter_ms, "code_score_bwd": bwd_score_ms},
+    }
+    if not args.no_cpu_baseline:
+        import oracle
+        n = 1024
+        npf = lambda t: t.detach().float().cpu().numpy()
+        idx_n, g_n, w_n, z_n = npf(idx[:n]).astype(np.int32), npf(g_out[:n]), npf(score[:n]), npf(z[:n])
+        flat_n = npf(flat)
+        reps, tt = 0, 0.0
+        while reps < 2 or (tt < 10.0 and reps < 1000):
+            t0 = time.perf_counter()
+            gs = oracle.indexed_inner_product(idx_n, g_n, flat_n)
+            oracle.scatter_add(idx_n, g_n, w_n, T * S)
+            gz = oracle.code_score_bwd(z_n, gs)
+            oracle.fht(np.ascontiguousarray(gz.reshape(n, T * 8)))
+            tt += time.perf_counter() - t0
+            reps += 1
+        res["cpu_baseline"] = {"value": n * reps / tt, "unit": "tokens/s", "cores": oracle.num_threads(), "kind": "port",
+                               "sample": f"first {n} tokens, {reps} passes of the C oracle's inner product, scatter-add "
+                                         f"(serial by definition), score derivative and one FHT, {tt:.1f} s"}
+    else:
+        res["cpu_baseline"] = None
+    print(json.dumps(res))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -133,6 +248,9 @@ def main():
         print("bench.py: this build runs the LookupFFN hot path on ONE GPU only "
               "(no multi-GPU form exists); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+
+    if args.workload == "cfg5":
+        return main_backward(args)
 
     import torch
 

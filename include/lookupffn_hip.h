@@ -175,6 +175,20 @@ int lffn_indexed_inner_product_f32(const int32_t *idx, const float *g, const flo
 int lffn_scatter_add_f32(const int32_t *idx, const float *g, const float *w, float *out,
                          int64_t B, int64_t I, int64_t out_size, int64_t Dv, void *stream);
 
+/*
+ * The scatter-add as the layer's backward issues it: table-local codes, the
+ * gradient of the whole [T, S, Do] table array in one call,
+ *   grad_tables[t, s, :] (+)= sum_{b : (code[b,t] & (S-1)) == s} score[b,t] * g[b,:]
+ * code: [B, T] int32; score: [B, T]; g: [B, Do]; grad_tables: [T, S, Do].
+ * accumulate == 0: grad_tables is overwritten (it needs no zero-fill); otherwise
+ * added to.  For S <= 256 the sums are formed in LDS (no global atomics); the
+ * order of additions is still free, as with the reference's atomics.
+ * Replaces WeightedVectorGatherAdd.backward's weighted_vector_scatter_add call
+ * (PL/gather/cuda/kernel.py:200) together with the index offset of PL/lookup.py:126.
+ */
+int lffn_lookup_scatter_f32(const int32_t *code, const float *score, const float *g, float *grad_tables,
+                            int64_t B, int64_t T, int64_t S, int64_t Do, int32_t accumulate, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -393,6 +393,16 @@ int lffn_internal_lookup_gather_token_major(const int32_t *code, const float *sc
                 : gather_entry<false>(code, tables, score, bias, out, B, T, rows, Do, S, stream);
 }
 
+// Atomic scatter-add on table-local codes (row = code & (S-1) + t*S), into a buffer
+// the caller has zeroed or wants accumulated into: the fallback of lookup_scatter.hip.
+int lffn_internal_lookup_scatter_atomic(const int32_t *code, const float *score, const float *g, float *out,
+                                        int64_t B, int64_t T, int64_t S, int64_t Do, void *stream) {
+    GatherArgs a{};
+    a.idx = code; a.src = nullptr; a.w = score; a.g = g; a.bias = nullptr; a.out = out;
+    a.B = B; a.I = (int)T; a.source_size = T * S; a.Dv = (int)Do; a.S = (int)S;
+    return launch<false, Op::Scatter>(a, static_cast<hipStream_t>(stream));
+}
+
 extern "C" int lffn_indexed_inner_product_f32(const int32_t *idx, const float *g, const float *src, float *out,
                                               int64_t B, int64_t I, int64_t source_size, int64_t Dv, void *stream) {
     int rc = check_common(idx, B, I, source_size, Dv);

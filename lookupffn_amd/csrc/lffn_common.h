@@ -28,6 +28,11 @@ int lffn_internal_lookup_gather_token_major(const int32_t *code, const float *sc
                                             const float *bias, float *out, int64_t B, int64_t T, int64_t S,
                                             int64_t Do, bool bf16, void *stream);
 
+// gather.hip: atomic scatter-add on table-local codes (not exported)
+__attribute__((visibility("hidden")))
+int lffn_internal_lookup_scatter_atomic(const int32_t *code, const float *score, const float *g, float *out,
+                                        int64_t B, int64_t T, int64_t S, int64_t Do, void *stream);
+
 static inline int lffn_launch_status() {
     return hipGetLastError() == hipSuccess ? LFFN_OK : LFFN_ERR_LAUNCH;
 }

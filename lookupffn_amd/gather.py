@@ -150,8 +150,7 @@ class LookupGather(Function):
         idx = (code & (S - 1)) + torch.arange(T, device=code.device, dtype=code.dtype)[None] * S
         flat = tables.reshape(T * S, Do)
         grad_score = ops.indexed_inner_product(idx, grad_outputs, flat) if ctx.needs_input_grad[1] else None
-        grad_tables = (ops.scatter_add(idx, grad_outputs, score, T * S).reshape(T, S, Do)
-                       if ctx.needs_input_grad[2] else None)
+        grad_tables = ops.lookup_scatter(code, score, grad_outputs, S) if ctx.needs_input_grad[2] else None
         grad_bias = grad_outputs.sum(dim=0) if (ctx.has_bias and ctx.needs_input_grad[3]) else None
         return None, grad_score, grad_tables, grad_bias
 

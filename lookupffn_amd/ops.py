@@ -305,6 +305,34 @@ def _(indexes, source, weights, output_size):
     return source.new_empty(output_size, source.shape[1])
 
 
+_L.define("lookup_scatter(Tensor code, Tensor score, Tensor g, int S) -> Tensor")
+
+
+def _lookup_scatter_impl(code, score, g, S):
+    _lib.require_gpu(code, score, g)
+    assert g.dim() == 2 and g.dtype == torch.float32 and g.is_contiguous()
+    assert score.dtype == torch.float32 and score.is_contiguous()
+    assert tuple(score.shape) == tuple(code.shape)
+    B, T = code.shape
+    Do = g.shape[1]
+    assert g.shape[0] == B and _is_pow2(S)
+    _check_gather_args(code, max(T * S, 1), Do)
+    out = torch.empty(T, S, Do, dtype=torch.float32, device=g.device)     # fully overwritten by the kernel
+    with _dev_guard(g):
+        rc = _lib.load().lffn_lookup_scatter_f32(_lib.ptr(code), _lib.ptr(score), _lib.ptr(g), _lib.ptr(out),
+                                                 B, T, S, Do, 0, _lib.stream_of(g))
+    _lib.check(rc, f"lffn_lookup_scatter_f32(B={B}, T={T}, S={S}, Do={Do})")
+    return out
+
+
+_L.impl("lookup_scatter", _lookup_scatter_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::lookup_scatter")
+def _(code, score, g, S):
+    return g.new_empty(code.shape[1], S, g.shape[1])
+
+
 fht = torch.ops.lookupffn.fht
 bh4_diag = torch.ops.lookupffn.bh4_diag
 project_hash = torch.ops.lookupffn.project_hash
@@ -314,3 +342,4 @@ gather_add = torch.ops.lookupffn.gather_add
 lookup_gather = torch.ops.lookupffn.lookup_gather
 indexed_inner_product = torch.ops.lookupffn.indexed_inner_product
 scatter_add = torch.ops.lookupffn.scatter_add
+lookup_scatter = torch.ops.lookupffn.lookup_scatter

@@ -120,3 +120,15 @@ def scatter_add(idx, g, w, out_size, init=None):
     out = torch.zeros(out_size, Dv, dtype=torch.float32, device=DEV) if init is None else dev(init)
     _call("lffn_scatter_add_f32", p(idd), p(gd), p(wd), p(out), B, I, out_size, Dv)
     return host(out)
+
+
+def lookup_scatter(code, score, g, S, accumulate=False, init=None):
+    cd, sd, gd = dev(code), dev(score), dev(g)
+    B, T = code.shape
+    Do = g.shape[1]
+    if init is None:
+        out = torch.full((T, S, Do), float("nan"), dtype=torch.float32, device=DEV)   # must be fully overwritten
+    else:
+        out = dev(init)
+    _call("lffn_lookup_scatter_f32", p(cd), p(sd), p(gd), p(out), B, T, S, Do, 1 if accumulate else 0)
+    return host(out)

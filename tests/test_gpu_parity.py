@@ -359,6 +359,57 @@ def test_backward_matches_oracle(B, T, S, Do):
     assert relmax(cabi.scatter_add(idx, g, w, T * S, init=init), want_t + init) <= 1e-5
 
 
+# (B, T, S, Do): odd table counts, tables smaller than the LDS
+# slice, ragged token counts around the 64-token batches and 1024-token strides, and a
+# table size (512) that takes the zero-fill + global-atomics path
+SCATTER_CASES = [(256, 32, 256, 256), (1, 2, 4, 64), (63, 3, 16, 128), (65, 5, 256, 192), (1025, 7, 8, 64),
+                 (2100, 6, 256, 128), (300, 1, 2, 64), (500, 4, 512, 128), (0, 4, 16, 64)]
+
+
+@pytest.mark.parametrize("B,T,S,Do", SCATTER_CASES)
+def test_lookup_scatter_matches_oracle(B, T, S, Do):
+    rng = np.random.RandomState(B + T + S + Do)
+    tables, code, idx, w = _rand_gather(rng, B, T, S, Do)
+    g = rng.randn(B, Do).astype(np.float32)
+    want = oracle.scatter_add(idx, g.astype(np.float64), w.astype(np.float64), T * S).reshape(T, S, Do)
+    got = cabi.lookup_scatter(code, w, g, S)
+    assert not np.isnan(got).any()                      # every row written, touched or not
+    assert relmax(got, want) <= 1e-5 if B else np.array_equal(got, np.zeros_like(got))
+    # accumulate into an existing buffer
+    init = rng.randn(T, S, Do).astype(np.float32)
+    assert relmax(cabi.lookup_scatter(code, w, g, S, accumulate=True, init=init), want + init) <= 1e-5
+    # codes are masked into their table
+    if B:
+        dirty = (code + S * rng.randint(0, 4, size=code.shape)).astype(np.int32)
+        assert relmax(cabi.lookup_scatter(dirty, w, g, S), want) <= 1e-5
+
+
+def test_lookup_scatter_full_size_zipf_properties():
+    # BASELINE config 5: config-2 shape, codes Zipf(1.1) over 256 entries
+    rng = np.random.RandomState(41)
+    B, T, S, Do = 16384, 128, 256, 768
+    p = 1.0 / np.arange(1, S + 1) ** 1.1
+    p /= p.sum()
+    code = rng.choice(S, size=(B, T), p=p).astype(np.int32)
+    w = (1.0 - rng.rand(B, T)).astype(np.float32)
+    g = rng.randn(B, Do).astype(np.float32)
+    got = cabi.lookup_scatter(code, w, g, S)
+    # column sums: sum_s grad[t,s,:] = sum_b w[b,t] g[b,:]
+    want_sum = w.astype(np.float64).T @ g.astype(np.float64)
+    assert relmax(got.astype(np.float64).sum(1), want_sum) <= 1e-5
+    # a few tables in full against the oracle (the hottest row takes ~18 % of the tokens)
+    for t in (0, 77, 127):
+        idx_t = code[:, t:t + 1]
+        want_t = oracle.scatter_add(idx_t, g.astype(np.float64), w[:, t:t + 1].astype(np.float64), S)
+        assert relmax(got[t], want_t) <= 1e-5
+    # duality with the forward: <G(w), g> = <grad_tables, tables>
+    tables = (0.02 * rng.randn(T, S, Do)).astype(np.float32)
+    fwd = cabi.lookup_gather(code, w, tables, None)
+    lhs = float((fwd.astype(np.float64) * g).sum())
+    rhs = float((got.astype(np.float64) * tables).sum())
+    assert abs(lhs - rhs) <= 1e-5 * max(abs(lhs), 1.0) * 10
+
+
 def test_scatter_duplicates_zipf():
     # heavy duplication of rows (BASELINE config 5 draws codes Zipf(1.1))
     rng = np.random.RandomState(40)
