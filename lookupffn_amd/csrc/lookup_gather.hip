@@ -14,13 +14,15 @@
 // workgroup copies that table's slice (S rows x 256 bytes, 64 KiB for S = 256)
 // into LDS once and all of its tokens read their rows from there: 16 lanes read
 // 256 contiguous bytes, one conflict-free ds_read_b128.  The slices are
-// double-buffered: the global loads of table t+1 are issued before the LDS reads
-// of table t and land in the other buffer, one barrier per table.
+// double-buffered and copied global -> LDS directly (global_load_lds_dwordx4, no
+// registers in between): the copy of table t+1 is issued before the LDS reads of
+// table t and lands in the other buffer, one barrier per table.
 //
 // So each table slice is fetched once per 64*NP tokens instead of once per
 // token, and the per-token row reads are LDS reads.  The (code, score) pairs are
-// read 16 tables at a time, one table per lane of the 16-lane token group, and
-// handed to the group's lanes with ds_bpermute when their table comes up.
+// read 16 tables at a time, one table per lane of the 16-lane token group (four
+// 8-bit codes packed per register), and handed to the group's lanes with
+// ds_bpermute when their table comes up.
 //
 // blockIdx -> (slice, token tile) is XCD-aware: workgroups are dealt round-robin
 // to the 8 XCDs, so block b runs on XCD b % 8; units are numbered so that the
@@ -48,48 +50,38 @@ struct LdsGatherArgs {
     int row_bytes;         // Do * element size
 };
 
-// One lane's share of a table slice: four 16-byte vectors, q = tid + 1024*i,
-// row q/16, vector q%16 of the 256-byte row segment.  Plain members (not an
-// array) so that they stay in registers across the table loop.
-struct SliceRegs {
-    uint4 v0, v1, v2, v3;
-};
-
-// FULL: the table has exactly MAX_S rows, so every lane moves all four vectors.
-template <bool FULL>
-__device__ __forceinline__ SliceRegs fetch_slice(const char *tb, int row_bytes, int tid, int buf_vecs) {
-    SliceRegs r;
-    const char *p = tb + (size_t)(tid >> 4) * row_bytes + (tid & 15) * 16;
-    const size_t step = (size_t)(WG / SEG_VECS) * row_bytes;   // 64 rows further down
-    if constexpr (FULL) {
-        r.v0 = *reinterpret_cast<const uint4 *>(p);
-        r.v1 = *reinterpret_cast<const uint4 *>(p + step);
-        r.v2 = *reinterpret_cast<const uint4 *>(p + 2 * step);
-        r.v3 = *reinterpret_cast<const uint4 *>(p + 3 * step);
-    } else {
-        // rows past the table's end re-read this lane's first row (always in range when
-        // tid < buf_vecs; lanes beyond read row 0) and are never written to LDS
-        const char *p0 = tid < buf_vecs ? p : tb + (tid & 15) * 16;
-        r.v0 = *reinterpret_cast<const uint4 *>(p0);
-        r.v1 = *reinterpret_cast<const uint4 *>(tid + WG < buf_vecs ? p + step : p0);
-        r.v2 = *reinterpret_cast<const uint4 *>(tid + 2 * WG < buf_vecs ? p + 2 * step : p0);
-        r.v3 = *reinterpret_cast<const uint4 *>(tid + 3 * WG < buf_vecs ? p + 3 * step : p0);
-    }
-    return r;
+// Copy this lane's four vectors of a table slice straight from global memory into
+// the LDS buffer `dst` (global_load_lds_dwordx4: lane i of a wavefront writes
+// 16 bytes at the wavefront-uniform LDS address in M0 + 16*i, so a wavefront fills
+// the 1 KiB of vectors q = wave*64 + [0,64) + 1024*i).  Nothing passes through
+// registers.  Issued as inline assembly on purpose: the compiler would otherwise
+// wait for the copy before the next LDS read of ANY address (it cannot tell the two
+// buffers apart), which would serialise the copy with the pass loop.  The caller
+// waits with vmcnt(0) before the barrier that publishes the buffer.
+__device__ __forceinline__ void lds_dma16(const char *gptr, uint32_t lds_byte_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(gptr), "s"(lds_byte_addr)
+                 : "memory");
 }
 
 template <bool FULL>
-__device__ __forceinline__ void stash_slice(const SliceRegs &r, uint4 *dst, int tid, int buf_vecs) {
-    if (FULL || tid < buf_vecs) dst[tid] = r.v0;
-    if (FULL || tid + WG < buf_vecs) dst[tid + WG] = r.v1;
-    if (FULL || tid + 2 * WG < buf_vecs) dst[tid + 2 * WG] = r.v2;
-    if (FULL || tid + 3 * WG < buf_vecs) dst[tid + 3 * WG] = r.v3;
+__device__ __forceinline__ void copy_slice_to_lds(const char *tb, int row_bytes, int tid, int buf_vecs, uint4 *dst) {
+    const char *p = tb + (size_t)(tid >> 4) * row_bytes + (tid & 15) * 16;
+    const size_t step = (size_t)(WG / SEG_VECS) * row_bytes;   // 64 rows further down
+    // LDS byte address of this wavefront's first vector in `dst`, made scalar
+    const uint32_t wbase = __builtin_amdgcn_readfirstlane(
+        (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint4 *)(dst + (tid & ~63)));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        if (FULL || tid + i * WG < buf_vecs) lds_dma16(p + i * step, wbase + i * (WG * 16));
+    }
 }
 
 template <bool BF16, int NP, bool FULL>
 __global__ __launch_bounds__(WG) void lookup_gather_lds_kernel(LdsGatherArgs a) {
     constexpr int EPV = BF16 ? 8 : 4;
-    static_assert(MAX_S * SEG_VECS == 4 * WG, "SliceRegs holds four vectors per lane");
+    static_assert(MAX_S * SEG_VECS == 4 * WG, "a lane copies four vectors of a slice");
     extern __shared__ uint4 lds[];                // 2 buffers of S * SEG_VECS vectors
 
     const int xcd = blockIdx.x % XCDS;
@@ -125,10 +117,8 @@ __global__ __launch_bounds__(WG) void lookup_gather_lds_kernel(LdsGatherArgs a) 
     const char *slice_base = a.tables + (size_t)slice * (SEG_VECS * 16);
     const size_t table_bytes = (size_t)a.S * a.row_bytes;
 
-    {
-        const SliceRegs first = fetch_slice<FULL>(slice_base, a.row_bytes, tid, buf_vecs);
-        stash_slice<FULL>(first, lds, tid, buf_vecs);
-    }
+    copy_slice_to_lds<FULL>(slice_base, a.row_bytes, tid, buf_vecs, lds);
+    __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0): this lane's copies have landed in LDS
     __syncthreads();
 
     constexpr int NQ = (NP + 3) / 4;     // codes are 8 bits (S <= 256): four passes' codes per register
@@ -169,42 +159,58 @@ __global__ __launch_bounds__(WG) void lookup_gather_lds_kernel(LdsGatherArgs a) 
         const int nt = min(CHUNK, a.T - t0);
         for (int tt = 0; tt < nt; ++tt) {
             const int t = t0 + tt;
-            // next table's slice (the last iteration re-reads the last table: harmless)
-            const SliceRegs nxt = fetch_slice<FULL>(slice_base + (size_t)min(t + 1, a.T - 1) * table_bytes,
-                                                    a.row_bytes, tid, buf_vecs);
+            // next table's slice goes straight into the other buffer, which was last read
+            // one table ago, before the previous barrier (the last iteration re-copies
+            // the last table: harmless)
+            copy_slice_to_lds<FULL>(slice_base + (size_t)min(t + 1, a.T - 1) * table_bytes, a.row_bytes, tid,
+                                    buf_vecs, lds + ((t + 1) & 1) * buf_vecs);
             const uint4 *buf = lds + (t & 1) * buf_vecs + j;
             const int src_lane = ((lane & 48) | tt) << 2;      // byte address of lane (grp*16 + tt)
+            // All code broadcasts first, then the passes in groups of at most GRP: a
+            // group's score broadcasts and row reads are issued together (GRP rows in
+            // flight per lane), then its fmas.  The scheduling barriers keep the
+            // compiler from merging groups, which would not fit the register file.
+            unsigned packed[NQ];
 #pragma unroll
-            for (int q = 0; q < NQ; ++q) {
-                const unsigned packed = (unsigned)__builtin_amdgcn_ds_bpermute(src_lane, (int)cd[q]);
+            for (int q = 0; q < NQ; ++q) packed[q] = (unsigned)__builtin_amdgcn_ds_bpermute(src_lane, (int)cd[q]);
+            constexpr int GRP = BF16 ? 4 : (NP >= 16 ? 4 : (NP > 8 ? 5 : NP));
 #pragma unroll
-                for (int pp = 0; pp < 4; ++pp) {
-                    const int p = 4 * q + pp;
+            for (int g0 = 0; g0 < NP; g0 += GRP) {
+                float w[GRP];
+                uint4 r[GRP];
+#pragma unroll
+                for (int i = 0; i < GRP; ++i) {
+                    const int p = g0 + i;
                     if (p < NP) {
-                        const float w = __int_as_float(__builtin_amdgcn_ds_bpermute(src_lane, __float_as_int(sc[p])));
-                        const unsigned row = (packed >> (8 * pp)) & 0xFFu;
-                        const uint4 r = buf[row * SEG_VECS];
+                        w[i] = __int_as_float(__builtin_amdgcn_ds_bpermute(src_lane, __float_as_int(sc[p])));
+                        const unsigned row = (packed[p / 4] >> (8 * (p % 4))) & 0xFFu;
+                        r[i] = buf[row * SEG_VECS];
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < GRP; ++i) {
+                    const int p = g0 + i;
+                    if (p < NP) {
                         if constexpr (BF16) {
-                            acc[p][0] = fmaf(bf16_lo(r.x), w, acc[p][0]);
-                            acc[p][1] = fmaf(bf16_hi(r.x), w, acc[p][1]);
-                            acc[p][2] = fmaf(bf16_lo(r.y), w, acc[p][2]);
-                            acc[p][3] = fmaf(bf16_hi(r.y), w, acc[p][3]);
-                            acc[p][4] = fmaf(bf16_lo(r.z), w, acc[p][4]);
-                            acc[p][5] = fmaf(bf16_hi(r.z), w, acc[p][5]);
-                            acc[p][6] = fmaf(bf16_lo(r.w), w, acc[p][6]);
-                            acc[p][7] = fmaf(bf16_hi(r.w), w, acc[p][7]);
+                            acc[p][0] = fmaf(bf16_lo(r[i].x), w[i], acc[p][0]);
+                            acc[p][1] = fmaf(bf16_hi(r[i].x), w[i], acc[p][1]);
+                            acc[p][2] = fmaf(bf16_lo(r[i].y), w[i], acc[p][2]);
+                            acc[p][3] = fmaf(bf16_hi(r[i].y), w[i], acc[p][3]);
+                            acc[p][4] = fmaf(bf16_lo(r[i].z), w[i], acc[p][4]);
+                            acc[p][5] = fmaf(bf16_hi(r[i].z), w[i], acc[p][5]);
+                            acc[p][6] = fmaf(bf16_lo(r[i].w), w[i], acc[p][6]);
+                            acc[p][7] = fmaf(bf16_hi(r[i].w), w[i], acc[p][7]);
                         } else {
-                            acc[p][0] = fmaf(__uint_as_float(r.x), w, acc[p][0]);
-                            acc[p][1] = fmaf(__uint_as_float(r.y), w, acc[p][1]);
-                            acc[p][2] = fmaf(__uint_as_float(r.z), w, acc[p][2]);
-                            acc[p][3] = fmaf(__uint_as_float(r.w), w, acc[p][3]);
+                            acc[p][0] = fmaf(__uint_as_float(r[i].x), w[i], acc[p][0]);
+                            acc[p][1] = fmaf(__uint_as_float(r[i].y), w[i], acc[p][1]);
+                            acc[p][2] = fmaf(__uint_as_float(r[i].z), w[i], acc[p][2]);
+                            acc[p][3] = fmaf(__uint_as_float(r[i].w), w[i], acc[p][3]);
                         }
                     }
                 }
-                __builtin_amdgcn_sched_barrier(0);   // bound the loads in flight to one group of four passes
+                __builtin_amdgcn_sched_barrier(0);
             }
-            // the other buffer was last read one table ago, before the previous barrier
-            stash_slice<FULL>(nxt, lds + ((t + 1) & 1) * buf_vecs, tid, buf_vecs);
+            __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0): the copies issued above have landed
             __syncthreads();
         }
     }
