@@ -87,6 +87,21 @@ int lffn_project_hash_f32(const float *x, const float *diag, const float *proj_b
                           int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
                           float decay, float residual, void *stream);
 
+/*
+ * lffn_project_hash_f32 with the layer's LayerNorm (PL/lookup.py:84,99) applied to
+ * each row of x on load: h = (x - mean) / sqrt(var + eps) * ln_weight + ln_bias over
+ * the H valid columns (biased variance), then exactly as above on h.
+ * ln_weight, ln_bias: [H].  Replaces nn.LayerNorm + BH4._forward + Hashing.forward +
+ * compute_code_score_torch (PL/lookup.py:29-39,64-77,99) for block size 1, 8-bit codes.
+ * The LayerNorm sums are formed in a different order than torch's kernel, so h (and
+ * with it z) agrees with torch to rounding, not bit for bit.
+ */
+int lffn_ln_project_hash_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
+                             const float *diag, const float *proj_bias,
+                             float *z_out, int32_t *codes, float *scores,
+                             int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
+                             float decay, float residual, void *stream);
+
 /* ---------------------------------------------------------------- code + score */
 
 /*

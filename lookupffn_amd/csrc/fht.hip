@@ -94,6 +94,9 @@ __device__ __forceinline__ void fht_rows(float (&v)[FhtCfg<LOGD>::NJ][4], int lr
 struct ProjectArgs {
     const float *x;       // [B, H]
     const float *diag;    // [R, J, D] or null (no scale)
+    const float *ln_w;    // [H] LayerNorm weight, or null: no LayerNorm
+    const float *ln_b;    // [H] LayerNorm bias (with ln_w)
+    float ln_eps;
     const float *pbias;   // [out_cols] or null
     float *out;           // [B, out_stride] or null
     int32_t *codes;       // [B, T] (HASH only)
@@ -147,6 +150,33 @@ __global__ __launch_bounds__(256) void project_kernel(ProjectArgs a) {
             }
         }
         orig[j][0] = t.x; orig[j][1] = t.y; orig[j][2] = t.z; orig[j][3] = t.w;
+    }
+
+    if (a.ln_w) {
+        // LayerNorm over the H valid columns (biased variance, two passes, eps inside the
+        // square root: torch.nn.LayerNorm, PL/lookup.py:84,99); padding columns stay zero.
+        float s1 = 0.f;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) s1 += orig[j][c];          // padding contributes 0
+        const float mean = lane_group_sum<LPR>(s1) / float(a.H);
+        float s2 = 0.f;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const float dlt = (256 * j + 4 * lr + c < a.H) ? orig[j][c] - mean : 0.f;
+                s2 += dlt * dlt;
+            }
+        const float rstd = 1.0f / sqrtf(lane_group_sum<LPR>(s2) / float(a.H) + a.ln_eps);
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int e = 256 * j + 4 * lr + c;
+                if (e < a.H) orig[j][c] = (orig[j][c] - mean) * rstd * a.ln_w[e] + a.ln_b[e];
+            }
     }
 
     for (int r = 0; r < a.R; ++r) {
@@ -281,10 +311,35 @@ extern "C" int lffn_bh4_diag_f32(const float *x, const float *diag, float *out,
     return launch_project<false>(a, lffn_log2(D), static_cast<hipStream_t>(stream));
 }
 
+static int project_hash_impl(const float *x, const float *ln_w, const float *ln_b, float ln_eps,
+                             const float *diag, const float *proj_bias,
+                             float *z_out, int32_t *codes, float *scores,
+                             int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
+                             float decay, float residual, void *stream);
+
+extern "C" int lffn_ln_project_hash_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
+                                        const float *diag, const float *proj_bias,
+                                        float *z_out, int32_t *codes, float *scores,
+                                        int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
+                                        float decay, float residual, void *stream) {
+    LFFN_REQUIRE(ln_weight && ln_bias && ln_eps >= 0.f, LFFN_ERR_BAD_ARG);
+    return project_hash_impl(x, ln_weight, ln_bias, ln_eps, diag, proj_bias, z_out, codes, scores,
+                             B, H, D, R, J, T, decay, residual, stream);
+}
+
 extern "C" int lffn_project_hash_f32(const float *x, const float *diag, const float *proj_bias,
                                      float *z_out, int32_t *codes, float *scores,
                                      int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
                                      float decay, float residual, void *stream) {
+    return project_hash_impl(x, nullptr, nullptr, 0.f, diag, proj_bias, z_out, codes, scores,
+                             B, H, D, R, J, T, decay, residual, stream);
+}
+
+static int project_hash_impl(const float *x, const float *ln_w, const float *ln_b, float ln_eps,
+                             const float *diag, const float *proj_bias,
+                             float *z_out, int32_t *codes, float *scores,
+                             int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
+                             float decay, float residual, void *stream) {
     LFFN_REQUIRE(x && diag && codes && scores, LFFN_ERR_BAD_ARG);
     int rc = check_dims(B, H, D, R, J);
     if (rc != LFFN_OK) return rc;
@@ -295,6 +350,7 @@ extern "C" int lffn_project_hash_f32(const float *x, const float *diag, const fl
                  LFFN_ERR_BAD_ARG);
     ProjectArgs a{};
     a.x = x; a.diag = diag; a.pbias = proj_bias; a.out = z_out; a.codes = codes; a.scores = scores;
+    a.ln_w = ln_w; a.ln_b = ln_b; a.ln_eps = ln_eps;
     a.B = B; a.H = (int)H; a.R = (int)R; a.J = (int)J;
     a.out_stride = (int)(T * 8); a.out_cols = (int)(T * 8); a.T = (int)T;
     a.decay = decay; a.residual = residual; a.mix = 1;

@@ -90,12 +90,18 @@ class Hashing(nn.Module):
                 and p.padded_in_dim <= 1024 and p.padded_in_dim >= 8
                 and x.dtype == torch.float32 and x.is_cuda and not needs_grad)
 
-    def forward_fused(self, x):
+    def forward_fused(self, x, layer_norm=None):
+        """One kernel: (LayerNorm ->) diagonal BH4 -> mix -> bias -> code + score."""
         p = self.projection
-        diag = p.weight.reshape(p.num_repeat, p.weight.shape[1], p.padded_in_dim)
-        code, score, _ = ops.project_hash(
-            x.contiguous(), diag.contiguous(), p.bias, self.num_table,
-            float(p.decay_coeff), float(1 - p.decay_coeff), False)
+        diag = p.weight.reshape(p.num_repeat, p.weight.shape[1], p.padded_in_dim).contiguous()
+        if layer_norm is not None:
+            code, score, _ = ops.ln_project_hash(
+                x.contiguous(), layer_norm.weight, layer_norm.bias, float(layer_norm.eps), diag, p.bias,
+                self.num_table, float(p.decay_coeff), float(1 - p.decay_coeff), False)
+        else:
+            code, score, _ = ops.project_hash(
+                x.contiguous(), diag, p.bias, self.num_table,
+                float(p.decay_coeff), float(1 - p.decay_coeff), False)
         return code, score
 
     def forward(self, x):
@@ -129,8 +135,15 @@ class LookupFFN(nn.Module):
                 f"table_size={self.table_size}, output_size={self.output_size}")
 
     def _forward(self, hidden_states):
-        hidden_states = self.LayerNorm(hidden_states)
-        code, score = self.hash(hidden_states)
+        ln = self.LayerNorm
+        if (self.hash.can_fuse(hidden_states) and ln.elementwise_affine and ln.weight is not None
+                and ln.bias is not None and ln.weight.dtype == torch.float32
+                and not (torch.is_grad_enabled() and (ln.weight.requires_grad or ln.bias.requires_grad))):
+            # inference: LayerNorm runs inside the projection kernel
+            code, score = self.hash.forward_fused(hidden_states, layer_norm=ln)
+        else:
+            hidden_states = ln(hidden_states)
+            code, score = self.hash(hidden_states)
         if self.output_size % 64 == 0 and self.tables.dtype in (torch.float32, torch.bfloat16):
             # table-local codes, offset and bias folded into the gather kernel
             return lookup_gather(code, score.float(), self.tables, self.bias.float())

@@ -115,6 +115,43 @@ def _(x, diag, bias, T, decay, residual, keep_z):
             x.new_empty((B, T * 8) if keep_z else (0,)))
 
 
+_L.define("ln_project_hash(Tensor x, Tensor ln_weight, Tensor ln_bias, float eps, Tensor diag, Tensor? bias, "
+          "int T, float decay, float residual, bool keep_z) -> (Tensor, Tensor, Tensor)")
+
+
+def _ln_project_hash_impl(x, ln_weight, ln_bias, eps, diag, bias, T, decay, residual, keep_z):
+    _lib.require_gpu(x, ln_weight, ln_bias, diag, bias)
+    assert x.dim() == 2 and diag.dim() == 3
+    assert x.dtype == torch.float32 and diag.dtype == torch.float32
+    assert ln_weight.dtype == torch.float32 and ln_bias.dtype == torch.float32
+    assert x.is_contiguous() and diag.is_contiguous() and ln_weight.is_contiguous() and ln_bias.is_contiguous()
+    B, H = x.shape
+    R, J, D = diag.shape
+    assert H <= D and T * 8 <= R * D and ln_weight.numel() == H and ln_bias.numel() == H
+    if bias is not None:
+        assert bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == T * 8
+    codes = torch.empty(B, T, dtype=torch.int32, device=x.device)
+    scores = torch.empty(B, T, dtype=torch.float32, device=x.device)
+    z = torch.empty((B, T * 8) if keep_z else (0,), dtype=torch.float32, device=x.device)
+    with _dev_guard(x):
+        rc = _lib.load().lffn_ln_project_hash_f32(
+            _lib.ptr(x), _lib.ptr(ln_weight), _lib.ptr(ln_bias), eps, _lib.ptr(diag), _lib.ptr(bias),
+            _lib.ptr(z) if keep_z else None, _lib.ptr(codes), _lib.ptr(scores),
+            B, H, D, R, J, T, decay, residual, _lib.stream_of(x))
+    _lib.check(rc, f"lffn_ln_project_hash_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T})")
+    return codes, scores, z
+
+
+_L.impl("ln_project_hash", _ln_project_hash_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::ln_project_hash")
+def _(x, ln_weight, ln_bias, eps, diag, bias, T, decay, residual, keep_z):
+    B = x.shape[0]
+    return (x.new_empty(B, T, dtype=torch.int32), x.new_empty(B, T),
+            x.new_empty((B, T * 8) if keep_z else (0,)))
+
+
 # ----------------------------------------------------------------------------- code_score
 
 _L.define("code_score(Tensor z) -> (Tensor, Tensor)")
@@ -336,6 +373,7 @@ def _(code, score, g, S):
 fht = torch.ops.lookupffn.fht
 bh4_diag = torch.ops.lookupffn.bh4_diag
 project_hash = torch.ops.lookupffn.project_hash
+ln_project_hash = torch.ops.lookupffn.ln_project_hash
 code_score = torch.ops.lookupffn.code_score
 code_score_bwd = torch.ops.lookupffn.code_score_bwd
 gather_add = torch.ops.lookupffn.gather_add

@@ -67,6 +67,18 @@ def project_hash(x, diag, bias, T, decay=0.7, keep_z=True):
     return host(codes), host(scores), (host(z) if keep_z else None)
 
 
+def ln_project_hash(x, ln_w, ln_b, eps, diag, bias, T, decay=0.7):
+    xd, wd, bd2, dd, bd = dev(x), dev(ln_w), dev(ln_b), dev(diag), dev(bias)
+    B, H = x.shape
+    R, J, D = diag.shape
+    codes = torch.full((B, T), -1, dtype=torch.int32, device=DEV)
+    scores = torch.full((B, T), float("nan"), dtype=torch.float32, device=DEV)
+    z = torch.full((B, T * 8), float("nan"), dtype=torch.float32, device=DEV)
+    _call("lffn_ln_project_hash_f32", p(xd), p(wd), p(bd2), float(np.float32(eps)), p(dd), p(bd), p(z), p(codes),
+          p(scores), B, H, D, R, J, T, float(np.float32(decay)), float(np.float32(1 - decay)))
+    return host(codes), host(scores), host(z)
+
+
 def code_score(z):
     zd = dev(z)
     k = z.shape[-1]

@@ -142,6 +142,41 @@ def test_project_hash_matches_oracle(H, D, R, T):
     assert np.array_equal(z3, z_nb) and np.array_equal(codes3, oracle.code_score(z_nb.reshape(B, T, 8))[0])
 
 
+@pytest.mark.parametrize("H,D,R,T", [(256, 256, 1, 32), (768, 1024, 1, 128), (1024, 1024, 4, 512), (100, 128, 2, 30),
+                                      (48, 64, 1, 5), (6, 8, 1, 1)])
+def test_ln_project_hash_matches_oracle(H, D, R, T):
+    """LayerNorm fused into the projection kernel.  Its sums run in another order than
+    the oracle's (and torch's), so h and z agree to rounding: z within 1e-5 of the
+    float64 truth, a code may differ only where the true z is within that rounding of 0."""
+    rng = np.random.RandomState(H + 7 * T)
+    B, J = 300, 4
+    x = (rng.randn(B, H) * 1.5 + 0.3).astype(np.float32)
+    ln_w = (1 + 0.1 * rng.randn(H)).astype(np.float32)
+    ln_b = (0.1 * rng.randn(H)).astype(np.float32)
+    diag = ((2 * rng.randint(0, 2, size=(R, J, D)) - 1) / math.sqrt(D)).astype(np.float32)
+    bias = (0.05 * rng.randn(T * 8)).astype(np.float32)
+    h64 = oracle.layernorm(x.astype(np.float64), ln_w, ln_b, 1e-5)
+    z64 = oracle.projection(h64, diag.reshape(R, J, D, 1, 1).astype(np.float64), bias.astype(np.float64), T * 8, 0.7)
+    code64, score64 = oracle.code_score(z64.reshape(B, T, 8))
+    codes, scores, z = cabi.ln_project_hash(x, ln_w, ln_b, 1e-5, diag, bias, T)
+    scale = np.abs(z64).max()
+    assert np.abs(z - z64).max() <= 1e-5 * scale
+    flipped = (z.reshape(B, T, 8) > 0) != (z64.reshape(B, T, 8) > 0)
+    assert np.all(np.abs(z64.reshape(B, T, 8)[flipped]) <= 1e-5 * scale)
+    same = codes == code64
+    assert same.mean() >= 0.999
+    np.testing.assert_allclose(scores[same], score64[same], rtol=2e-4)   # |z| enters the score: 1e-5*scale on z
+    # the kernel's own codes and scores are those of its own z, exactly
+    code_z, score_z = oracle.code_score(z.reshape(B, T, 8))
+    assert np.array_equal(codes, code_z)
+    np.testing.assert_allclose(scores, score_z, rtol=2e-6)
+    # against the two-kernel path (torch LayerNorm on the GPU, then the projection kernel)
+    h_gpu = torch.nn.functional.layer_norm(torch.tensor(x, device="cuda:0"), (H,), torch.tensor(ln_w, device="cuda:0"),
+                                           torch.tensor(ln_b, device="cuda:0"), 1e-5).cpu().numpy()
+    _, _, z2 = cabi.project_hash(h_gpu, diag, bias, T)
+    assert np.abs(z - z2).max() <= 1e-5 * scale
+
+
 def test_project_hash_near_zero_flip_count():
     # end to end against the float64 truth: flips may only happen where |z| is tiny
     rng = np.random.RandomState(9)
