@@ -161,13 +161,35 @@ int lffn_lookup_gather_bf16(const int32_t *code, const float *score, const uint1
                             int64_t B, int64_t T, int64_t S, int64_t Do, void *stream);
 
 /*
- * Which kernel lffn_lookup_gather_{f32,bf16} runs for a shape: the number of
- * tokens whose accumulators one workgroup keeps in registers while it walks the
+ * Which kernel lffn_lookup_gather_{f32,bf16} runs for a shape.  Returns the number
+ * of tokens whose accumulators one workgroup keeps in registers while it walks the
  * tables through LDS, or 0 when the token-major kernel is used (small batches,
- * S > 256).  Pure host function, no GPU work; negative on bad arguments.
+ * S > 256); *tables_per_buffer (may be NULL) receives 0 (token-major), 1 (256-byte
+ * column slices, one table per LDS buffer) or 2 (128-byte slices, two tables per
+ * buffer).  Pure host function, no GPU work; negative on bad arguments.
  * No counterpart in the reference (its gather has one kernel, gather_fp32.cu:6-36).
  */
-int lffn_lookup_gather_plan(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t bf16);
+int lffn_lookup_gather_plan(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t bf16,
+                            int32_t *tables_per_buffer);
+
+/*
+ * lffn_lookup_gather_{f32,bf16} with the kernel named by the caller instead of
+ * chosen by lffn_lookup_gather_plan (for tuning, and so that every built kernel
+ * can be tested on any shape): tables_per_buffer 0, 1 or 2 as reported by the plan
+ * function; tokens_per_workgroup a multiple of 64 (one table per buffer: 256, 512,
+ * 832, 1024; bf16 256, 512) or of 128 (two tables per buffer: 512, 1024, 1664,
+ * 2048; bf16 512, 1024), ignored for 0.  LFFN_ERR_UNSUPPORTED if that kernel is not
+ * built or the shape does not meet its conditions (S <= 256, Do a multiple of the
+ * slice width).  No counterpart in the reference.
+ */
+int lffn_lookup_gather_planned_f32(const int32_t *code, const float *score, const float *tables,
+                                   const float *bias, float *out,
+                                   int64_t B, int64_t T, int64_t S, int64_t Do,
+                                   int32_t tables_per_buffer, int32_t tokens_per_workgroup, void *stream);
+int lffn_lookup_gather_planned_bf16(const int32_t *code, const float *score, const uint16_t *tables,
+                                    const float *bias, float *out,
+                                    int64_t B, int64_t T, int64_t S, int64_t Do,
+                                    int32_t tables_per_buffer, int32_t tokens_per_workgroup, void *stream);
 
 /*
  * out[b,i] = <g[b,:], src[idx[b,i],:]>   (gradient w.r.t. the weights).

@@ -39,7 +39,11 @@ SIGNATURES = {
     "lffn_gather_add_bf16": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "lffn_lookup_gather_f32": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "lffn_lookup_gather_bf16": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
-    "lffn_lookup_gather_plan": [_i64, _i64, _i64, _i64, ctypes.c_int32],
+    "lffn_lookup_gather_planned_f32": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
+                                       ctypes.c_int32, ctypes.c_int32, _vp],
+    "lffn_lookup_gather_planned_bf16": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
+                                        ctypes.c_int32, ctypes.c_int32, _vp],
+    "lffn_lookup_gather_plan": [_i64, _i64, _i64, _i64, ctypes.c_int32, ctypes.POINTER(ctypes.c_int32)],
     "lffn_indexed_inner_product_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "lffn_scatter_add_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "lffn_lookup_scatter_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, ctypes.c_int32, _vp],

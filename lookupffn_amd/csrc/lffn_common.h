@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "../../include/lookupffn_hip.h"
 
 #define LFFN_WAVE 64
@@ -33,6 +35,12 @@ __attribute__((visibility("hidden")))
 int lffn_internal_lookup_scatter_atomic(const int32_t *code, const float *score, const float *g, float *out,
                                         int64_t B, int64_t T, int64_t S, int64_t Do, void *stream);
 
+// lookup_gather_pair.hip: the two-tables-per-buffer LDS gather (not exported)
+__attribute__((visibility("hidden")))
+int lffn_internal_lookup_gather_pair(const int32_t *code, const float *score, const void *tables,
+                                     const float *bias, float *out, int64_t B, int64_t T, int64_t S,
+                                     int64_t Do, bool bf16, int np, void *stream);
+
 static inline int lffn_launch_status() {
     return hipGetLastError() == hipSuccess ? LFFN_OK : LFFN_ERR_LAUNCH;
 }
@@ -52,6 +60,24 @@ constexpr int DPP_QUAD_XOR2 = 0x4E;   // quad_perm [2,3,0,1]
 constexpr int DPP_ROW_SHL4 = 0x104;   // lane i <- lane i+4
 constexpr int DPP_ROW_SHR4 = 0x114;   // lane i <- lane i-4
 constexpr int DPP_ROW_ROR8 = 0x128;   // lane i <- lane (i-8) mod 16 == i xor 8
+constexpr int DPP_ROW_NEWBCAST0 = 0x150;   // + n: every lane of a 16-lane row <- lane n of that row
+
+// Value held by lane N of the caller's 16-lane row, in every lane of the row (one
+// vector-ALU move, no LDS traffic).  N is a compile-time constant.
+template <int N>
+__device__ __forceinline__ int row_broadcast(int v) {
+    static_assert(N >= 0 && N < 16, "row_broadcast: lane within the row");
+    return __builtin_amdgcn_update_dpp(v, v, DPP_ROW_NEWBCAST0 + N, 0xF, 0xF, false);
+}
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>)
+template <int N, typename F, int I = 0>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<N, F, I + 1>(static_cast<F &&>(f));
+    }
+}
 
 // Value held by lane (lane ^ M), for M a power of two below 64.
 template <int M>

@@ -21,14 +21,15 @@
 // So each table slice is fetched once per 64*NP tokens instead of once per
 // token, and the per-token row reads are LDS reads.  The (code, score) pairs are
 // read 16 tables at a time, one table per lane of the 16-lane token group (four
-// 8-bit codes packed per register), and handed to the group's lanes with
-// ds_bpermute when their table comes up.
+// 8-bit codes packed per register), and handed to the group's lanes with a DPP
+// row broadcast when their table comes up.
 //
 // blockIdx -> (slice, token tile) is XCD-aware: workgroups are dealt round-robin
 // to the 8 XCDs, so block b runs on XCD b % 8; units are numbered so that the
 // workgroups of one XCD share as few slices as possible and the slice they
 // stream stays in that XCD's L2.
 #include "lffn_common.h"
+
 
 namespace {
 
@@ -157,62 +158,65 @@ __global__ __launch_bounds__(WG) void lookup_gather_lds_kernel(LdsGatherArgs a) 
         for (int p = 0; p < NP; ++p) asm volatile("" : "+v"(sc[p]));
 
         const int nt = min(CHUNK, a.T - t0);
-        for (int tt = 0; tt < nt; ++tt) {
-            const int t = t0 + tt;
-            // next table's slice goes straight into the other buffer, which was last read
-            // one table ago, before the previous barrier (the last iteration re-copies
-            // the last table: harmless)
-            copy_slice_to_lds<FULL>(slice_base + (size_t)min(t + 1, a.T - 1) * table_bytes, a.row_bytes, tid,
-                                    buf_vecs, lds + ((t + 1) & 1) * buf_vecs);
-            const uint4 *buf = lds + (t & 1) * buf_vecs + j;
-            const int src_lane = ((lane & 48) | tt) << 2;      // byte address of lane (grp*16 + tt)
-            // All code broadcasts first, then the passes in groups of at most GRP: a
-            // group's score broadcasts and row reads are issued together (GRP rows in
-            // flight per lane), then its fmas.  The scheduling barriers keep the
-            // compiler from merging groups, which would not fit the register file.
-            unsigned packed[NQ];
+        // The 16 tables of the chunk, unrolled: table t0 + TT takes its codes and scores
+        // from lane TT of each 16-lane token group with a DPP row broadcast (a vector-ALU
+        // move), so that the only LDS traffic of the pass loop is the row reads.
+        static_for<CHUNK>([&](auto tt_c) {
+            constexpr int TT = decltype(tt_c)::value;
+            if (TT < nt) {                                     // uniform
+                const int t = t0 + TT;
+                // next table's slice goes straight into the other buffer, which was last
+                // read one table ago, before the previous barrier (the last iteration
+                // re-copies the last table: harmless)
+                copy_slice_to_lds<FULL>(slice_base + (size_t)min(t + 1, a.T - 1) * table_bytes, a.row_bytes, tid,
+                                        buf_vecs, lds + ((t + 1) & 1) * buf_vecs);
+                const uint4 *buf = lds + (t & 1) * buf_vecs + j;
+                unsigned packed[NQ];
 #pragma unroll
-            for (int q = 0; q < NQ; ++q) packed[q] = (unsigned)__builtin_amdgcn_ds_bpermute(src_lane, (int)cd[q]);
-            constexpr int GRP = BF16 ? 4 : (NP >= 16 ? 4 : (NP > 8 ? 5 : NP));
+                for (int q = 0; q < NQ; ++q) packed[q] = (unsigned)row_broadcast<TT>((int)cd[q]);
+                // passes in groups of at most GRP: a group's row reads are issued together
+                // (GRP rows in flight per lane), then its fmas; the scheduling barriers keep
+                // the compiler from merging groups, which would not fit the register file
+                constexpr int GRP = BF16 ? 4 : (NP >= 16 ? 4 : (NP > 8 ? 5 : NP));
 #pragma unroll
-            for (int g0 = 0; g0 < NP; g0 += GRP) {
-                float w[GRP];
-                uint4 r[GRP];
+                for (int g0 = 0; g0 < NP; g0 += GRP) {
+                    uint4 r[GRP];
 #pragma unroll
-                for (int i = 0; i < GRP; ++i) {
-                    const int p = g0 + i;
-                    if (p < NP) {
-                        w[i] = __int_as_float(__builtin_amdgcn_ds_bpermute(src_lane, __float_as_int(sc[p])));
-                        const unsigned row = (packed[p / 4] >> (8 * (p % 4))) & 0xFFu;
-                        r[i] = buf[row * SEG_VECS];
-                    }
-                }
-#pragma unroll
-                for (int i = 0; i < GRP; ++i) {
-                    const int p = g0 + i;
-                    if (p < NP) {
-                        if constexpr (BF16) {
-                            acc[p][0] = fmaf(bf16_lo(r[i].x), w[i], acc[p][0]);
-                            acc[p][1] = fmaf(bf16_hi(r[i].x), w[i], acc[p][1]);
-                            acc[p][2] = fmaf(bf16_lo(r[i].y), w[i], acc[p][2]);
-                            acc[p][3] = fmaf(bf16_hi(r[i].y), w[i], acc[p][3]);
-                            acc[p][4] = fmaf(bf16_lo(r[i].z), w[i], acc[p][4]);
-                            acc[p][5] = fmaf(bf16_hi(r[i].z), w[i], acc[p][5]);
-                            acc[p][6] = fmaf(bf16_lo(r[i].w), w[i], acc[p][6]);
-                            acc[p][7] = fmaf(bf16_hi(r[i].w), w[i], acc[p][7]);
-                        } else {
-                            acc[p][0] = fmaf(__uint_as_float(r[i].x), w[i], acc[p][0]);
-                            acc[p][1] = fmaf(__uint_as_float(r[i].y), w[i], acc[p][1]);
-                            acc[p][2] = fmaf(__uint_as_float(r[i].z), w[i], acc[p][2]);
-                            acc[p][3] = fmaf(__uint_as_float(r[i].w), w[i], acc[p][3]);
+                    for (int i = 0; i < GRP; ++i) {
+                        const int p = g0 + i;
+                        if (p < NP) {
+                            const unsigned row = (packed[p / 4] >> (8 * (p % 4))) & 0xFFu;
+                            r[i] = buf[row * SEG_VECS];
                         }
                     }
+#pragma unroll
+                    for (int i = 0; i < GRP; ++i) {
+                        const int p = g0 + i;
+                        if (p < NP) {
+                            const float w = __int_as_float(row_broadcast<TT>(__float_as_int(sc[p])));
+                            if constexpr (BF16) {
+                                acc[p][0] = fmaf(bf16_lo(r[i].x), w, acc[p][0]);
+                                acc[p][1] = fmaf(bf16_hi(r[i].x), w, acc[p][1]);
+                                acc[p][2] = fmaf(bf16_lo(r[i].y), w, acc[p][2]);
+                                acc[p][3] = fmaf(bf16_hi(r[i].y), w, acc[p][3]);
+                                acc[p][4] = fmaf(bf16_lo(r[i].z), w, acc[p][4]);
+                                acc[p][5] = fmaf(bf16_hi(r[i].z), w, acc[p][5]);
+                                acc[p][6] = fmaf(bf16_lo(r[i].w), w, acc[p][6]);
+                                acc[p][7] = fmaf(bf16_hi(r[i].w), w, acc[p][7]);
+                            } else {
+                                acc[p][0] = fmaf(__uint_as_float(r[i].x), w, acc[p][0]);
+                                acc[p][1] = fmaf(__uint_as_float(r[i].y), w, acc[p][1]);
+                                acc[p][2] = fmaf(__uint_as_float(r[i].z), w, acc[p][2]);
+                                acc[p][3] = fmaf(__uint_as_float(r[i].w), w, acc[p][3]);
+                            }
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
-                __builtin_amdgcn_sched_barrier(0);
+                __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0): the copy issued above has landed
+                __syncthreads();
             }
-            __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0): the copies issued above have landed
-            __syncthreads();
-        }
+        });
     }
 
 #pragma unroll
@@ -249,40 +253,66 @@ int launch_lds(const LdsGatherArgs &a, hipStream_t stream) {
     return a.S == MAX_S ? launch_lds_full<BF16, NP, true>(a, stream) : launch_lds_full<BF16, NP, false>(a, stream);
 }
 
-// Plan for a shape: 0 = token-major kernel (gather.hip), otherwise NP of the
-// LDS-tiled kernel (64*NP tokens per workgroup).
-//
-// The LDS-tiled form needs the table to fit the buffers (S <= 256), rows that
-// split into whole 256-byte segments, and enough (token tile, slice) units to
-// occupy most of the 256 CUs even at the smallest tile.  Among the NP that are
-// built, the measured time per workgroup per table is close to (7 + NP) * 0.1 us
-// (staging a slice costs as much as seven passes), and workgroups run in
-// ceil(units / 256) rounds, one workgroup per CU.
+// Which kernel a shape gets.
+//   kind 0  token-major kernel (gather.hip): small batches, S > 256
+//   kind 1  one table per LDS buffer (this file): 256-byte slices, 64*np tokens per workgroup
+//   kind 2  two tables per LDS buffer (lookup_gather_pair.hip): 128-byte slices, 128*np tokens
+// The LDS forms need the table to fit the buffers (S <= 256), rows that split into
+// whole slices, and enough (token tile, slice) units to occupy most of the 256 CUs
+// at the smallest tile.  Workgroups run one per CU in ceil(units / 256) rounds; the
+// time of a round is T tables times a per-table cost measured on MI355X for each
+// built tile size (microseconds, tables that fit the 256 MB Infinity Cache; larger
+// table sets cost BIG times more).  The cheapest predicted time wins.
+struct GatherPlan {
+    int kind, np;
+};
+
 template <bool BF16>
-int plan_np(int64_t B, int64_t T, int64_t S, int64_t Do) {
-    const int cols = BF16 ? 128 : 64;
-    if (S > MAX_S || Do % cols != 0 || T < 4) return 0;
-    const int64_t nslices = Do / cols;
-    if (((B + 255) / 256) * nslices < 192) return 0;
-    if (B * nslices > (int64_t(1) << 30)) return 0;
-    constexpr int NPS_F32[] = {16, 13, 8, 4};
-    constexpr int NPS_BF16[] = {8, 4, 4, 4};
-    double best_cost = 1e300;
-    int best = 0;
-    for (int k = 0; k < 4; ++k) {
-        const int np = BF16 ? NPS_BF16[k] : NPS_F32[k];
-        if (S != MAX_S && np > (BF16 ? 4 : 8)) continue;   // the partial-table variants have fewer free registers
-        const int64_t tiles = (B + 64 * np - 1) / (64 * np);
+GatherPlan plan_gather(int64_t B, int64_t T, int64_t S, int64_t Do) {
+    GatherPlan best{0, 0};
+    if (S > MAX_S || T < 4 || B * T >= (int64_t(1) << 31)) return best;
+    struct Option { int kind, np; double us_per_table; };
+    static const Option f32_opts[] = {{1, 4, 1.15}, {1, 8, 1.18}, {1, 13, 1.30}, {1, 16, 1.60},
+                                      {2, 4, 0.88}, {2, 8, 1.01}, {2, 13, 1.47}, {2, 16, 1.79}};
+    static const Option bf16_opts[] = {{1, 4, 1.21}, {1, 8, 1.32}, {2, 4, 0.97}, {2, 8, 1.20}};
+    const Option *opts = BF16 ? bf16_opts : f32_opts;
+    const int nopts = BF16 ? 4 : 8;
+    const bool big = double(T) * double(S) * double(Do) * (BF16 ? 2 : 4) > 200e6;
+    double best_us = 1e300;
+    for (int k = 0; k < nopts; ++k) {
+        const Option &o = opts[k];
+        const int cols = (o.kind == 1 ? 256 : 128) / (BF16 ? 2 : 4);
+        const int tok = (o.kind == 1 ? 64 : 128) * o.np;
+        if (Do % cols != 0) continue;
+        const int64_t nslices = Do / cols;
+        // enough units at the smallest tile of this form to be worth staging tables at all
+        if (((B + tok / o.np * 4 - 1) / (tok / o.np * 4)) * nslices < 192) continue;
+        if (B * nslices > (int64_t(1) << 30)) continue;
+        const int64_t tiles = (B + tok - 1) / tok;
         const int64_t rounds = (tiles * nslices + 255) / 256;
-        const double cost = double(rounds) * (7.0 + np);
-        if (cost < best_cost) { best_cost = cost; best = np; }
+        const double us = double(rounds) * double(T) * o.us_per_table * (big ? (o.kind == 1 ? 1.3 : 1.15) : 1.0);
+        if (us < best_us) { best_us = us; best = GatherPlan{o.kind, o.np}; }
     }
     return best;
 }
 
+// Is (kind, np) a kernel that is built, and does the shape meet its preconditions?
+template <bool BF16>
+bool plan_is_valid(const GatherPlan &p, int64_t B, int64_t T, int64_t S, int64_t Do) {
+    if (p.kind == 0) return true;
+    if (p.kind != 1 && p.kind != 2) return false;
+    const bool np_ok = BF16 ? (p.np == 4 || p.np == 8) : (p.np == 4 || p.np == 8 || p.np == 13 || p.np == 16);
+    const int cols = (p.kind == 1 ? 256 : 128) / (BF16 ? 2 : 4);
+    return np_ok && S <= MAX_S && T >= 1 && Do % cols == 0 && B * T < (int64_t(1) << 31) &&
+           B * (Do / cols) <= (int64_t(1) << 30);
+}
+
+// kind_req < 0: choose the kernel with plan_gather; otherwise run exactly the
+// requested kernel (kind_req tables per buffer, tokens_req tokens per workgroup).
 template <bool BF16>
 int lookup_gather_entry(const int32_t *code, const float *score, const void *tables, const float *bias,
-                        float *out, int64_t B, int64_t T, int64_t S, int64_t Do, void *stream) {
+                        float *out, int64_t B, int64_t T, int64_t S, int64_t Do, int kind_req, int tokens_req,
+                        void *stream) {
     LFFN_REQUIRE(B >= 0 && T >= 0 && Do >= 1, LFFN_ERR_BAD_ARG);
     LFFN_REQUIRE(lffn_is_pow2(S) && S <= (1 << 24) && T * S <= 0x7fffffff, LFFN_ERR_UNSUPPORTED);
     LFFN_REQUIRE(Do % 64 == 0 && Do <= (1 << 20) && T <= (1 << 24), LFFN_ERR_UNSUPPORTED);
@@ -290,9 +320,21 @@ int lookup_gather_entry(const int32_t *code, const float *score, const void *tab
     LFFN_REQUIRE(tables && out && ((code && score) || B * T == 0), LFFN_ERR_BAD_ARG);
     LFFN_REQUIRE(lffn_aligned16(tables) && lffn_aligned16(out) && (!bias || lffn_aligned16(bias)), LFFN_ERR_BAD_ARG);
     if (B == 0) return LFFN_OK;
-    const int np = plan_np<BF16>(B, T, S, Do);
-    if (np == 0)
+    GatherPlan plan;
+    if (kind_req < 0) {
+        plan = plan_gather<BF16>(B, T, S, Do);
+    } else {
+        plan.kind = kind_req;
+        const int per_np = kind_req == 1 ? 64 : 128;
+        plan.np = kind_req == 0 ? 0 : tokens_req / per_np;
+        LFFN_REQUIRE(kind_req == 0 || (tokens_req > 0 && tokens_req % per_np == 0), LFFN_ERR_BAD_ARG);
+        LFFN_REQUIRE(plan_is_valid<BF16>(plan, B, T, S, Do), LFFN_ERR_UNSUPPORTED);
+    }
+    if (plan.kind == 0)
         return lffn_internal_lookup_gather_token_major(code, score, tables, bias, out, B, T, S, Do, BF16, stream);
+    if (plan.kind == 2)
+        return lffn_internal_lookup_gather_pair(code, score, tables, bias, out, B, T, S, Do, BF16, plan.np, stream);
+    const int np = plan.np;
     LdsGatherArgs a{};
     a.code = code; a.score = score; a.tables = static_cast<const char *>(tables); a.bias = bias; a.out = out;
     a.B = B; a.T = (int)T; a.S = (int)S; a.Do = (int)Do;
@@ -316,16 +358,37 @@ int lookup_gather_entry(const int32_t *code, const float *score, const void *tab
 extern "C" int lffn_lookup_gather_f32(const int32_t *code, const float *score, const float *tables,
                                       const float *bias, float *out,
                                       int64_t B, int64_t T, int64_t S, int64_t Do, void *stream) {
-    return lookup_gather_entry<false>(code, score, tables, bias, out, B, T, S, Do, stream);
+    return lookup_gather_entry<false>(code, score, tables, bias, out, B, T, S, Do, -1, 0, stream);
 }
 
 extern "C" int lffn_lookup_gather_bf16(const int32_t *code, const float *score, const uint16_t *tables,
                                        const float *bias, float *out,
                                        int64_t B, int64_t T, int64_t S, int64_t Do, void *stream) {
-    return lookup_gather_entry<true>(code, score, tables, bias, out, B, T, S, Do, stream);
+    return lookup_gather_entry<true>(code, score, tables, bias, out, B, T, S, Do, -1, 0, stream);
 }
 
-extern "C" int lffn_lookup_gather_plan(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t bf16) {
+extern "C" int lffn_lookup_gather_planned_f32(const int32_t *code, const float *score, const float *tables,
+                                              const float *bias, float *out,
+                                              int64_t B, int64_t T, int64_t S, int64_t Do,
+                                              int32_t tables_per_buffer, int32_t tokens_per_workgroup, void *stream) {
+    LFFN_REQUIRE(tables_per_buffer >= 0, LFFN_ERR_BAD_ARG);
+    return lookup_gather_entry<false>(code, score, tables, bias, out, B, T, S, Do, tables_per_buffer,
+                                      tokens_per_workgroup, stream);
+}
+
+extern "C" int lffn_lookup_gather_planned_bf16(const int32_t *code, const float *score, const uint16_t *tables,
+                                               const float *bias, float *out,
+                                               int64_t B, int64_t T, int64_t S, int64_t Do,
+                                               int32_t tables_per_buffer, int32_t tokens_per_workgroup, void *stream) {
+    LFFN_REQUIRE(tables_per_buffer >= 0, LFFN_ERR_BAD_ARG);
+    return lookup_gather_entry<true>(code, score, tables, bias, out, B, T, S, Do, tables_per_buffer,
+                                     tokens_per_workgroup, stream);
+}
+
+extern "C" int lffn_lookup_gather_plan(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t bf16,
+                                       int32_t *tables_per_buffer) {
     if (B < 0 || T < 0 || Do < 1 || !lffn_is_pow2(S) || Do % 64 != 0) return LFFN_ERR_BAD_ARG;
-    return 64 * (bf16 ? plan_np<true>(B, T, S, Do) : plan_np<false>(B, T, S, Do));
+    const GatherPlan plan = bf16 ? plan_gather<true>(B, T, S, Do) : plan_gather<false>(B, T, S, Do);
+    if (tables_per_buffer) *tables_per_buffer = plan.kind;
+    return plan.kind == 0 ? 0 : (plan.kind == 1 ? 64 : 128) * plan.np;
 }

@@ -106,14 +106,26 @@ def gather_add(idx, src, w, bf16=False):
     return host(out)
 
 
-def lookup_gather(code, score, tables, bias=None, bf16=False):
+def lookup_gather(code, score, tables, bias=None, bf16=False, plan=None):
+    """plan = (tables_per_buffer, tokens_per_workgroup) runs exactly that kernel."""
     cd, sd, td, bd = dev(code), dev(score), dev(tables), dev(bias)
     B, T = code.shape
     _, S, Do = tables.shape
     out = torch.full((B, Do), float("nan"), dtype=torch.float32, device=DEV)
-    _call("lffn_lookup_gather_bf16" if bf16 else "lffn_lookup_gather_f32",
-          p(cd), p(sd), p(td), p(bd), p(out), B, T, S, Do)
+    if plan is None:
+        _call("lffn_lookup_gather_bf16" if bf16 else "lffn_lookup_gather_f32",
+              p(cd), p(sd), p(td), p(bd), p(out), B, T, S, Do)
+    else:
+        _call("lffn_lookup_gather_planned_bf16" if bf16 else "lffn_lookup_gather_planned_f32",
+              p(cd), p(sd), p(td), p(bd), p(out), B, T, S, Do, plan[0], plan[1])
     return host(out)
+
+
+def lookup_gather_plan(B, T, S, Do, bf16=False):
+    import ctypes
+    kind = ctypes.c_int32(-1)
+    tokens = _lib.load().lffn_lookup_gather_plan(B, T, S, Do, int(bf16), ctypes.byref(kind))
+    return kind.value, tokens
 
 
 def indexed_inner_product(idx, g, src):

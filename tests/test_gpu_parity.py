@@ -297,25 +297,21 @@ def test_gather_add_bf16_matches_oracle(B, T, S, Do):
         assert relmax(cabi.lookup_gather(code, w, bits.reshape(T, S, Do), None, bf16=True), want_bf) <= 1e-5
 
 
-# shapes that take the LDS-tiled kernel, with the tokens per workgroup the plan must pick:
-# every tile size that is built (256/512/832/1024 tokens), ragged token counts, table
-# counts that are not multiples of the 16-table chunk, tables smaller than the LDS buffer
-LDS_CASES = [(3000, 20, 256, 1024, False, 256), (16384, 6, 256, 512, False, 512), (16384, 5, 256, 768, False, 832),
-             (16384, 7, 256, 1024, False, 1024), (16301, 33, 256, 768, False, 832), (3001, 17, 64, 1024, False, 256),
-             (16384, 35, 128, 512, False, 512), (16384, 6, 256, 1024, True, 512), (5003, 19, 256, 2048, True, 512),
-             (3000, 18, 32, 2048, True, 256), (16384, 4, 256, 256, False, 256)]
+# Every LDS-tiled gather kernel that is built: (tables per buffer, tokens per workgroup).
+F32_PLANS = [(1, 256), (1, 512), (1, 832), (1, 1024), (2, 512), (2, 1024), (2, 1664), (2, 2048)]
+BF16_PLANS = [(1, 256), (1, 512), (2, 512), (2, 1024)]
+# (B, T, S, Do): ragged token counts, table counts that are odd / not multiples of the 8-
+# and 16-table chunks, tables smaller than the LDS buffer, one and several token tiles
+LDS_SHAPES = [(3000, 20, 256, 256), (4133, 5, 256, 384), (2049, 33, 64, 128), (1000, 17, 256, 128), (5000, 8, 32, 256)]
 
 
-@pytest.mark.parametrize("B,T,S,Do,bf16,tokens_per_wg", LDS_CASES)
-def test_lookup_gather_lds_tiled_matches_oracle(B, T, S, Do, bf16, tokens_per_wg):
-    from lookupffn_amd import _lib
-    assert _lib.load().lffn_lookup_gather_plan(B, T, S, Do, int(bf16)) == tokens_per_wg
-    rng = np.random.RandomState(B + T + S + Do)
+def _check_lds_gather(B, T, S, Do, bf16, plan):
+    rng = np.random.RandomState(B + T + S + Do + 131 * plan[0] + plan[1])
     tables, code, idx, w = _rand_gather(rng, B, T, S, Do)
     bias = (0.001 * rng.randn(Do)).astype(np.float32)
     flat = tables.reshape(T * S, Do)
     src = oracle.bf16_round(flat) if bf16 else flat
-    got = cabi.lookup_gather(code, w, src.reshape(T, S, Do), bias, bf16=bf16)
+    got = cabi.lookup_gather(code, w, src.reshape(T, S, Do), bias, bf16=bf16, plan=plan)
     assert not np.isnan(got).any()
     # a random sample of tokens plus the whole ragged tail
     sub = np.unique(np.concatenate([rng.choice(B, 96, replace=False), np.arange(B - 80, B), np.arange(0, 8)]))
@@ -325,14 +321,52 @@ def test_lookup_gather_lds_tiled_matches_oracle(B, T, S, Do, bf16, tokens_per_wg
     else:
         want = oracle.gather_add(idx[sub], flat.astype(np.float64), w64) + bias
     assert relmax(got[sub], want) <= 1e-5
-    # the two kernels (LDS-tiled, token-major) agree on every token
-    assert relmax(got, cabi.gather_add(idx, src, w, bf16=bf16).astype(np.float64) + bias) <= 1e-6
+    # the LDS-tiled and the token-major kernels agree on every token
+    assert relmax(got, cabi.gather_add(idx, src, w, bf16=bf16).astype(np.float64) + bias) <= 2e-6
     # codes are masked into their table: bits above log2(S) are ignored
     dirty = (code + S * rng.randint(0, 5, size=code.shape)).astype(np.int32)
-    assert np.array_equal(cabi.lookup_gather(dirty, w, src.reshape(T, S, Do), bias, bf16=bf16), got)
+    assert np.array_equal(cabi.lookup_gather(dirty, w, src.reshape(T, S, Do), bias, bf16=bf16, plan=plan), got)
     # no bias
-    got_nb = cabi.lookup_gather(code, w, src.reshape(T, S, Do), None, bf16=bf16)
+    got_nb = cabi.lookup_gather(code, w, src.reshape(T, S, Do), None, bf16=bf16, plan=plan)
     assert relmax(got_nb[sub], want - bias) <= 1e-5
+
+
+@pytest.mark.parametrize("plan", F32_PLANS)
+@pytest.mark.parametrize("B,T,S,Do", LDS_SHAPES)
+def test_lookup_gather_lds_kernels_match_oracle(B, T, S, Do, plan):
+    _check_lds_gather(B, T, S, Do, False, plan)
+
+
+@pytest.mark.parametrize("plan", BF16_PLANS)
+@pytest.mark.parametrize("B,T,S,Do", LDS_SHAPES)
+def test_lookup_gather_lds_kernels_bf16_match_oracle(B, T, S, Do, plan):
+    _check_lds_gather(B, T, S, Do, True, plan)
+
+
+def test_lookup_gather_plan_and_planned_entry():
+    from lookupffn_amd import _lib
+    # what the heuristic picks at the BASELINE shapes
+    assert cabi.lookup_gather_plan(16384, 128, 256, 768) == (1, 832)            # config 2
+    assert cabi.lookup_gather_plan(16384, 512, 256, 1024) == (2, 2048)          # config 3 fp32
+    assert cabi.lookup_gather_plan(16384, 512, 256, 1024, bf16=True) == (2, 1024)
+    assert cabi.lookup_gather_plan(256, 32, 256, 256) == (0, 0)                 # config 1: token-major
+    assert cabi.lookup_gather_plan(16384, 128, 512, 768) == (0, 0)              # S > 256
+    # every plan the heuristic can return is one of the built kernels
+    for B in (1024, 3000, 16384, 100000):
+        for T in (4, 32, 128, 512):
+            for Do in (64, 256, 768, 1024, 2048):
+                for bf in (False, True):
+                    kind, tokens = cabi.lookup_gather_plan(B, T, 256, Do, bf16=bf)
+                    assert (kind, tokens) == (0, 0) or (kind, tokens) in (BF16_PLANS if bf else F32_PLANS)
+    # a kernel that is not built, or a shape it cannot take, is refused before any launch
+    lib = _lib.load()
+    args = (256, 256, 256, None, 256, 3000, 20, 256, 256)
+    assert lib.lffn_lookup_gather_planned_f32(*args, 1, 320, None) == _lib.LFFN_ERR_UNSUPPORTED      # 5 passes: not built
+    assert lib.lffn_lookup_gather_planned_f32(*args, 1, 100, None) == _lib.LFFN_ERR_BAD_ARG          # not a multiple of 64
+    assert lib.lffn_lookup_gather_planned_f32(*args, 3, 512, None) == _lib.LFFN_ERR_UNSUPPORTED      # no such kernel
+    assert lib.lffn_lookup_gather_planned_bf16(*args, 2, 2048, None) == _lib.LFFN_ERR_UNSUPPORTED    # fp32 only
+    big_s = (256, 256, 256, None, 256, 3000, 20, 512, 256)
+    assert lib.lffn_lookup_gather_planned_f32(*big_s, 1, 512, None) == _lib.LFFN_ERR_UNSUPPORTED     # S > 256
 
 
 def test_gather_special_cases():
