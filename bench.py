@@ -42,6 +42,10 @@ WORKLOADS = {
                  desc="config 3: 16384 tokens, d=1024, 512 tables x 256 x 1024 fp32"),
     "cfg3bf16": dict(B=16384, H=1024, T=512, S=256, Do=1024, bf16=True,
                      desc="config 3: 16384 tokens, d=1024, 512 tables x 256 x 1024 bf16 rows, fp32 accumulate"),
+    # BASELINE.json configs[3]: the 12-layer encoder with every FFN a config-2 LookupFFN
+    "cfg4": dict(B=16384, H=768, T=128, S=256, Do=768, bf16=False,
+                 desc="config 4: 12-layer pre-norm RoBERTa-base encoder (hidden 768, 12 heads, seq 512, batch 32), "
+                      "every FFN a config-2 LookupFFN"),
     # BASELINE.json configs[4]: the backward at the config-2 shape, codes drawn Zipf(1.1)
     "cfg5": dict(B=16384, H=768, T=128, S=256, Do=768, bf16=False,
                  desc="config 5: backward at the config-2 shape, codes Zipf(s=1.1) over 256 entries"),
@@ -233,6 +237,85 @@ def main_backward(args):
     print(json.dumps(res))
 
 
+def main_encoder(args):
+    """End-to-end forward of the 12-layer encoder (attention, LayerNorm, embeddings in
+    PyTorch-ROCm; LookupFFN on this package's kernels) and the LookupFFN share of it."""
+    import torch
+
+    import lookupffn_amd
+    from lookupffn_amd import _lib
+    _lib.load()
+    assert torch.cuda.is_available(), "bench.py needs an MI355X"
+    dev = torch.device("cuda:0")
+    wl = WORKLOADS["cfg4"]
+    batch, seq = 32, 512
+    cfg = Namespace(hidden_size=768, num_attention_heads=12, attention_head_size=64,
+                    attention_probs_dropout_prob=0.1, hidden_dropout_prob=0.1, layer_norm_eps=1e-5,
+                    num_hidden_layers=12, vocab_size=50265, max_position_embeddings=512, type_vocab_size=1,
+                    pad_token_id=1, ffn_num_table=wl["T"], ffn_table_size=wl["S"], projection_type="bh4",
+                    block_size=1)
+    torch.manual_seed(1234)
+    model = lookupffn_amd.Lookup(cfg).eval()
+    with torch.no_grad():
+        for layer in model.encoder.layer:
+            p = layer.FFN.hash.projection
+            p.weight.copy_((2.0 * torch.randint(0, 2, p.weight.shape).float() - 1.0) / math.sqrt(p.padded_in_dim))
+    model = model.to(dev)
+    ids = torch.randint(0, cfg.vocab_size, (batch, seq), device=dev)
+    tt = torch.zeros_like(ids)
+    pos = torch.arange(seq, device=dev)[None].expand(batch, seq).contiguous()
+    mask = torch.ones(batch, seq, device=dev)
+
+    ffn_events = []
+
+    def pre_hook(mod, inp):
+        e = torch.cuda.Event(enable_timing=True); e.record(); mod._ev0 = e
+
+    def post_hook(mod, inp, out):
+        e = torch.cuda.Event(enable_timing=True); e.record(); ffn_events.append((mod._ev0, e))
+
+    def run():
+        with torch.no_grad():
+            return model(ids, tt, pos, mask)[0]
+
+    for _ in range(args.warmup):
+        run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run()
+    torch.cuda.synchronize()
+    sec = time.perf_counter() - t0
+    # LookupFFN share: a separate pass with events around every FFN call
+    hooks = []
+    for layer in model.encoder.layer:
+        hooks.append(layer.FFN.register_forward_pre_hook(pre_hook))
+        hooks.append(layer.FFN.register_forward_hook(post_hook))
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(5):
+        run()
+    e1.record()
+    torch.cuda.synchronize()
+    for h in hooks:
+        h.remove()
+    ffn_ms = sum(a.elapsed_time(b) for a, b in ffn_events) / 5
+    total_ms = e0.elapsed_time(e1) / 5
+    res = {
+        "metric": "12-layer RoBERTa-base encoder with LookupFFN, fwd tokens/s and LookupFFN share of time",
+        "value": batch * seq * args.steps / sec, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": sec / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic (random token ids, random-init weights, seeded sign diagonals)",
+        "config": {"workload": wl["desc"], "tokens": batch * seq, "layers": 12, "hidden": 768, "heads": 12,
+                   "seq_len": seq, "batch": batch, "tables": wl["T"], "table_size": wl["S"],
+                   "attention": "torch scaled_dot_product_attention, fp32"},
+        "roofline": None, "cpu_baseline": None,
+        "lookupffn_ms_per_forward": ffn_ms, "forward_ms_with_events": total_ms,
+        "lookupffn_share": ffn_ms / total_ms,
+    }
+    print(json.dumps(res))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -251,6 +334,8 @@ def main():
 
     if args.workload == "cfg5":
         return main_backward(args)
+    if args.workload == "cfg4":
+        return main_encoder(args)
 
     import torch
 

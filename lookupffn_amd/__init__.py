@@ -11,9 +11,11 @@ from .compute_code_score import ComputeCodeScore, bin2dec, compute_code_score, c
 from .gather import (LookupGather, WeightedVectorGatherAdd, gather, indexed_inner_product, lookup_gather,
                      weighted_gather_add, weighted_vector_gather_add, weighted_vector_scatter_add)
 from .lookup import BH4, Hashing, LookupFFN
+from .encoder import Attention, Encoder, EncoderLayer, Lookup, RobertaEmbeddings
 
 __all__ = [
     "BH4", "Hashing", "LookupFFN",
+    "Attention", "EncoderLayer", "Encoder", "Lookup", "RobertaEmbeddings",
     "bh4", "bh4_cuda", "hadamard", "hadamard_transform", "fast_hadamard_transform",
     "FastHadamardTransform", "FastHadamardTransformDim512", "FastHadamardTransformDim1024",
     "compute_code_score", "compute_code_score_torch", "bin2dec", "ComputeCodeScore",

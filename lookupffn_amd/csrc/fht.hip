@@ -112,14 +112,13 @@ struct ProjectArgs {
     int vec_in;           // x rows are 16-byte aligned and H % 4 == 0
 };
 
-// Local part of the score recurrence over the four values of one float4:
-// s <- s + |z_c|, p <- p * (1 + exp(-2|z_c|)), c ascending.
-__device__ __forceinline__ void score_chain(const float (&z)[4], float &s, float &p) {
+// Part of the score recurrence over the four values of one float4:
+// s <- s + a_c, p <- p * f_c with a_c = |z_c| and f_c = 1 + exp(-2|z_c|), c ascending.
+__device__ __forceinline__ void score_chain(const float (&a)[4], const float (&f)[4], float &s, float &p) {
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-        const float a = fabsf(z[c]);
-        s = s + a;
-        p = p * (1.0f + expf(-2.0f * a));
+        s = s + a[c];
+        p = p * f[c];
     }
 }
 
@@ -233,12 +232,18 @@ __global__ __launch_bounds__(256) void project_kernel(ProjectArgs a) {
                 // compute_code_score/torch_extension.cc:31-37.
                 const int nib = (z[0] > 0.f ? 8 : 0) | (z[1] > 0.f ? 4 : 0) |
                                 (z[2] > 0.f ? 2 : 0) | (z[3] > 0.f ? 1 : 0);
+                float az[4], fz[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    az[c] = fabsf(z[c]);
+                    fz[c] = 1.0f + expf(-2.0f * az[c]);
+                }
                 float s_loc = 0.f, p_loc = 1.f;
-                score_chain(z, s_loc, p_loc);
+                score_chain(az, fz, s_loc, p_loc);                 // what an even lane hands over
                 float s_run = lane_xor<1>(s_loc);
                 float p_run = lane_xor<1>(p_loc);
                 const int nib_hi = __float_as_int(lane_xor<1>(__int_as_float(nib)));
-                score_chain(z, s_run, p_run);
+                score_chain(az, fz, s_run, p_run);                 // an odd lane continues from there
                 const int t = col >> 3;
                 if (live && (lr & 1) && t < a.T) {
                     a.codes[row * a.T + t] = (nib_hi << 4) | nib;

@@ -134,3 +134,54 @@ def test_ops_have_fake_implementations():
     t = torch.empty(8, 256, 64, device="meta")
     assert torch.ops.lookupffn.lookup_gather(c, s, t, None).shape == (5, 64)
     assert torch.ops.lookupffn.fht(torch.empty(3, 64, device="meta")).shape == (3, 64)
+
+
+def _encoder_config(**kw):
+    base = dict(hidden_size=64, num_attention_heads=4, attention_head_size=16, attention_probs_dropout_prob=0.1,
+                hidden_dropout_prob=0.1, layer_norm_eps=1e-5, num_hidden_layers=2, vocab_size=100,
+                max_position_embeddings=32, type_vocab_size=1, pad_token_id=1,
+                ffn_num_table=8, ffn_table_size=256, projection_type="bh4", block_size=1)
+    base.update(kw)
+    return Namespace(**base)
+
+
+def test_encoder_parameter_names_match_reference():
+    # names a reference checkpoint of PL/encoder.py's Lookup model carries (after the
+    # "model." prefix is stripped, roberta_to_hf_checkpoint.py:102-111)
+    m = lookupffn_amd.Lookup(_encoder_config())
+    keys = set(m.state_dict())
+    for k in ["embeddings.word_embeddings.weight", "embeddings.position_embeddings.weight",
+              "embeddings.token_type_embeddings.weight", "embeddings.LayerNorm.weight",
+              "encoder.LayerNorm.bias", "encoder.layer.0.attention.LayerNorm.weight",
+              "encoder.layer.0.attention.query.weight", "encoder.layer.0.attention.key.bias",
+              "encoder.layer.0.attention.value.weight", "encoder.layer.0.attention.dense.weight",
+              "encoder.layer.1.FFN.LayerNorm.weight", "encoder.layer.1.FFN.hash.projection.weight",
+              "encoder.layer.1.FFN.hash.projection.bias", "encoder.layer.1.FFN.tables", "encoder.layer.1.FFN.bias"]:
+        assert k in keys, k
+    assert tuple(m.state_dict()["embeddings.position_embeddings.weight"].shape) == (34, 64)   # max_position + 2
+    assert len(keys) == 5 + 2 + 2 * (2 + 8 + 6)
+
+
+def test_attention_fused_equals_literal_formula_on_cpu():
+    # the attention block is plain torch and runs anywhere; the fused evaluation must
+    # equal the reference's literal matmul-softmax-matmul (PL/layer.py:55-64)
+    torch.manual_seed(0)
+    cfg = _encoder_config()
+    att = lookupffn_amd.Attention(cfg).eval().double()
+    x = torch.randn(3, 10, 64, dtype=torch.float64)
+    mask = torch.ones(3, 10)
+    mask[1, 7:] = 0
+    att.fused = True
+    a = att(x, mask)
+    att.fused = False
+    b = att(x, mask)
+    # the module computes attention in float32 whatever the input dtype, as the reference does
+    assert torch.allclose(a, b, rtol=1e-5, atol=1e-6)
+    emb = lookupffn_amd.RobertaEmbeddings(cfg).eval()
+    ids = torch.randint(0, 100, (2, 5))
+    pos = torch.arange(5)[None].expand(2, 5)
+    out = emb(ids, torch.zeros_like(ids), pos)
+    want = torch.nn.functional.layer_norm(
+        emb.word_embeddings.weight[ids] + emb.token_type_embeddings.weight[0] + emb.position_embeddings.weight[pos + 2],
+        (64,), emb.LayerNorm.weight, emb.LayerNorm.bias, 1e-5)
+    assert torch.allclose(out, want, atol=1e-6)

@@ -192,3 +192,53 @@ def test_reference_call_sequence_of_lookup_gather():
         a = layer.gather(code, score, layer.tables) + layer.bias
         b = lookupffn_amd.lookup_gather(code, score, layer.tables, layer.bias)
     assert relmax(npf(a), npf(b)) <= 1e-6
+
+
+def test_encoder_layers_match_float64_composition():
+    """The pre-norm encoder with LookupFFN (PL/layer.py:66-78, PL/encoder.py:9-37): each
+    layer's output on the GPU against attention evaluated in float64 with the literal
+    formula plus the oracle's LookupFFN, from the GPU's own layer input (so that a code
+    flip in one layer does not compound)."""
+    torch.manual_seed(11)
+    cfg = Namespace(hidden_size=64, num_attention_heads=4, attention_head_size=16, attention_probs_dropout_prob=0.1,
+                    hidden_dropout_prob=0.1, layer_norm_eps=1e-5, num_hidden_layers=3, vocab_size=100,
+                    max_position_embeddings=32, type_vocab_size=1, pad_token_id=1,
+                    ffn_num_table=8, ffn_table_size=256, projection_type="bh4", block_size=1)
+    model = lookupffn_amd.Lookup(cfg).eval().to(DEV)
+    Bq, L = 4, 24
+    ids = torch.randint(0, 100, (Bq, L), device=DEV)
+    pos = torch.arange(L, device=DEV)[None].expand(Bq, L)
+    mask = torch.ones(Bq, L, device=DEV)
+    mask[2, 20:] = 0
+    with torch.no_grad():
+        out, extra = model(ids, torch.zeros_like(ids), pos, mask)
+        assert extra == {} and out.shape == (Bq, L, 64)
+        h = model.embeddings(ids, torch.zeros_like(ids), pos)
+        for layer in model.encoder.layer:
+            got = layer(h, mask)
+            # float64 reference of this layer from the same input
+            ref = lookupffn_amd.EncoderLayer.__new__(lookupffn_amd.EncoderLayer)
+            att = layer.attention
+            x64 = h.double().cpu()
+            a = torch.nn.functional.layer_norm(x64, (64,), att.LayerNorm.weight.double().cpu(),
+                                               att.LayerNorm.bias.double().cpu(), 1e-5)
+            def heads(t):
+                return t.view(Bq, L, 4, 16).permute(0, 2, 1, 3)
+            lin = lambda m, t: t @ m.weight.double().cpu().T + m.bias.double().cpu()
+            q, k, v = heads(lin(att.query, a)), heads(lin(att.key, a)), heads(lin(att.value, a))
+            bias = -1000.0 * (1.0 - mask.double().cpu()[:, None, None, :])
+            probs = torch.softmax(q @ k.transpose(-1, -2) / 4.0 + bias, dim=-1)
+            ctx = (probs @ v).permute(0, 2, 1, 3).reshape(Bq, L, 64)
+            attn_out = lin(att.dense, ctx) + x64
+            ffn = layer.FFN
+            p = ffn.hash.projection
+            y, _, code64, _ = oracle.lookup_ffn(
+                attn_out.reshape(-1, 64).numpy(), npf(ffn.LayerNorm.weight), npf(ffn.LayerNorm.bias), 1e-5,
+                npf(p.weight), npf(p.bias), npf(ffn.tables), npf(ffn.bias), decay=0.7, return_parts=True)
+            want = y + attn_out.reshape(-1, 64).numpy()
+            err = np.abs(npf(got).reshape(-1, 64) - want).max(axis=1) / np.abs(want).max()
+            # tokens whose hash codes are the same in float32 and float64 agree closely;
+            # at most a few tokens sit on a sign boundary of the projection
+            assert (err <= 5e-5).mean() >= 0.9, err
+            h = got
+        assert relmax(npf(model.encoder.LayerNorm(h)), npf(out)) <= 1e-6
