@@ -54,7 +54,7 @@ WORKLOADS = {
 # HBM bytes per launch of the gather kernel measured with rocprofv3 --pmc
 # (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); the summaries
 # are kept under profiles/.  None until measured for that workload.
-MEASURED_TRAFFIC_BYTES = {"cfg2": 454936243, "cfg3": 2865333908, "cfg3bf16": 1397976562}
+MEASURED_TRAFFIC_BYTES = {"cfg2": 477412788, "cfg3": 3169016070, "cfg3bf16": 2250808112, "cfg5": 504127966}
 
 
 def build_layer(wl, device):
@@ -125,6 +125,17 @@ def cpu_baseline(layer, x, wl, budget_s=12.0):
     return out
 
 
+def calibrate_copy(dev):
+    """One plain 1 GiB device-to-device copy: a kernel of known traffic for scaling
+    FETCH_SIZE / WRITE_SIZE in a rocprofv3 --pmc run of this command."""
+    import torch
+    src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+    dst = torch.empty_like(src)
+    dst.copy_(src)                 # reads 1 GiB, writes 1 GiB
+    torch.cuda.synchronize()
+    del src, dst
+
+
 def zipf_codes(B, T, S, gen, s=1.1):
     """Per (token, table) a rank drawn with p_r ~ r^-s, mapped to a table entry by a
     fixed seeded permutation per table."""
@@ -176,6 +187,8 @@ def main_backward(args):
         g_h = (ops.bh4_diag((p.decay_coeff * g_z).contiguous(), diag_t) * d0 + (1 - p.decay_coeff) * g_z)[:, :H]
         return g_score, g_tables, g_z, g_h
 
+    if args.calibrate_copy:
+        calibrate_copy(dev)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -210,7 +223,8 @@ def main_backward(args):
                    "step": "inner product (grad score) + scatter-add (grad tables) + score "
                            "derivative + transposed BH4(block 1)x4"},
         "roofline": {"bound": "hbm", "kernel": "lookup_scatter", "achieved": achieved,
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get("cfg5"),
                      "algorithmic_bytes": scatter_bytes, "avg_kernel_ms": scatter_ms},
         "stages_ms": {"indexed_inner_product": inner_ms, "scatter_add": scatter_ms, "code_score_bwd": bwd_score_ms},
     }
@@ -366,11 +380,7 @@ def main():
         assert torch.equal(step(), layer(x)), "bench step and LookupFFN.forward disagree"
 
     if args.calibrate_copy:
-        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
-        dst = torch.empty_like(src)
-        dst.copy_(src)                 # reads 1 GiB, writes 1 GiB
-        torch.cuda.synchronize()
-        del src, dst
+        calibrate_copy(dev)
 
     for _ in range(args.warmup):
         step()
