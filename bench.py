@@ -167,8 +167,8 @@ def main_backward(args):
     g_out_cpu = torch.randn(B, Do, generator=g)
     score_cpu = 1.0 - torch.rand(B, T, generator=g)
     code, z, g_out, score = code_cpu.to(dev), z_cpu.to(dev), g_out_cpu.to(dev), score_cpu.to(dev)
-    idx = code + torch.arange(T, device=dev, dtype=torch.int32)[None] * S
-    flat = layer.tables.detach().reshape(T * S, Do)
+    tables = layer.tables.detach()
+    flat = tables.reshape(T * S, Do)
     p = layer.hash.projection
     D = p.padded_in_dim
     diag = p.weight.detach().reshape(1, 4, D)
@@ -177,7 +177,7 @@ def main_backward(args):
     d0 = diag[0, 0].contiguous()
 
     def step(events=None):
-        g_score = ops.indexed_inner_product(idx, g_out, flat)
+        g_score = ops.lookup_inner(code, g_out, tables)
         if events is not None:
             events[0].record()
         g_tables = ops.lookup_scatter(code, score, g_out, S)
@@ -210,8 +210,8 @@ def main_backward(args):
             fn()
         b.record(); torch.cuda.synchronize()
         return a.elapsed_time(b) / n
-    inner_ms = timed(lambda: ops.indexed_inner_product(idx, g_out, flat))
-    g_score = ops.indexed_inner_product(idx, g_out, flat)
+    inner_ms = timed(lambda: ops.lookup_inner(code, g_out, tables))
+    g_score = ops.lookup_inner(code, g_out, tables)
     bwd_score_ms = timed(lambda: ops.code_score_bwd(z, g_score))
 
     res = {
@@ -226,13 +226,14 @@ def main_backward(args):
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get("cfg5"),
                      "algorithmic_bytes": scatter_bytes, "avg_kernel_ms": scatter_ms},
-        "stages_ms": {"indexed_inner_product": inner_ms, "scatter_add": scatter_ms, "code_score_bwd": bwd_score_ms},
+        "stages_ms": {"lookup_inner": inner_ms, "scatter_add": scatter_ms, "code_score_bwd": bwd_score_ms},
     }
     if not args.no_cpu_baseline:
         import oracle
         n = 1024
         npf = lambda t: t.detach().float().cpu().numpy()
-        idx_n, g_n, w_n, z_n = npf(idx[:n]).astype(np.int32), npf(g_out[:n]), npf(score[:n]), npf(z[:n])
+        idx_n = (code[:n] + torch.arange(T, device=dev, dtype=torch.int32)[None] * S).cpu().numpy().astype(np.int32)
+        g_n, w_n, z_n = npf(g_out[:n]), npf(score[:n]), npf(z[:n])
         flat_n = npf(flat)
         reps, tt = 0, 0.0
         while reps < 2 or (tt < 10.0 and reps < 1000):

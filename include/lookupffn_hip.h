@@ -226,6 +226,20 @@ int lffn_scatter_add_f32(const int32_t *idx, const float *g, const float *w, flo
 int lffn_lookup_scatter_f32(const int32_t *code, const float *score, const float *g, float *grad_tables,
                             int64_t B, int64_t T, int64_t S, int64_t Do, int32_t accumulate, void *stream);
 
+/*
+ * The indexed inner product as the layer's backward issues it: table-local codes,
+ *   grad_score[b, t] = < g[b, :], tables[t, code[b,t] & (S-1), :] >
+ * code: [B, T] int32; g: [B, Do]; tables: [T, S, Do] fp32; grad_score: [B, T],
+ * overwritten (it needs no zero-fill).  For S <= 256 the table slices are staged
+ * in LDS and the partial sums of the 64-column slices of a row are combined with
+ * global atomics, in no fixed order (as the partial sums of the reference's
+ * kernel are, PL/gather/cuda/extension/gather_kernel_fp32.cu:141).
+ * Replaces WeightedVectorGatherAdd.backward's indexed_inner_product call
+ * (PL/gather/cuda/kernel.py:199) together with the index offset of PL/lookup.py:126.
+ */
+int lffn_lookup_inner_f32(const int32_t *code, const float *g, const float *tables, float *grad_score,
+                          int64_t B, int64_t T, int64_t S, int64_t Do, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -403,6 +403,16 @@ int lffn_internal_lookup_scatter_atomic(const int32_t *code, const float *score,
     return launch<false, Op::Scatter>(a, static_cast<hipStream_t>(stream));
 }
 
+// Token-major inner product on table-local codes: the fallback of lookup_inner.hip.
+int lffn_internal_lookup_inner_token_major(const int32_t *code, const float *g, const float *tables,
+                                           float *out, int64_t B, int64_t T, int64_t S, int64_t Do,
+                                           void *stream) {
+    GatherArgs a{};
+    a.idx = code; a.src = tables; a.w = nullptr; a.g = g; a.bias = nullptr; a.out = out;
+    a.B = B; a.I = (int)T; a.source_size = T * S; a.Dv = (int)Do; a.S = (int)S;
+    return launch<false, Op::Inner>(a, static_cast<hipStream_t>(stream));
+}
+
 extern "C" int lffn_indexed_inner_product_f32(const int32_t *idx, const float *g, const float *src, float *out,
                                               int64_t B, int64_t I, int64_t source_size, int64_t Dv, void *stream) {
     int rc = check_common(idx, B, I, source_size, Dv);

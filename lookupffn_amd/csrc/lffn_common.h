@@ -35,6 +35,12 @@ __attribute__((visibility("hidden")))
 int lffn_internal_lookup_scatter_atomic(const int32_t *code, const float *score, const float *g, float *out,
                                         int64_t B, int64_t T, int64_t S, int64_t Do, void *stream);
 
+// gather.hip: token-major indexed inner product on table-local codes (not exported)
+__attribute__((visibility("hidden")))
+int lffn_internal_lookup_inner_token_major(const int32_t *code, const float *g, const float *tables,
+                                           float *out, int64_t B, int64_t T, int64_t S, int64_t Do,
+                                           void *stream);
+
 // lookup_gather_pair.hip: the two-tables-per-buffer LDS gather (not exported)
 __attribute__((visibility("hidden")))
 int lffn_internal_lookup_gather_pair(const int32_t *code, const float *score, const void *tables,

@@ -147,9 +147,7 @@ class LookupGather(Function):
             raise NotImplementedError("backward through bfloat16 tables is not built (inference format)")
         grad_outputs = grad_outputs.contiguous()
         T, S, Do = tables.shape
-        idx = (code & (S - 1)) + torch.arange(T, device=code.device, dtype=code.dtype)[None] * S
-        flat = tables.reshape(T * S, Do)
-        grad_score = ops.indexed_inner_product(idx, grad_outputs, flat) if ctx.needs_input_grad[1] else None
+        grad_score = ops.lookup_inner(code, grad_outputs, tables) if ctx.needs_input_grad[1] else None
         grad_tables = ops.lookup_scatter(code, score, grad_outputs, S) if ctx.needs_input_grad[2] else None
         grad_bias = grad_outputs.sum(dim=0) if (ctx.has_bias and ctx.needs_input_grad[3]) else None
         return None, grad_score, grad_tables, grad_bias

@@ -370,6 +370,33 @@ def _(code, score, g, S):
     return g.new_empty(code.shape[1], S, g.shape[1])
 
 
+_L.define("lookup_inner(Tensor code, Tensor g, Tensor tables) -> Tensor")
+
+
+def _lookup_inner_impl(code, g, tables):
+    _lib.require_gpu(code, g, tables)
+    assert g.dim() == 2 and g.dtype == torch.float32 and g.is_contiguous()
+    assert tables.dim() == 3 and tables.dtype == torch.float32 and tables.is_contiguous()
+    B, T = code.shape
+    Tt, S, Do = tables.shape
+    assert Tt == T and g.shape[0] == B and g.shape[1] == Do and _is_pow2(S)
+    _check_gather_args(code, max(T * S, 1), Do)
+    out = torch.empty(B, T, dtype=torch.float32, device=g.device)     # fully overwritten by the kernels
+    with _dev_guard(g):
+        rc = _lib.load().lffn_lookup_inner_f32(_lib.ptr(code), _lib.ptr(g), _lib.ptr(tables), _lib.ptr(out),
+                                               B, T, S, Do, _lib.stream_of(g))
+    _lib.check(rc, f"lffn_lookup_inner_f32(B={B}, T={T}, S={S}, Do={Do})")
+    return out
+
+
+_L.impl("lookup_inner", _lookup_inner_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::lookup_inner")
+def _(code, g, tables):
+    return g.new_empty(code.shape[0], code.shape[1])
+
+
 fht = torch.ops.lookupffn.fht
 bh4_diag = torch.ops.lookupffn.bh4_diag
 project_hash = torch.ops.lookupffn.project_hash
@@ -381,3 +408,4 @@ lookup_gather = torch.ops.lookupffn.lookup_gather
 indexed_inner_product = torch.ops.lookupffn.indexed_inner_product
 scatter_add = torch.ops.lookupffn.scatter_add
 lookup_scatter = torch.ops.lookupffn.lookup_scatter
+lookup_inner = torch.ops.lookupffn.lookup_inner

@@ -156,3 +156,12 @@ def lookup_scatter(code, score, g, S, accumulate=False, init=None):
         out = dev(init)
     _call("lffn_lookup_scatter_f32", p(cd), p(sd), p(gd), p(out), B, T, S, Do, 1 if accumulate else 0)
     return host(out)
+
+
+def lookup_inner(code, g, tables):
+    cd, gd, td = dev(code), dev(g), dev(tables)
+    B, T = code.shape
+    _, S, Do = tables.shape
+    out = torch.full((B, T), float("nan"), dtype=torch.float32, device=DEV)   # must be fully overwritten
+    _call("lffn_lookup_inner_f32", p(cd), p(gd), p(td), p(out), B, T, S, Do)
+    return host(out)

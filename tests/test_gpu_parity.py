@@ -479,6 +479,52 @@ def test_lookup_scatter_full_size_zipf_properties():
     assert abs(lhs - rhs) <= 1e-5 * max(abs(lhs), 1.0) * 10
 
 
+# (B, T, S, Do): the LDS kernel needs ceil(B/256) * Do/64 >= 192 units, T >= 4 and S <= 256; the
+# first rows take it with each token tile (832, 512, 256 tokens), ragged token counts, table counts
+# that are no multiple of the 16-table chunk and tables smaller than the LDS slice; the rest fall
+# back to the token-major kernel
+INNER_CASES = [(16384, 20, 256, 768), (4100, 17, 256, 768), (3000, 5, 64, 1024), (12289, 33, 16, 768),
+               (8191, 16, 256, 1536), (8191, 9, 128, 768), (256, 32, 256, 256), (1, 2, 4, 64), (65, 5, 256, 192),
+               (500, 4, 512, 128), (2000, 3, 256, 1024), (0, 4, 16, 64)]
+
+
+@pytest.mark.parametrize("B,T,S,Do", INNER_CASES)
+def test_lookup_inner_matches_oracle(B, T, S, Do):
+    rng = np.random.RandomState(B + T + S + Do + 1)
+    tables, code, idx, _ = _rand_gather(rng, B, T, S, Do)
+    g = rng.randn(B, Do).astype(np.float32)
+    got = cabi.lookup_inner(code, g, tables)
+    if B == 0:
+        assert got.shape == (0, T)
+        return
+    assert not np.isnan(got).any()                      # every entry written
+    want = oracle.indexed_inner_product(idx, g.astype(np.float64), tables.reshape(T * S, Do).astype(np.float64))
+    assert relmax(got, want) <= 1e-5
+    # the same numbers as the flat-index entry point, up to the order of the additions
+    assert relmax(got, cabi.indexed_inner_product(idx, g, tables.reshape(T * S, Do))) <= 1e-5
+    # codes are masked into their table; a second call overwrites the first result
+    dirty = (code + S * rng.randint(0, 4, size=code.shape)).astype(np.int32)
+    assert relmax(cabi.lookup_inner(dirty, g, tables), want) <= 1e-5
+
+
+def test_lookup_inner_full_size_duality():
+    # BASELINE config 2 shape: <G(w), g> = sum_bt w[b,t] * grad_score[b,t], and linearity in g
+    rng = np.random.RandomState(43)
+    B, T, S, Do = 16384, 128, 256, 768
+    tables, code, idx, w = _rand_gather(rng, B, T, S, Do)
+    g = rng.randn(B, Do).astype(np.float32)
+    got = cabi.lookup_inner(code, g, tables)
+    fwd = cabi.lookup_gather(code, w, tables, None)
+    lhs = float((fwd.astype(np.float64) * g).sum())
+    rhs = float((got.astype(np.float64) * w).sum())
+    assert abs(lhs - rhs) <= 1e-5 * max(abs(lhs), 1.0) * 10
+    sub = slice(5000, 5200)
+    want = oracle.indexed_inner_product(idx[sub], g[sub].astype(np.float64),
+                                        tables.reshape(T * S, Do).astype(np.float64))
+    assert relmax(got[sub], want) <= 1e-5
+    assert relmax(cabi.lookup_inner(code, 2.0 * g, tables), 2.0 * got.astype(np.float64)) <= 1e-6
+
+
 def test_scatter_duplicates_zipf():
     # heavy duplication of rows (BASELINE config 5 draws codes Zipf(1.1))
     rng = np.random.RandomState(40)
