@@ -16,6 +16,14 @@
 // the workgroups arrive (the reference's kernel, PL/gather/cuda/extension/gather_kernel_fp32.cu:141,
 // also combines its partial sums with atomics).  grad_score must be zero when the
 // kernel starts; the entry point clears it first.
+//
+// Measured at 16384 tokens x 128 tables x 256 x 768 (MI355X): 255 us, of which about
+// 35 us are the atomics.  Summing four tokens' partial products together with a
+// lane-transposing reduction (12 instead of 20 vector instructions per four sums)
+// and requesting the LDS rows of the next pass group ahead of time both left the
+// time unchanged: with 832 tokens a tile the table time is the slice copy
+// (about 1.1 us for 64 KB per compute unit) plus the part of the arithmetic that
+// does not overlap with it.
 #include "lffn_common.h"
 
 #include <hip/amd_detail/amd_hip_unsafe_atomics.h>
