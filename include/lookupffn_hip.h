@@ -69,6 +69,25 @@ int lffn_bh4_diag_f32(const float *x, const float *diag, float *out,
                       int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, void *stream);
 
 /*
+ * BH4 mixing with 64 x 64 blocks, all stages of a repeat in one kernel:
+ *   for r < R:  y = pad(x);  for j < J:  y = FHT(blockdiag(w[r,j]) y);  out[b, r*D:(r+1)*D] = y
+ * x: [B, H], H <= D, H % 4 == 0 (zero-padded on load, PL/lookup.py:32-34);
+ * out: [B, R*D]; D = 64 * num_block a power of two, 64 <= D <= 1024; block_size must be 64.
+ * The 64-point part of every transform is applied to the weights beforehand:
+ * lffn_bh4_fold_f32 turns w [R, J, num_block, 64, 64] (PL/lookup.py:22) into
+ * w_folded (same shape, caller-allocated, must not alias w), which
+ * lffn_bh4_block_f32 takes.  Fold again whenever w changes.  The products run on
+ * the fp32 matrix cores; results agree with "product, then transform" to fp32
+ * rounding, not bit for bit.
+ * Replaces bh4_cuda (PL/bh4/kernel.py:23-36): the einsum "bni,noi->bno" (":32")
+ * and hadamard (":34") of every stage.
+ */
+int lffn_bh4_fold_f32(const float *w, float *w_folded, int64_t R, int64_t J, int64_t num_block,
+                      int64_t block_size, void *stream);
+int lffn_bh4_block_f32(const float *x, const float *w_folded, float *out, int64_t B, int64_t H,
+                       int64_t D, int64_t R, int64_t J, int64_t block_size, void *stream);
+
+/*
  * The whole hashing front-end of the layer in one pass over x, for block size 1
  * and 8-bit codes (PL/lookup.py:29-39,64-77 + PL/compute_code_score/kernel.py:43-55):
  *   y      = bh4_diag(x)                                   (as above)

@@ -30,6 +30,8 @@ _f32 = ctypes.c_float
 SIGNATURES = {
     "lffn_fht_f32": [_vp, _vp, _i64, _i64, _vp],
     "lffn_bh4_diag_f32": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp],
+    "lffn_bh4_fold_f32": [_vp, _vp, _i64, _i64, _i64, _i64, _vp],
+    "lffn_bh4_block_f32": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp],
     "lffn_project_hash_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _vp],
     "lffn_ln_project_hash_f32": [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _vp,
                                  _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _vp],

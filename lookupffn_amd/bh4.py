@@ -99,8 +99,9 @@ def hadamard(inp, use_torch=False):
 def bh4_cuda(x, w):
     """PL/bh4/kernel.py:23-36.  w: [R, 4, D/bs, bs, bs].
 
-    Block size 1 without autograd runs as one fused kernel (all stages and
-    repeats in registers).  Otherwise each stage is the block-diagonal product
+    Without autograd, block size 1 runs as one fused kernel (all stages and
+    repeats in registers) and block size 64 (D <= 1024) as a weight-folding
+    kernel plus one fused matrix-core kernel.  Otherwise each stage is the block-diagonal product
     followed by the transform kernel, differentiable through
     ``FastHadamardTransform``."""
     BS = w.shape[-1]
@@ -109,6 +110,8 @@ def bh4_cuda(x, w):
     needs_grad = torch.is_grad_enabled() and (x.requires_grad or w.requires_grad)
     if BS == 1 and not needs_grad and x.dtype == torch.float32:
         return ops.bh4_diag(x.contiguous(), w.reshape(w.shape[0], w.shape[1], D).contiguous())
+    if BS == 64 and D <= 1024 and not needs_grad and x.dtype == torch.float32:
+        return ops.bh4_block(x.contiguous(), ops.bh4_fold(w.contiguous()))
     out = []
     for i in range(w.shape[0]):
         y = x

@@ -1,0 +1,222 @@
+// BH4 with 64x64 blocks (PL/bh4/kernel.py:23-36), all stages of a repeat in one kernel:
+//
+//   y <- pad(x);  for s < J:  y <- FHT_D( blockdiag(W[r,s]) y );   out[:, r*D:(r+1)*D] = y
+//
+// D = 64*NB.  In natural (Sylvester) order H_D = H_NB (x) H_64 with the block number
+// as the high index bits, so a stage is  (H_NB (x) I_64) * blockdiag(H_64 W[r,s,n]):
+// the 64-point part of the transform is folded into the weights once per call
+// (lffn_bh4_fold_f32, a 64-point transform down the output index of every 64x64
+// block), and the part across blocks is NB-point butterflies between accumulators.
+//
+// One workgroup = 4 wavefronts = 32 tokens, whose rows stay in LDS between the
+// stages ((D+4)-float rows: conflict-free 16-byte accesses down a column of
+// tokens).  Wavefront w owns output columns [16w, 16w+16) of every block for both
+// 16-token halves, so a weight fragment fetched from L2 is used for 32 tokens.  The
+// products run on v_mfma_f32_16x16x4_f32 with the weights as the A operand
+// (rows = output columns) and the tokens as the B operand, which leaves each lane
+// with four consecutive output columns of one token: one 16-byte LDS store per
+// (block, half).  2*NB accumulator tiles per wavefront; the butterflies across
+// blocks are register adds.
+//
+// Rounding differs from doing the product first and the full transform after it
+// (the reference's order): the 64-point part is applied to the weights, in fp32,
+// before the product.  Results agree to fp32 rounding (1e-5 of the row's largest
+// magnitude), not bit for bit.
+#include "lffn_common.h"
+
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int BS = 64;          // block size this file is built for
+constexpr int TOK = 32;         // tokens per workgroup
+constexpr int PAD = 4;          // floats of padding per LDS row
+
+// 64-point unnormalised Hadamard transform down the output index o of every block:
+// wf[blk][o'][i] = sum_o H64[o'][o] * w[blk][o][i].  One lane per (blk, i).
+__global__ __launch_bounds__(256) void bh4_fold_kernel(const float *w, float *wf, int64_t nblk) {
+    const int64_t gid = int64_t(blockIdx.x) * 256 + threadIdx.x;
+    if (gid >= nblk * BS) return;
+    const int64_t blk = gid / BS;
+    const int i = (int)(gid % BS);
+    const float *src = w + blk * (BS * BS) + i;
+    float v[BS];
+#pragma unroll
+    for (int o = 0; o < BS; ++o) v[o] = src[o * BS];
+#pragma unroll
+    for (int h = BS / 2; h >= 1; h >>= 1) {
+#pragma unroll
+        for (int o = 0; o < BS; ++o) {
+            if ((o & h) == 0) {
+                const float lo = v[o], hi = v[o + h];
+                v[o] = lo + hi;
+                v[o + h] = lo - hi;
+            }
+        }
+    }
+    float *dst = wf + blk * (BS * BS) + i;
+#pragma unroll
+    for (int o = 0; o < BS; ++o) dst[o * BS] = v[o];
+}
+
+template <int NB>
+__global__ __launch_bounds__(256) void bh4_block_kernel(const float *__restrict__ x, const float *__restrict__ wf,
+                                                        float *__restrict__ out, int64_t B, int H, int R,
+                                                        int J) {
+    constexpr int D = BS * NB;
+    constexpr int LDR = D + PAD;
+    extern __shared__ float xs[];                 // TOK rows of LDR floats
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;                    // output columns [16*wave, 16*wave + 16) of each block
+    const int c = lane & 15;                      // A operand: output column; B operand and result: token
+    const int kq = lane >> 4;                     // k index inside an MFMA; result: output columns 4*kq .. 4*kq+3
+    const int64_t tok_base = int64_t(blockIdx.x) * TOK;
+
+    // this lane's weight fragment of block n: wf[..][n][16*wave + c][16*kq .. 16*kq + 15]
+    const int w_lane_off = (16 * wave + c) * BS + 16 * kq;
+    // this lane's token values of block n, half h: xs[(16*h + c) * LDR + 64*n + 16*kq ..]
+    const int x_lane_off = c * LDR + 16 * kq;
+    // where this lane's results of block n, half h go: xs[(16*h + c) * LDR + 64*n + 16*wave + 4*kq ..]
+    const int y_lane_off = c * LDR + 16 * wave + 4 * kq;
+
+    for (int r = 0; r < R; ++r) {
+        __syncthreads();                          // the previous repeat's last stage has been read
+        for (int e = tid; e < TOK * (D / 4); e += 256) {
+            const int row = e / (D / 4), col = (e % (D / 4)) * 4;
+            const int64_t tok = tok_base + row;
+            const float4 v = (tok < B && col < H) ? *reinterpret_cast<const float4 *>(x + tok * H + col)
+                                                  : make_float4(0.f, 0.f, 0.f, 0.f);      // zero padding to D
+            *reinterpret_cast<float4 *>(xs + row * LDR + col) = v;
+        }
+        __syncthreads();
+
+#pragma unroll 1
+        for (int s = 0; s < J; ++s) {
+            const float *wst = wf + (size_t)((r * J + s) * NB) * (BS * BS) + w_lane_off;
+            f32x4 acc[2][NB];
+#pragma unroll
+            for (int n = 0; n < NB; ++n) {
+                acc[0][n] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                acc[1][n] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            }
+            // weight fragments two blocks ahead of their use
+            float4 wq[3][4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                wq[0][q] = *reinterpret_cast<const float4 *>(wst + q * 4);
+                if (NB > 1) wq[1][q] = *reinterpret_cast<const float4 *>(wst + BS * BS + q * 4);
+            }
+            static_for<NB>([&](auto n_c) {
+                constexpr int n = decltype(n_c)::value;
+                if constexpr (n + 2 < NB) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        wq[(n + 2) % 3][q] = *reinterpret_cast<const float4 *>(wst + (n + 2) * (BS * BS) + q * 4);
+                }
+                float4 xa[4], xb[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    xa[q] = *reinterpret_cast<const float4 *>(xs + x_lane_off + n * BS + q * 4);
+                    xb[q] = *reinterpret_cast<const float4 *>(xs + 16 * LDR + x_lane_off + n * BS + q * 4);
+                }
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float4 wv = wq[n % 3][q];
+                    acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv.x, xa[q].x, acc[0][n], 0, 0, 0);
+                    acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv.x, xb[q].x, acc[1][n], 0, 0, 0);
+                    acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv.y, xa[q].y, acc[0][n], 0, 0, 0);
+                    acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv.y, xb[q].y, acc[1][n], 0, 0, 0);
+                    acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv.z, xa[q].z, acc[0][n], 0, 0, 0);
+                    acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv.z, xb[q].z, acc[1][n], 0, 0, 0);
+                    acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv.w, xa[q].w, acc[0][n], 0, 0, 0);
+                    acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv.w, xb[q].w, acc[1][n], 0, 0, 0);
+                }
+            });
+
+            // H_NB across the blocks
+#pragma unroll
+            for (int h = NB / 2; h >= 1; h >>= 1) {
+#pragma unroll
+                for (int n = 0; n < NB; ++n) {
+                    if ((n & h) == 0) {
+#pragma unroll
+                        for (int t = 0; t < 2; ++t) {
+                            const f32x4 lo = acc[t][n], hi = acc[t][n + h];
+                            acc[t][n] = lo + hi;
+                            acc[t][n + h] = lo - hi;
+                        }
+                    }
+                }
+            }
+
+            __syncthreads();                      // every wavefront has read this stage's input
+            if (s + 1 < J) {
+#pragma unroll
+                for (int n = 0; n < NB; ++n) {
+                    *reinterpret_cast<f32x4 *>(xs + y_lane_off + n * BS) = acc[0][n];
+                    *reinterpret_cast<f32x4 *>(xs + 16 * LDR + y_lane_off + n * BS) = acc[1][n];
+                }
+                __syncthreads();
+            } else {
+                const int64_t ld_out = int64_t(R) * D;
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const int64_t tok = tok_base + 16 * t + c;
+                    if (tok < B) {
+                        float *o = out + tok * ld_out + (size_t)r * D + 16 * wave + 4 * kq;
+#pragma unroll
+                        for (int n = 0; n < NB; ++n) *reinterpret_cast<f32x4 *>(o + n * BS) = acc[t][n];
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <int NB>
+int launch_block(const float *x, const float *wf, float *out, int64_t B, int H, int R, int J, hipStream_t st) {
+    const size_t lds_bytes = size_t(TOK) * (BS * NB + PAD) * sizeof(float);
+    auto kern = bh4_block_kernel<NB>;
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds_bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        return LFFN_ERR_LAUNCH;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)((B + TOK - 1) / TOK)), dim3(256), lds_bytes, st, x, wf, out, B, H, R, J);
+    return lffn_launch_status();
+}
+
+}  // namespace
+
+extern "C" int lffn_bh4_fold_f32(const float *w, float *w_folded, int64_t R, int64_t stages, int64_t num_block,
+                                 int64_t block_size, void *stream) {
+    LFFN_REQUIRE(R >= 1 && stages >= 1 && num_block >= 1, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(block_size == BS, LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(w && w_folded && w != w_folded, LFFN_ERR_BAD_ARG);
+    const int64_t nblk = R * stages * num_block;
+    LFFN_REQUIRE(nblk <= (int64_t(1) << 24), LFFN_ERR_UNSUPPORTED);
+    hipLaunchKernelGGL(bh4_fold_kernel, dim3((unsigned)((nblk * BS + 255) / 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), w, w_folded, nblk);
+    return lffn_launch_status();
+}
+
+extern "C" int lffn_bh4_block_f32(const float *x, const float *w_folded, float *out, int64_t B, int64_t H,
+                                  int64_t D, int64_t R, int64_t J, int64_t block_size, void *stream) {
+    LFFN_REQUIRE(B >= 0 && R >= 1 && J >= 1 && D >= 1 && H >= 1 && H <= D, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(H % 4 == 0 && J <= 64, LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(block_size == BS && lffn_is_pow2(D) && D >= BS && D <= 1024, LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(R <= 4096 && B <= (int64_t(1) << 31) - 1, LFFN_ERR_UNSUPPORTED);
+    if (B == 0) return LFFN_OK;
+    LFFN_REQUIRE(x && w_folded && out, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_aligned16(x) && lffn_aligned16(w_folded) && lffn_aligned16(out), LFFN_ERR_BAD_ARG);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (D / BS) {
+        case 1: return launch_block<1>(x, w_folded, out, B, (int)H, (int)R, (int)J, st);
+        case 2: return launch_block<2>(x, w_folded, out, B, (int)H, (int)R, (int)J, st);
+        case 4: return launch_block<4>(x, w_folded, out, B, (int)H, (int)R, (int)J, st);
+        case 8: return launch_block<8>(x, w_folded, out, B, (int)H, (int)R, (int)J, st);
+        default: return launch_block<16>(x, w_folded, out, B, (int)H, (int)R, (int)J, st);
+    }
+}

@@ -78,6 +78,59 @@ def _(x, diag):
     return x.new_empty(x.shape[0], diag.shape[0] * diag.shape[2])
 
 
+# ----------------------------------------------------------------------------- bh4_block
+
+_L.define("bh4_fold(Tensor w) -> Tensor")
+
+
+def _bh4_fold_impl(w: torch.Tensor) -> torch.Tensor:
+    _lib.require_gpu(w)
+    assert w.dim() == 5 and w.dtype == torch.float32 and w.is_contiguous()
+    R, J, NB, bs, bs2 = w.shape
+    assert bs == bs2
+    out = torch.empty_like(w)
+    with _dev_guard(w):
+        rc = _lib.load().lffn_bh4_fold_f32(_lib.ptr(w), _lib.ptr(out), R, J, NB, bs, _lib.stream_of(w))
+    _lib.check(rc, f"lffn_bh4_fold_f32(R={R}, J={J}, num_block={NB}, block_size={bs})")
+    return out
+
+
+_L.impl("bh4_fold", _bh4_fold_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::bh4_fold")
+def _(w):
+    return torch.empty_like(w)
+
+
+_L.define("bh4_block(Tensor x, Tensor w_folded) -> Tensor")
+
+
+def _bh4_block_impl(x: torch.Tensor, w_folded: torch.Tensor) -> torch.Tensor:
+    _lib.require_gpu(x, w_folded)
+    assert x.dim() == 2 and w_folded.dim() == 5
+    assert x.dtype == torch.float32 and w_folded.dtype == torch.float32
+    assert x.is_contiguous() and w_folded.is_contiguous()
+    B, H = x.shape
+    R, J, NB, bs, _ = w_folded.shape
+    D = NB * bs
+    assert H <= D
+    out = torch.empty(B, R * D, dtype=torch.float32, device=x.device)
+    with _dev_guard(x):
+        rc = _lib.load().lffn_bh4_block_f32(_lib.ptr(x), _lib.ptr(w_folded), _lib.ptr(out), B, H, D, R, J, bs,
+                                            _lib.stream_of(x))
+    _lib.check(rc, f"lffn_bh4_block_f32(B={B}, H={H}, D={D}, R={R}, J={J}, block_size={bs})")
+    return out
+
+
+_L.impl("bh4_block", _bh4_block_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::bh4_block")
+def _(x, w_folded):
+    return x.new_empty(x.shape[0], w_folded.shape[0] * w_folded.shape[2] * w_folded.shape[3])
+
+
 # ----------------------------------------------------------------------------- project_hash
 
 _L.define("project_hash(Tensor x, Tensor diag, Tensor? bias, int T, float decay, float residual, bool keep_z)"
@@ -399,6 +452,8 @@ def _(code, g, tables):
 
 fht = torch.ops.lookupffn.fht
 bh4_diag = torch.ops.lookupffn.bh4_diag
+bh4_fold = torch.ops.lookupffn.bh4_fold
+bh4_block = torch.ops.lookupffn.bh4_block
 project_hash = torch.ops.lookupffn.project_hash
 ln_project_hash = torch.ops.lookupffn.ln_project_hash
 code_score = torch.ops.lookupffn.code_score

@@ -55,6 +55,18 @@ def bh4_diag(x, diag):
     return host(out)
 
 
+def bh4_block(x, w):
+    """fold + fused kernel; w: [R, J, NB, 64, 64]."""
+    xd, wd = dev(x), dev(w)
+    B, H = x.shape
+    R, J, NB, bs, _ = w.shape
+    wf = torch.empty_like(wd)
+    _call("lffn_bh4_fold_f32", p(wd), p(wf), R, J, NB, bs)
+    out = torch.full((B, R * NB * bs), float("nan"), dtype=torch.float32, device=DEV)
+    _call("lffn_bh4_block_f32", p(xd), p(wf), p(out), B, H, NB * bs, R, J, bs)
+    return host(out), host(wf)
+
+
 def project_hash(x, diag, bias, T, decay=0.7, keep_z=True):
     xd, dd, bd = dev(x), dev(diag), dev(bias)
     B, H = x.shape

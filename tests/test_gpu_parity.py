@@ -110,6 +110,55 @@ def test_bh4_diag_matches_oracle(H, D, R, J):
     assert relmax(got, want64) <= 1e-5
 
 
+# (B, H, D, R, J): every block count the kernel is built for (D/64 = 1..16), ragged token counts
+# around the 32-token tile, zero padding H < D, several repeats, stage counts other than 4
+BH4_BLOCK_CASES = [(37, 256, 256, 1, 4), (100, 768, 1024, 1, 4), (33, 1024, 1024, 4, 4), (1, 64, 64, 2, 4),
+                   (64, 100, 128, 1, 3), (31, 512, 512, 2, 1), (0, 64, 64, 1, 4)]
+
+
+@pytest.mark.parametrize("B,H,D,R,J", BH4_BLOCK_CASES)
+def test_bh4_block_matches_oracle(B, H, D, R, J):
+    import scipy.linalg
+    rng = np.random.RandomState(B + H + D + R + J)
+    NB = D // 64
+    x = rng.randn(B, H).astype(np.float32)
+    w = (rng.randn(R, J, NB, 64, 64) / math.sqrt(64 * D)).astype(np.float32)     # PL/lookup.py:22-23
+    got, folded = cabi.bh4_block(x, w)
+    # the folded weights are H_64 applied down the output index, exact up to fp32 rounding
+    want_f = np.einsum("po,rjnoi->rjnpi", scipy.linalg.hadamard(64).astype(np.float64), w.astype(np.float64))
+    assert relmax(folded, want_f) <= 1e-6
+    if B == 0:
+        assert got.shape == (0, R * D)
+        return
+    assert not np.isnan(got).any()
+    xp = np.concatenate([x, np.zeros((B, D - H), np.float32)], axis=1)
+    want64 = oracle.bh4(xp.astype(np.float64), w.astype(np.float64))
+    assert relmax(got, want64) <= 1e-5
+    # no further from the truth than the reference's own order of operations in fp32 (x3)
+    ref32 = oracle.bh4(xp, w)
+    assert relmax(got, want64) <= max(3 * relmax(ref32, want64), 2e-6)
+
+
+def test_bh4_block_exact_on_integers():
+    # identity blocks scaled by powers of two: every product and sum is exact, so the result is
+    # the plain transform applied J times, bit for bit
+    import scipy.linalg
+    rng = np.random.RandomState(12)
+    B, D, J = 40, 512, 2
+    NB = D // 64
+    x = rng.randint(-4, 5, size=(B, D)).astype(np.float32)
+    w = np.zeros((1, J, NB, 64, 64), np.float32)
+    for j in range(J):
+        for n in range(NB):
+            w[0, j, n] = np.eye(64, dtype=np.float32)[rng.permutation(64)] * (2.0 ** rng.randint(-2, 1))
+    got, _ = cabi.bh4_block(x, w)
+    want = x.astype(np.float64)
+    for j in range(J):
+        want = np.einsum("bni,noi->bno", want.reshape(B, NB, 64), w[0, j].astype(np.float64)).reshape(B, D)
+        want = want @ scipy.linalg.hadamard(D)
+    assert np.array_equal(got.astype(np.float64), want)
+
+
 def test_sign_diagonal_fht_exact():
     # the BASELINE "random +-1 sign diagonal from seed": one round, exact on integers
     rng = np.random.RandomState(8)
