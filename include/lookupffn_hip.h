@@ -75,7 +75,9 @@ int lffn_bh4_diag_f32(const float *x, const float *diag, float *out,
  * out: [B, R*D]; D = 64 * num_block a power of two, 64 <= D <= 1024; block_size must be 64.
  * The 64-point part of every transform is applied to the weights beforehand:
  * lffn_bh4_fold_f32 turns w [R, J, num_block, 64, 64] (PL/lookup.py:22) into
- * w_folded (same shape, caller-allocated, must not alias w), which
+ * w_folded (same size, caller-allocated, must not alias w; each 64 x 64 block
+ * is stored in the order the product kernel's lanes fetch it:
+ * [o/16][(i%16)/4][i/16][o%16][i%4] for output o, input i), which
  * lffn_bh4_block_f32 takes.  Fold again whenever w changes.  The products run on
  * the fp32 matrix cores; results agree with "product, then transform" to fp32
  * rounding, not bit for bit.

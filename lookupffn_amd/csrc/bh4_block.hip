@@ -33,7 +33,8 @@ constexpr int TOK = 32;         // tokens per workgroup
 constexpr int PAD = 4;          // floats of padding per LDS row
 
 // 64-point unnormalised Hadamard transform down the output index o of every block:
-// wf[blk][o'][i] = sum_o H64[o'][o] * w[blk][o][i].  One lane per (blk, i).
+// wf[blk]{o', i} = sum_o H64[o'][o] * w[blk][o][i], stored in the order the product kernel's
+// lanes fetch it.  One lane per (blk, i).
 __global__ __launch_bounds__(256) void bh4_fold_kernel(const float *w, float *wf, int64_t nblk) {
     const int64_t gid = int64_t(blockIdx.x) * 256 + threadIdx.x;
     if (gid >= nblk * BS) return;
@@ -54,10 +55,14 @@ __global__ __launch_bounds__(256) void bh4_fold_kernel(const float *w, float *wf
             }
         }
     }
-    float *dst = wf + blk * (BS * BS) + i;
+    // fragment order: [wavefront = o/16][q = (i%16)/4][lane = 16*(i/16) + o%16][i%4], so that a
+    // wavefront's load of (block, q) is 1 KB of contiguous memory, 16 bytes per lane
+    float *dst = wf + blk * (BS * BS) + ((i % 16) / 4) * 256 + (i / 16) * 64 + (i % 4);
 #pragma unroll
-    for (int o = 0; o < BS; ++o) dst[o * BS] = v[o];
+    for (int o = 0; o < BS; ++o) dst[(o / 16) * 1024 + (o % 16) * 4] = v[o];
 }
+
+#define LFFN_MFMA(acc, a, b) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc, 0, 0, 0)
 
 template <int NB>
 __global__ __launch_bounds__(256) void bh4_block_kernel(const float *__restrict__ x, const float *__restrict__ wf,
@@ -65,7 +70,10 @@ __global__ __launch_bounds__(256) void bh4_block_kernel(const float *__restrict_
                                                         int J) {
     constexpr int D = BS * NB;
     constexpr int LDR = D + PAD;
-    extern __shared__ float xs[];                 // TOK rows of LDR floats
+    constexpr int G = NB >= 2 ? 2 : 1;            // blocks worked on together
+    constexpr int NS = 2 * G;                     // register slots: block n sits in slot n % NS
+    constexpr bool AHEAD = NB >= NS;              // first blocks of a stage fetched during the previous one
+    extern __shared__ __attribute__((aligned(16))) float xs[];   // TOK rows of LDR floats
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -74,24 +82,53 @@ __global__ __launch_bounds__(256) void bh4_block_kernel(const float *__restrict_
     const int kq = lane >> 4;                     // k index inside an MFMA; result: output columns 4*kq .. 4*kq+3
     const int64_t tok_base = int64_t(blockIdx.x) * TOK;
 
-    // this lane's weight fragment of block n: wf[..][n][16*wave + c][16*kq .. 16*kq + 15]
-    const int w_lane_off = (16 * wave + c) * BS + 16 * kq;
+    // this lane's weight fragment of block n, quarter q (input columns 16*kq + 4*q .. +3 of output
+    // column 16*wave + c): wf[..][n][wave][q][lane][0..3]
+    const int w_lane_off = wave * 1024 + lane * 4;
     // this lane's token values of block n, half h: xs[(16*h + c) * LDR + 64*n + 16*kq ..]
     const int x_lane_off = c * LDR + 16 * kq;
     // where this lane's results of block n, half h go: xs[(16*h + c) * LDR + 64*n + 16*wave + 4*kq ..]
     const int y_lane_off = c * LDR + 16 * wave + 4 * kq;
 
+    auto load_w = [&](const float *wst, int n, int q) {
+        return *reinterpret_cast<const float4 *>(wst + n * (BS * BS) + q * 256);
+    };
+    auto read_x = [&](int h, int n, int q) {
+        return *reinterpret_cast<const float4 *>(xs + h * 16 * LDR + x_lane_off + n * BS + q * 4);
+    };
+
     for (int r = 0; r < R; ++r) {
         __syncthreads();                          // the previous repeat's last stage has been read
-        for (int e = tid; e < TOK * (D / 4); e += 256) {
-            const int row = e / (D / 4), col = (e % (D / 4)) * 4;
-            const int64_t tok = tok_base + row;
-            const float4 v = (tok < B && col < H) ? *reinterpret_cast<const float4 *>(x + tok * H + col)
-                                                  : make_float4(0.f, 0.f, 0.f, 0.f);      // zero padding to D
-            *reinterpret_cast<float4 *>(xs + row * LDR + col) = v;
+        {
+            // all of the tile's loads in flight before the first LDS store (one at a time, each
+            // would pay the full memory latency)
+            constexpr int NV = TOK * (D / 4) / 256;
+            float4 v[NV];
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int e = tid + i * 256;
+                const int row = e / (D / 4), col = (e % (D / 4)) * 4;
+                const int64_t tok = tok_base + row;
+                v[i] = (tok < B && col < H) ? *reinterpret_cast<const float4 *>(x + tok * H + col)
+                                            : make_float4(0.f, 0.f, 0.f, 0.f);      // zero padding to D
+            }
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int e = tid + i * 256;
+                const int row = e / (D / 4), col = (e % (D / 4)) * 4;
+                *reinterpret_cast<float4 *>(xs + row * LDR + col) = v[i];
+            }
         }
         __syncthreads();
 
+        float4 wq[NS][4];                         // weight fragments
+        if constexpr (AHEAD) {
+            const float *w0 = wf + (size_t)(r * J * NB) * (BS * BS) + w_lane_off;
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int g = 0; g < G; ++g) wq[g][q] = load_w(w0, g, q);
+        }
 #pragma unroll 1
         for (int s = 0; s < J; ++s) {
             const float *wst = wf + (size_t)((r * J + s) * NB) * (BS * BS) + w_lane_off;
@@ -101,39 +138,91 @@ __global__ __launch_bounds__(256) void bh4_block_kernel(const float *__restrict_
                 acc[0][n] = (f32x4){0.f, 0.f, 0.f, 0.f};
                 acc[1][n] = (f32x4){0.f, 0.f, 0.f, 0.f};
             }
-            // weight fragments two blocks ahead of their use
-            float4 wq[3][4];
+            if constexpr (!AHEAD) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                wq[0][q] = *reinterpret_cast<const float4 *>(wst + q * 4);
-                if (NB > 1) wq[1][q] = *reinterpret_cast<const float4 *>(wst + BS * BS + q * 4);
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                    for (int g = 0; g < G; ++g) wq[g][q] = load_w(wst, g, q);
             }
-            static_for<NB>([&](auto n_c) {
-                constexpr int n = decltype(n_c)::value;
-                if constexpr (n + 2 < NB) {
+            float4 xa[NS][4], xb[NS][4];          // token values, halves 0 and 1
 #pragma unroll
-                    for (int q = 0; q < 4; ++q)
-                        wq[(n + 2) % 3][q] = *reinterpret_cast<const float4 *>(wst + (n + 2) * (BS * BS) + q * 4);
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int g = 0; g < G; ++g) {
+                    xa[g][q] = read_x(0, g, q);
+                    xb[g][q] = read_x(1, g, q);
                 }
-                float4 xa[4], xb[4];
+
+            // A wavefront is alone on its SIMD and issues in order.  Two things keep the matrix
+            // core busy: (1) a product that accumulates into the result of an earlier one waits
+            // for it, and two chains in flight (the two token halves of one block) left the
+            // core idle 45 % of the time, so two blocks are worked on together: four independent
+            // chains; (2) the loads for the next pair of blocks are spread between the products
+            // instead of queueing in a burst at the LDS and the texture unit.
+            static_for<NB / G>([&](auto p_c) {
+                constexpr int n0 = decltype(p_c)::value * G;
+                constexpr int n1 = n0 + G - 1;                  // == n0 when G == 1
+                constexpr bool more = n0 + G < NB;              // another pair follows in this stage
+                constexpr int m0 = (n0 + G) % NS, m1 = (n1 + G) % NS;
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    xa[q] = *reinterpret_cast<const float4 *>(xs + x_lane_off + n * BS + q * 4);
-                    xb[q] = *reinterpret_cast<const float4 *>(xs + 16 * LDR + x_lane_off + n * BS + q * 4);
-                }
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const float4 wv = wq[n % 3][q];
-                    acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv.x, xa[q].x, acc[0][n], 0, 0, 0);
-                    acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv.x, xb[q].x, acc[1][n], 0, 0, 0);
-                    acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv.y, xa[q].y, acc[0][n], 0, 0, 0);
-                    acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv.y, xb[q].y, acc[1][n], 0, 0, 0);
-                    acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv.z, xa[q].z, acc[0][n], 0, 0, 0);
-                    acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv.z, xb[q].z, acc[1][n], 0, 0, 0);
-                    acc[0][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv.w, xa[q].w, acc[0][n], 0, 0, 0);
-                    acc[1][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv.w, xb[q].w, acc[1][n], 0, 0, 0);
+                    const float4 w0v = wq[n0 % NS][q], w1v = wq[n1 % NS][q];
+                    const float4 a0 = xa[n0 % NS][q], b0 = xb[n0 % NS][q];
+                    const float4 a1 = xa[n1 % NS][q], b1 = xb[n1 % NS][q];
+                    if constexpr (more) wq[m0][q] = load_w(wst, n0 + G, q);
+                    __builtin_amdgcn_sched_barrier(0);
+                    LFFN_MFMA(acc[0][n0], w0v.x, a0.x);
+                    LFFN_MFMA(acc[1][n0], w0v.x, b0.x);
+                    if constexpr (G == 2) {
+                        LFFN_MFMA(acc[0][n1], w1v.x, a1.x);
+                        LFFN_MFMA(acc[1][n1], w1v.x, b1.x);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    if constexpr (more) {
+                        xa[m0][q] = read_x(0, n0 + G, q);
+                        xb[m0][q] = read_x(1, n0 + G, q);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    LFFN_MFMA(acc[0][n0], w0v.y, a0.y);
+                    LFFN_MFMA(acc[1][n0], w0v.y, b0.y);
+                    if constexpr (G == 2) {
+                        LFFN_MFMA(acc[0][n1], w1v.y, a1.y);
+                        LFFN_MFMA(acc[1][n1], w1v.y, b1.y);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    if constexpr (more && G == 2) wq[m1][q] = load_w(wst, n1 + G, q);
+                    __builtin_amdgcn_sched_barrier(0);
+                    LFFN_MFMA(acc[0][n0], w0v.z, a0.z);
+                    LFFN_MFMA(acc[1][n0], w0v.z, b0.z);
+                    if constexpr (G == 2) {
+                        LFFN_MFMA(acc[0][n1], w1v.z, a1.z);
+                        LFFN_MFMA(acc[1][n1], w1v.z, b1.z);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    if constexpr (more && G == 2) {
+                        xa[m1][q] = read_x(0, n1 + G, q);
+                        xb[m1][q] = read_x(1, n1 + G, q);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    LFFN_MFMA(acc[0][n0], w0v.w, a0.w);
+                    LFFN_MFMA(acc[1][n0], w0v.w, b0.w);
+                    if constexpr (G == 2) {
+                        LFFN_MFMA(acc[0][n1], w1v.w, a1.w);
+                        LFFN_MFMA(acc[1][n1], w1v.w, b1.w);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             });
+            // the next stage's first blocks (a harmless re-read after the last stage): every product
+            // that read slots 0 .. G-1 was issued at least one pair ago
+            if constexpr (AHEAD) {
+                const float *wnx = wf + (size_t)((r * J + min(s + 1, J - 1)) * NB) * (BS * BS) + w_lane_off;
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                    for (int g = 0; g < G; ++g) wq[g][q] = load_w(wnx, g, q);
+                __builtin_amdgcn_sched_barrier(0);
+            }
 
             // H_NB across the blocks
 #pragma unroll

@@ -124,9 +124,11 @@ def test_bh4_block_matches_oracle(B, H, D, R, J):
     x = rng.randn(B, H).astype(np.float32)
     w = (rng.randn(R, J, NB, 64, 64) / math.sqrt(64 * D)).astype(np.float32)     # PL/lookup.py:22-23
     got, folded = cabi.bh4_block(x, w)
-    # the folded weights are H_64 applied down the output index, exact up to fp32 rounding
+    # the folded weights are H_64 applied down the output index, exact up to fp32 rounding, stored
+    # per block as [o/16][(i%16)/4][i/16][o%16][i%4]
     want_f = np.einsum("po,rjnoi->rjnpi", scipy.linalg.hadamard(64).astype(np.float64), w.astype(np.float64))
-    assert relmax(folded, want_f) <= 1e-6
+    unpacked = folded.reshape(R, J, NB, 4, 4, 4, 16, 4).transpose(0, 1, 2, 3, 6, 5, 4, 7).reshape(R, J, NB, 64, 64)
+    assert relmax(unpacked, want_f) <= 1e-6
     if B == 0:
         assert got.shape == (0, R * D)
         return
