@@ -1,6 +1,6 @@
 """Benchmark of the LookupFFN hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg1|cfg3|cfg3bf16]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg1|cfg3|cfg3bf16|cfg2b64|cfg4|cfg5]
 
 A step is one forward pass of the layer over one batch of synthetic tokens that
 is already resident in HBM: fused LayerNorm+projection+hash kernel -> gather-add
@@ -42,6 +42,11 @@ WORKLOADS = {
                  desc="config 3: 16384 tokens, d=1024, 512 tables x 256 x 1024 fp32"),
     "cfg3bf16": dict(B=16384, H=1024, T=512, S=256, Do=1024, bf16=True,
                      desc="config 3: 16384 tokens, d=1024, 512 tables x 256 x 1024 bf16 rows, fp32 accumulate"),
+    # config 2 with the 64 x 64 block-diagonal BH4 the reference's training configs use
+    # (cfgs/roberta/small-512/lookup-t128-s8-bh4.py:25-26) instead of the sign diagonal
+    "cfg2b64": dict(B=16384, H=768, T=128, S=256, Do=768, bf16=False, bs=64,
+                    desc="config 2 shape with BH4 block size 64 (the reference's training config): 32x512 tokens, "
+                         "d=768 padded to 1024, 4 stages of 16 blocks 64x64, 128 tables x 256 x 768 fp32"),
     # BASELINE.json configs[3]: the 12-layer encoder with every FFN a config-2 LookupFFN
     "cfg4": dict(B=16384, H=768, T=128, S=256, Do=768, bf16=False,
                  desc="config 4: 12-layer pre-norm RoBERTa-base encoder (hidden 768, 12 heads, seq 512, batch 32), "
@@ -63,15 +68,19 @@ def build_layer(wl, device):
     import lookupffn_amd
 
     cfg = Namespace(hidden_size=wl["H"], ffn_num_table=wl["T"], ffn_table_size=wl["S"],
-                    layer_norm_eps=1e-5, projection_type="bh4", block_size=1)
+                    layer_norm_eps=1e-5, projection_type="bh4", block_size=wl.get("bs", 1))
     g = torch.Generator().manual_seed(1234)
     layer = lookupffn_amd.LookupFFN(cfg, wl["Do"]).eval()
     p = layer.hash.projection
     with torch.no_grad():
-        # seeded +-1 sign diagonals, scaled by 1/sqrt(D) so that each of the four
-        # (diagonal, Hadamard) stages is orthonormal
-        sign = 2.0 * torch.randint(0, 2, p.weight.shape, generator=g).float() - 1.0
-        p.weight.copy_(sign / math.sqrt(p.padded_in_dim))
+        if p.block_size == 1:
+            # seeded +-1 sign diagonals, scaled by 1/sqrt(D) so that each of the four
+            # (diagonal, Hadamard) stages is orthonormal
+            sign = 2.0 * torch.randint(0, 2, p.weight.shape, generator=g).float() - 1.0
+            p.weight.copy_(sign / math.sqrt(p.padded_in_dim))
+        else:
+            # the reference's initialisation, PL/lookup.py:22-23
+            p.weight.copy_(torch.randn(p.weight.shape, generator=g) / math.sqrt(p.block_size * p.padded_in_dim))
         layer.tables.copy_(0.02 * torch.randn(layer.tables.shape, generator=g))
         layer.bias.copy_(0.001 * torch.randn(layer.bias.shape, generator=g))
     x = torch.randn(wl["B"], wl["H"], generator=g)
@@ -365,11 +374,18 @@ def main():
     esz = 2 if wl["bf16"] else 4
     gather_bytes = B * T * Do * esz + B * T * 8 + B * Do * 4
 
+    block = layer.hash.projection.block_size != 1
+
+    def hash_front():
+        if block:        # one kernel: LayerNorm, BH4 on the matrix cores, mix + hash
+            return layer.hash.forward_block(x, layer_norm=layer.LayerNorm)
+        return layer.hash.forward_fused(x, layer_norm=layer.LayerNorm)
+
     def step(events=None):
         # exactly what LookupFFN.forward runs in eval mode (checked below), with an
         # event pair around the gather launch
         with torch.no_grad():
-            code, score = layer.hash.forward_fused(x, layer_norm=layer.LayerNorm)
+            code, score = hash_front()
             if events is not None:
                 events[0].record()
             out = ops.lookup_gather(code, score, layer.tables, layer.bias)
@@ -407,7 +423,7 @@ def main():
         b.record(); torch.cuda.synchronize()
         return a.elapsed_time(b) / n
     with torch.no_grad():
-        hash_ms = timed(lambda: layer.hash.forward_fused(x, layer_norm=layer.LayerNorm))
+        hash_ms = timed(hash_front)
 
     res = {
         "metric": "LookupFFN fwd tokens/s + gather-add GB/s as % of HBM peak, RoBERTa-base",
@@ -421,14 +437,19 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16 rows, f32 accumulate" if wl["bf16"] else "f32",
-        "data": "synthetic (seeded N(0,1) tokens, seeded +-1/sqrt(D) sign diagonals, N(0,0.02) tables)",
+        "data": ("synthetic (seeded N(0,1) tokens, N(0,1)/sqrt(64 D) block weights, N(0,0.02) tables)" if block else
+                 "synthetic (seeded N(0,1) tokens, seeded +-1/sqrt(D) sign diagonals, N(0,0.02) tables)"),
         "config": {"workload": wl["desc"], "tokens": B, "d_model": H, "fht_dim": layer.hash.projection.padded_in_dim,
-                   "tables": T, "table_size": S, "d_out": Do, "step": "one kernel: LayerNorm + BH4(block 1)x4 + mix + hash; one kernel: gather-add + bias"},
+                   "tables": T, "table_size": S, "d_out": Do,
+                   "step": ("one kernel: LayerNorm + BH4(block 64)x4 on fp32 MFMA + mix + hash (weights folded once, "
+                            "outside the step); one kernel: gather-add + bias") if block else
+                           "one kernel: LayerNorm + BH4(block 1)x4 + mix + hash; one kernel: gather-add + bias"},
         "roofline": {"bound": "hbm", "kernel": "lookup_gather", "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
                      "algorithmic_bytes": gather_bytes, "avg_kernel_ms": gather_ms},
-        "stages_ms": {"layernorm_project_hash": hash_ms, "gather_add": gather_ms},
+        "stages_ms": {("layernorm_bh4block_hash" if block else "layernorm_project_hash"): hash_ms,
+                      "gather_add": gather_ms},
         "gather_tokens_per_s": B / (gather_ms * 1e-3),
     }
     if not args.no_cpu_baseline:

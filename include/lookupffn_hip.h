@@ -90,6 +90,34 @@ int lffn_bh4_block_f32(const float *x, const float *w_folded, float *out, int64_
                        int64_t D, int64_t R, int64_t J, int64_t block_size, void *stream);
 
 /*
+ * The whole hashing front end of the layer for 64 x 64 blocks and 8-bit codes, one kernel:
+ * (LayerNorm ->) zero-pad -> BH4 as lffn_bh4_block_f32 -> z = decay*y + residual*pad(h) + bias
+ * -> code and score of every 8 columns of z[:, :T*8].  ln_weight == NULL: no LayerNorm
+ * (h = x), else h = LayerNorm(x; ln_weight, ln_bias, ln_eps) over the H columns.
+ * x: [B, H], H % 4 == 0; w_folded from lffn_bh4_fold_f32; proj_bias: [T*8] or NULL;
+ * codes: [B, T] int32; scores: [B, T]; T*8 <= R*D.  Neither y nor z is written.
+ * Replaces self.LayerNorm (PL/lookup.py:99), BH4._forward (PL/lookup.py:29-39) and
+ * compute_code_score (PL/compute_code_score/kernel.py:22-55) for block_size == 64.
+ */
+int lffn_ln_bh4_block_hash_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
+                               const float *w_folded, const float *proj_bias, int32_t *codes, float *scores,
+                               int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
+                               int64_t block_size, float decay, float residual, void *stream);
+
+/*
+ * The tail of the BH4 module and the hash in one pass, for any block size:
+ *   z[b, c] = decay * y[b, c] + residual * pad(x)[b, c % D] + bias[c],  c < T*k
+ *   (code, score)[b, t] = code and score of z[b, t*k : (t+1)*k]   (as lffn_code_score_f32)
+ * y: [B, ldy], the output of bh4 (ldy = R*D >= T*k); x: [B, H], H <= D, the projection's
+ * input before zero padding; bias: [T*k] or NULL; codes: [B, T] int32; scores: [B, T].
+ * z is not written.  Replaces the mix, slice and bias of BH4._forward (PL/lookup.py:36-37)
+ * together with compute_code_score (PL/compute_code_score/kernel.py:22-55).
+ */
+int lffn_mix_code_score_f32(const float *y, const float *x, const float *bias, int32_t *codes,
+                            float *scores, int64_t B, int64_t T, int64_t k, int64_t H, int64_t D,
+                            int64_t ldy, float decay, float residual, void *stream);
+
+/*
  * The whole hashing front-end of the layer in one pass over x, for block size 1
  * and 8-bit codes (PL/lookup.py:29-39,64-77 + PL/compute_code_score/kernel.py:43-55):
  *   y      = bh4_diag(x)                                   (as above)

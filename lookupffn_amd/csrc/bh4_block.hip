@@ -22,7 +22,19 @@
 // (the reference's order): the 64-point part is applied to the weights, in fp32,
 // before the product.  Results agree to fp32 rounding (1e-5 of the row's largest
 // magnitude), not bit for bit.
+//
+// The same kernel also runs the layer's whole hashing front end for 8-bit codes
+// (lffn_ln_bh4_block_hash_f32): LayerNorm while the token tile is loaded (a wavefront
+// owns 8 rows, a row is spread over its 64 lanes; mean and 1/sigma are kept in LDS),
+// and after the last stage, instead of storing y, z = decay*y + residual*LN(x) + bias
+// on the accumulators (x is read again and normalised with the kept statistics) and
+// the code and score of every 8 columns: a group is split over the lane pair
+// (l, l+16), whose second lane continues the first lane's running sum and product so
+// that the operations run in column order.
 #include "lffn_common.h"
+
+// the mix and the score keep the reference's operation order: no fused multiply-add
+#pragma clang fp contract(off)
 
 namespace {
 
@@ -64,16 +76,36 @@ __global__ __launch_bounds__(256) void bh4_fold_kernel(const float *w, float *wf
 
 #define LFFN_MFMA(acc, a, b) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc, 0, 0, 0)
 
-template <int NB>
-__global__ __launch_bounds__(256) void bh4_block_kernel(const float *__restrict__ x, const float *__restrict__ wf,
-                                                        float *__restrict__ out, int64_t B, int H, int R,
-                                                        int J) {
+struct BlockArgs {
+    const float *x;        // [B, H]
+    const float *ln_w;     // [H] LayerNorm weight, or null: no LayerNorm
+    const float *ln_b;     // [H]
+    float ln_eps;
+    const float *wf;       // folded weights
+    float *out;            // [B, R*D]            (plain form)
+    const float *pbias;    // [T*8] or null       (hash form)
+    int32_t *codes;        // [B, T]              (hash form)
+    float *scores;         // [B, T]              (hash form)
+    int64_t B;
+    int H, R, J, T;
+    float decay, residual;
+};
+
+template <int NB, bool HASH>
+__global__ __launch_bounds__(256) void bh4_block_kernel(BlockArgs a) {
+    const float *__restrict__ x = a.x;
+    const float *__restrict__ wf = a.wf;
+    const int64_t B = a.B;
+    const int H = a.H, R = a.R, J = a.J;
     constexpr int D = BS * NB;
     constexpr int LDR = D + PAD;
     constexpr int G = NB >= 2 ? 2 : 1;            // blocks worked on together
     constexpr int NS = 2 * G;                     // register slots: block n sits in slot n % NS
     constexpr bool AHEAD = NB >= NS;              // first blocks of a stage fetched during the previous one
-    extern __shared__ __attribute__((aligned(16))) float xs[];   // TOK rows of LDR floats
+    extern __shared__ __attribute__((aligned(16))) float xs[];   // TOK rows of LDR floats, then the row statistics
+    float *stats = xs + TOK * LDR;                // [TOK][2]: mean and 1/sigma of LayerNorm
+    float *lnw_s = stats + 2 * TOK;               // [D] LayerNorm weight and bias (hash form, for the epilogue)
+    float *lnb_s = lnw_s + D;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -81,6 +113,15 @@ __global__ __launch_bounds__(256) void bh4_block_kernel(const float *__restrict_
     const int c = lane & 15;                      // A operand: output column; B operand and result: token
     const int kq = lane >> 4;                     // k index inside an MFMA; result: output columns 4*kq .. 4*kq+3
     const int64_t tok_base = int64_t(blockIdx.x) * TOK;
+    if (HASH && a.ln_w) {
+        for (int e = tid * 4; e < D; e += 1024) {
+            const bool in = e < H;
+            *reinterpret_cast<float4 *>(lnw_s + e) = in ? *reinterpret_cast<const float4 *>(a.ln_w + e)
+                                                        : make_float4(0.f, 0.f, 0.f, 0.f);
+            *reinterpret_cast<float4 *>(lnb_s + e) = in ? *reinterpret_cast<const float4 *>(a.ln_b + e)
+                                                        : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
 
     // this lane's weight fragment of block n, quarter q (input columns 16*kq + 4*q .. +3 of output
     // column 16*wave + c): wf[..][n][wave][q][lane][0..3]
@@ -100,24 +141,70 @@ __global__ __launch_bounds__(256) void bh4_block_kernel(const float *__restrict_
     for (int r = 0; r < R; ++r) {
         __syncthreads();                          // the previous repeat's last stage has been read
         {
-            // all of the tile's loads in flight before the first LDS store (one at a time, each
-            // would pay the full memory latency)
-            constexpr int NV = TOK * (D / 4) / 256;
-            float4 v[NV];
+            // A wavefront loads 8 rows, 16 bytes per lane and 1 KB of a row per instruction, all
+            // loads in flight before the first use (one at a time, each would pay the full
+            // memory latency).  Columns at or beyond H are zero.
+            constexpr int RPW = TOK / 4;
+            constexpr int NQ = D >= 256 ? D / 256 : 1;
+            float4 v[RPW][NQ];
 #pragma unroll
-            for (int i = 0; i < NV; ++i) {
-                const int e = tid + i * 256;
-                const int row = e / (D / 4), col = (e % (D / 4)) * 4;
-                const int64_t tok = tok_base + row;
-                v[i] = (tok < B && col < H) ? *reinterpret_cast<const float4 *>(x + tok * H + col)
-                                            : make_float4(0.f, 0.f, 0.f, 0.f);      // zero padding to D
+            for (int i = 0; i < RPW; ++i) {
+                const int64_t tok = tok_base + wave * RPW + i;
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) {
+                    const int col = (q * 64 + lane) * 4;
+                    v[i][q] = (tok < B && col < H) ? *reinterpret_cast<const float4 *>(x + tok * H + col)
+                                                   : make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+            }
+            if (a.ln_w) {
+                // LayerNorm over the H valid columns (biased variance, two passes, eps inside the
+                // square root: torch.nn.LayerNorm, PL/lookup.py:84,99)
+                float4 lw[NQ], lb[NQ];
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) {
+                    const int col = (q * 64 + lane) * 4;
+                    lw[q] = col < H ? *reinterpret_cast<const float4 *>(a.ln_w + col) : make_float4(0.f, 0.f, 0.f, 0.f);
+                    lb[q] = col < H ? *reinterpret_cast<const float4 *>(a.ln_b + col) : make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+#pragma unroll
+                for (int i = 0; i < RPW; ++i) {
+                    float s1 = 0.f;
+#pragma unroll
+                    for (int q = 0; q < NQ; ++q) s1 += (v[i][q].x + v[i][q].y) + (v[i][q].z + v[i][q].w);
+                    const float mean = wave_sum(s1) / float(H);
+                    float s2 = 0.f;
+#pragma unroll
+                    for (int q = 0; q < NQ; ++q) {
+                        if ((q * 64 + lane) * 4 < H) {
+                            const float d0 = v[i][q].x - mean, d1 = v[i][q].y - mean;
+                            const float d2 = v[i][q].z - mean, d3 = v[i][q].w - mean;
+                            s2 += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
+                        }
+                    }
+                    const float rstd = 1.0f / sqrtf(wave_sum(s2) / float(H) + a.ln_eps);
+#pragma unroll
+                    for (int q = 0; q < NQ; ++q) {
+                        if ((q * 64 + lane) * 4 < H) {
+                            v[i][q].x = (v[i][q].x - mean) * rstd * lw[q].x + lb[q].x;
+                            v[i][q].y = (v[i][q].y - mean) * rstd * lw[q].y + lb[q].y;
+                            v[i][q].z = (v[i][q].z - mean) * rstd * lw[q].z + lb[q].z;
+                            v[i][q].w = (v[i][q].w - mean) * rstd * lw[q].w + lb[q].w;
+                        }
+                    }
+                    if (lane == 0) {
+                        stats[2 * (wave * RPW + i)] = mean;
+                        stats[2 * (wave * RPW + i) + 1] = rstd;
+                    }
+                }
             }
 #pragma unroll
-            for (int i = 0; i < NV; ++i) {
-                const int e = tid + i * 256;
-                const int row = e / (D / 4), col = (e % (D / 4)) * 4;
-                *reinterpret_cast<float4 *>(xs + row * LDR + col) = v[i];
-            }
+            for (int i = 0; i < RPW; ++i)
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) {
+                    const int col = (q * 64 + lane) * 4;
+                    if (col < D) *reinterpret_cast<float4 *>(xs + (wave * RPW + i) * LDR + col) = v[i][q];
+                }
         }
         __syncthreads();
 
@@ -248,15 +335,117 @@ __global__ __launch_bounds__(256) void bh4_block_kernel(const float *__restrict_
                     *reinterpret_cast<f32x4 *>(xs + 16 * LDR + y_lane_off + n * BS) = acc[1][n];
                 }
                 __syncthreads();
-            } else {
+            } else if constexpr (!HASH) {
                 const int64_t ld_out = int64_t(R) * D;
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
                     const int64_t tok = tok_base + 16 * t + c;
                     if (tok < B) {
-                        float *o = out + tok * ld_out + (size_t)r * D + 16 * wave + 4 * kq;
+                        float *o = a.out + tok * ld_out + (size_t)r * D + 16 * wave + 4 * kq;
 #pragma unroll
                         for (int n = 0; n < NB; ++n) *reinterpret_cast<f32x4 *>(o + n * BS) = acc[t][n];
+                    }
+                }
+            } else {
+                const int ncols = a.T * 8;
+                constexpr int CROW = D / 8 + 1;                // padded: tokens down a column hit different banks
+                int *cs = reinterpret_cast<int *>(xs);         // [TOK][CROW] codes of this repeat
+                float *ss = xs + TOK * CROW;                   // [TOK][CROW] scores
+                // the addresses below do not change from stage to stage; computed from an opaque
+                // zero they are formed here instead of being kept in registers through the stages
+                int opq = 0;
+                asm volatile("" : "+v"(opq));
+                int64_t tokv[2];
+                bool livev[2];
+                float meanv[2], rstdv[2];
+                // the two tokens' input values for every block, all requested before the first use
+                float4 xin[2][NB];
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    tokv[t] = tok_base + 16 * t + c + opq;
+                    livev[t] = tokv[t] < B;
+                    meanv[t] = a.ln_w ? stats[2 * (16 * t + c + opq)] : 0.f;
+                    rstdv[t] = a.ln_w ? stats[2 * (16 * t + c + opq) + 1] : 1.f;
+#pragma unroll
+                    for (int n = 0; n < NB; ++n) {
+                        const int xc = n * BS + 16 * wave + 4 * kq + opq;
+                        xin[t][n] = (livev[t] && xc < H) ? *reinterpret_cast<const float4 *>(x + tokv[t] * H + xc)
+                                                         : make_float4(0.f, 0.f, 0.f, 0.f);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int n = 0; n < NB; ++n) {
+                    const int xc = n * BS + 16 * wave + 4 * kq + opq;      // column of the padded input
+                    const int col = r * D + xc;                            // column of z
+                    const bool in_cols = col < ncols;                      // whole groups of 8: all or nothing
+                    float4 lw = make_float4(0.f, 0.f, 0.f, 0.f), lb = lw, bb = lw;
+                    if (a.ln_w && xc < H) {
+                        lw = *reinterpret_cast<const float4 *>(lnw_s + xc);
+                        lb = *reinterpret_cast<const float4 *>(lnb_s + xc);
+                    }
+                    if (a.pbias && in_cols) bb = *reinterpret_cast<const float4 *>(a.pbias + col);
+                    // the two token halves side by side: independent work for a wavefront that has
+                    // its SIMD to itself
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        float4 xv = xin[t][n];
+                        if (a.ln_w && xc < H) {
+                            xv.x = (xv.x - meanv[t]) * rstdv[t] * lw.x + lb.x;
+                            xv.y = (xv.y - meanv[t]) * rstdv[t] * lw.y + lb.y;
+                            xv.z = (xv.z - meanv[t]) * rstdv[t] * lw.z + lb.z;
+                            xv.w = (xv.w - meanv[t]) * rstdv[t] * lw.w + lb.w;
+                        }
+                        float z[4];
+                        z[0] = a.decay * acc[t][n].x + a.residual * xv.x;
+                        z[1] = a.decay * acc[t][n].y + a.residual * xv.y;
+                        z[2] = a.decay * acc[t][n].z + a.residual * xv.z;
+                        z[3] = a.decay * acc[t][n].w + a.residual * xv.w;
+                        if (a.pbias && in_cols) {
+                            z[0] = z[0] + bb.x; z[1] = z[1] + bb.y; z[2] = z[2] + bb.z; z[3] = z[3] + bb.w;
+                        }
+                        // columns 8g .. 8g+3 sit in the lane with even kq (the high nibble),
+                        // 8g+4 .. 8g+7 in lane + 16, which continues the sum and the product
+                        // (d = 0..7 in order, compute_code_score/torch_extension.cc:31-37)
+                        const int nib = (z[0] > 0.f ? 8 : 0) | (z[1] > 0.f ? 4 : 0) | (z[2] > 0.f ? 2 : 0) |
+                                        (z[3] > 0.f ? 1 : 0);
+                        float az[4], fz[4];
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            az[i] = fabsf(z[i]);
+                            fz[i] = 1.0f + expf(-2.0f * az[i]);
+                        }
+                        float s_loc = 0.f, p_loc = 1.f;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) { s_loc = s_loc + az[i]; p_loc = p_loc * fz[i]; }
+                        float s_run = lane_xor<16>(s_loc);
+                        float p_run = lane_xor<16>(p_loc);
+                        const int nib_hi = __float_as_int(lane_xor<16>(__int_as_float(nib)));
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) { s_run = s_run + az[i]; p_run = p_run * fz[i]; }
+                        // staged in LDS (the stage buffer is free now), written out row by row below:
+                        // straight from here a store would scatter 4-byte pieces over 32 rows
+                        if (kq & 1) {
+                            cs[(16 * t + c) * CROW + (xc >> 3)] = (nib_hi << 4) | nib;
+                            ss[(16 * t + c) * CROW + (xc >> 3)] = s_run / p_run;
+                        }
+                    }
+                }
+                __syncthreads();
+                // wavefront w writes the D/8 codes and scores of tokens 8w .. 8w+7
+#pragma unroll 1
+                for (int i = 0; i < TOK / 4; ++i) {
+                    const int row = wave * (TOK / 4) + i;
+                    const int64_t tok = tok_base + row;
+                    if (tok >= B) break;
+#pragma unroll
+                    for (int e0 = 0; e0 < D / 8; e0 += 64) {
+                        const int e = e0 + lane;
+                        const int tt = r * (D / 8) + e;
+                        if (e < D / 8 && tt < a.T) {
+                            a.codes[tok * a.T + tt] = cs[row * CROW + e];
+                            a.scores[tok * a.T + tt] = ss[row * CROW + e];
+                        }
                     }
                 }
             }
@@ -264,17 +453,28 @@ __global__ __launch_bounds__(256) void bh4_block_kernel(const float *__restrict_
     }
 }
 
-template <int NB>
-int launch_block(const float *x, const float *wf, float *out, int64_t B, int H, int R, int J, hipStream_t st) {
-    const size_t lds_bytes = size_t(TOK) * (BS * NB + PAD) * sizeof(float);
-    auto kern = bh4_block_kernel<NB>;
+template <int NB, bool HASH>
+int launch_block(const BlockArgs &a, hipStream_t st) {
+    const size_t lds_bytes = (size_t(TOK) * (BS * NB + PAD) + 2 * TOK + (HASH ? 2 * BS * NB : 0)) * sizeof(float);
+    auto kern = bh4_block_kernel<NB, HASH>;
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds_bytes) != hipSuccess) {
         (void)hipGetLastError();
         return LFFN_ERR_LAUNCH;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)((B + TOK - 1) / TOK)), dim3(256), lds_bytes, st, x, wf, out, B, H, R, J);
+    hipLaunchKernelGGL(kern, dim3((unsigned)((a.B + TOK - 1) / TOK)), dim3(256), lds_bytes, st, a);
     return lffn_launch_status();
+}
+
+template <bool HASH>
+int dispatch_block(const BlockArgs &a, int64_t D, hipStream_t st) {
+    switch (D / BS) {
+        case 1: return launch_block<1, HASH>(a, st);
+        case 2: return launch_block<2, HASH>(a, st);
+        case 4: return launch_block<4, HASH>(a, st);
+        case 8: return launch_block<8, HASH>(a, st);
+        default: return launch_block<16, HASH>(a, st);
+    }
 }
 
 }  // namespace
@@ -300,12 +500,30 @@ extern "C" int lffn_bh4_block_f32(const float *x, const float *w_folded, float *
     if (B == 0) return LFFN_OK;
     LFFN_REQUIRE(x && w_folded && out, LFFN_ERR_BAD_ARG);
     LFFN_REQUIRE(lffn_aligned16(x) && lffn_aligned16(w_folded) && lffn_aligned16(out), LFFN_ERR_BAD_ARG);
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    switch (D / BS) {
-        case 1: return launch_block<1>(x, w_folded, out, B, (int)H, (int)R, (int)J, st);
-        case 2: return launch_block<2>(x, w_folded, out, B, (int)H, (int)R, (int)J, st);
-        case 4: return launch_block<4>(x, w_folded, out, B, (int)H, (int)R, (int)J, st);
-        case 8: return launch_block<8>(x, w_folded, out, B, (int)H, (int)R, (int)J, st);
-        default: return launch_block<16>(x, w_folded, out, B, (int)H, (int)R, (int)J, st);
-    }
+    BlockArgs a{};
+    a.x = x; a.wf = w_folded; a.out = out; a.B = B; a.H = (int)H; a.R = (int)R; a.J = (int)J;
+    return dispatch_block<false>(a, D, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int lffn_ln_bh4_block_hash_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
+                                          const float *w_folded, const float *proj_bias, int32_t *codes,
+                                          float *scores, int64_t B, int64_t H, int64_t D, int64_t R, int64_t J,
+                                          int64_t T, int64_t block_size, float decay, float residual,
+                                          void *stream) {
+    LFFN_REQUIRE(B >= 0 && R >= 1 && J >= 1 && D >= 1 && H >= 1 && H <= D && T >= 0, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(H % 4 == 0 && J <= 64, LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(block_size == BS && lffn_is_pow2(D) && D >= BS && D <= 1024, LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(R <= 4096 && B <= (int64_t(1) << 31) - 1 && T <= (1 << 24), LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(T * 8 <= R * D, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(!ln_weight || (ln_bias && ln_eps >= 0.f), LFFN_ERR_BAD_ARG);
+    if (B == 0 || T == 0) return LFFN_OK;
+    LFFN_REQUIRE(x && w_folded && codes && scores, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_aligned16(x) && lffn_aligned16(w_folded) && (!proj_bias || lffn_aligned16(proj_bias)) &&
+                     (!ln_weight || (lffn_aligned16(ln_weight) && lffn_aligned16(ln_bias))),
+                 LFFN_ERR_BAD_ARG);
+    BlockArgs a{};
+    a.x = x; a.ln_w = ln_weight; a.ln_b = ln_bias; a.ln_eps = ln_eps; a.wf = w_folded; a.pbias = proj_bias;
+    a.codes = codes; a.scores = scores; a.B = B; a.H = (int)H; a.R = (int)R; a.J = (int)J; a.T = (int)T;
+    a.decay = decay; a.residual = residual;
+    return dispatch_block<true>(a, D, static_cast<hipStream_t>(stream));
 }

@@ -104,10 +104,50 @@ class Hashing(nn.Module):
                 float(p.decay_coeff), float(1 - p.decay_coeff), False)
         return code, score
 
+    def can_fuse_block(self, x):
+        """Two kernels for 64 x 64 blocks without gradient: all BH4 stages on the matrix
+        cores, then mix + bias + code + score."""
+        p = self.projection
+        needs_grad = torch.is_grad_enabled() and (
+            x.requires_grad or any(q.requires_grad for q in self.parameters()))
+        return (isinstance(p, BH4) and p.block_size == 64 and 64 <= p.padded_in_dim <= 1024
+                and p.in_dim % 4 == 0 and self.code_length <= 24
+                and x.dtype == torch.float32 and x.is_cuda and not needs_grad)
+
+    def folded_weight(self):
+        """The BH4 weights with the 64-point transform applied (what ops.bh4_block takes), kept
+        until the parameter is modified or moved."""
+        w = self.projection.weight
+        key = (w._version, w.data_ptr(), w.device)
+        cached = getattr(self, "_folded", None)
+        if cached is None or cached[0] != key:
+            cached = (key, ops.bh4_fold(w.detach().contiguous()))
+            self._folded = cached
+        return cached[1]
+
+    def forward_block(self, x, layer_norm=None):
+        """8-bit codes: one kernel, (LayerNorm ->) BH4 on the matrix cores -> mix -> bias ->
+        code + score.  Other code lengths: the BH4 kernel, then mix + hash in a second one."""
+        p = self.projection
+        x = x.contiguous()
+        if self.code_length == 8:
+            lw = None if layer_norm is None else layer_norm.weight
+            lb = None if layer_norm is None else layer_norm.bias
+            eps = 0.0 if layer_norm is None else float(layer_norm.eps)
+            return ops.ln_bh4_block_hash(x, lw, lb, eps, self.folded_weight(), p.bias, self.num_table,
+                                         float(p.decay_coeff), float(1 - p.decay_coeff))
+        if layer_norm is not None:
+            x = layer_norm(x)
+        y = ops.bh4_block(x, self.folded_weight())
+        return ops.mix_code_score(y, x, p.bias, self.num_table, self.code_length, p.padded_in_dim,
+                                  float(p.decay_coeff), float(1 - p.decay_coeff))
+
     def forward(self, x):
         B, D = x.shape
         if self.can_fuse(x):
             return self.forward_fused(x)
+        if self.can_fuse_block(x):
+            return self.forward_block(x)
         z = self.projection(x)
         z = z.reshape(B, self.num_table, self.code_length)
         code, score = compute_code_score(z, training=self.training)
@@ -136,11 +176,14 @@ class LookupFFN(nn.Module):
 
     def _forward(self, hidden_states):
         ln = self.LayerNorm
-        if (self.hash.can_fuse(hidden_states) and ln.elementwise_affine and ln.weight is not None
-                and ln.bias is not None and ln.weight.dtype == torch.float32
-                and not (torch.is_grad_enabled() and (ln.weight.requires_grad or ln.bias.requires_grad))):
+        ln_fusable = (ln.elementwise_affine and ln.weight is not None and ln.bias is not None
+                      and ln.weight.dtype == torch.float32
+                      and not (torch.is_grad_enabled() and (ln.weight.requires_grad or ln.bias.requires_grad)))
+        if ln_fusable and self.hash.can_fuse(hidden_states):
             # inference: LayerNorm runs inside the projection kernel
             code, score = self.hash.forward_fused(hidden_states, layer_norm=ln)
+        elif ln_fusable and self.hash.can_fuse_block(hidden_states):
+            code, score = self.hash.forward_block(hidden_states, layer_norm=ln)
         else:
             hidden_states = ln(hidden_states)
             code, score = self.hash(hidden_states)

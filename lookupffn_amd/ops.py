@@ -131,6 +131,81 @@ def _(x, w_folded):
     return x.new_empty(x.shape[0], w_folded.shape[0] * w_folded.shape[2] * w_folded.shape[3])
 
 
+# ----------------------------------------------------------------------------- ln_bh4_block_hash
+
+_L.define("ln_bh4_block_hash(Tensor x, Tensor? ln_weight, Tensor? ln_bias, float ln_eps, Tensor w_folded, "
+          "Tensor? bias, int T, float decay, float residual) -> (Tensor, Tensor)")
+
+
+def _ln_bh4_block_hash_impl(x, ln_weight, ln_bias, ln_eps, w_folded, bias, T, decay, residual):
+    _lib.require_gpu(x, ln_weight, ln_bias, w_folded, bias)
+    assert x.dim() == 2 and w_folded.dim() == 5
+    assert x.dtype == torch.float32 and w_folded.dtype == torch.float32
+    assert x.is_contiguous() and w_folded.is_contiguous()
+    B, H = x.shape
+    R, J, NB, bs, _ = w_folded.shape
+    D = NB * bs
+    assert H <= D and T * 8 <= R * D
+    for t in (ln_weight, ln_bias):
+        if t is not None:
+            assert t.dtype == torch.float32 and t.is_contiguous() and t.numel() == H
+    assert (ln_weight is None) == (ln_bias is None)
+    if bias is not None:
+        assert bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == T * 8
+    codes = torch.empty(B, T, dtype=torch.int32, device=x.device)
+    scores = torch.empty(B, T, dtype=torch.float32, device=x.device)
+    with _dev_guard(x):
+        rc = _lib.load().lffn_ln_bh4_block_hash_f32(
+            _lib.ptr(x), _lib.ptr(ln_weight), _lib.ptr(ln_bias), ln_eps, _lib.ptr(w_folded), _lib.ptr(bias),
+            _lib.ptr(codes), _lib.ptr(scores), B, H, D, R, J, T, bs, decay, residual, _lib.stream_of(x))
+    _lib.check(rc, f"lffn_ln_bh4_block_hash_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T}, block_size={bs})")
+    return codes, scores
+
+
+_L.impl("ln_bh4_block_hash", _ln_bh4_block_hash_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::ln_bh4_block_hash")
+def _(x, ln_weight, ln_bias, ln_eps, w_folded, bias, T, decay, residual):
+    return (torch.empty(x.shape[0], T, dtype=torch.int32, device=x.device),
+            torch.empty(x.shape[0], T, dtype=torch.float32, device=x.device))
+
+
+# ----------------------------------------------------------------------------- mix_code_score
+
+_L.define("mix_code_score(Tensor y, Tensor x, Tensor? bias, int T, int k, int D, float decay, float residual)"
+          " -> (Tensor, Tensor)")
+
+
+def _mix_code_score_impl(y, x, bias, T, k, D, decay, residual):
+    _lib.require_gpu(y, x, bias)
+    assert y.dim() == 2 and x.dim() == 2 and y.shape[0] == x.shape[0]
+    assert y.dtype == torch.float32 and x.dtype == torch.float32
+    assert y.is_contiguous() and x.is_contiguous()
+    B, ldy = y.shape
+    H = x.shape[1]
+    assert H <= D and T * k <= ldy
+    if bias is not None:
+        assert bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == T * k
+    codes = torch.empty(B, T, dtype=torch.int32, device=y.device)
+    scores = torch.empty(B, T, dtype=torch.float32, device=y.device)
+    with _dev_guard(y):
+        rc = _lib.load().lffn_mix_code_score_f32(_lib.ptr(y), _lib.ptr(x), _lib.ptr(bias), _lib.ptr(codes),
+                                                 _lib.ptr(scores), B, T, k, H, D, ldy, decay, residual,
+                                                 _lib.stream_of(y))
+    _lib.check(rc, f"lffn_mix_code_score_f32(B={B}, T={T}, k={k}, H={H}, D={D}, ldy={ldy})")
+    return codes, scores
+
+
+_L.impl("mix_code_score", _mix_code_score_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::mix_code_score")
+def _(y, x, bias, T, k, D, decay, residual):
+    return (torch.empty(y.shape[0], T, dtype=torch.int32, device=y.device),
+            torch.empty(y.shape[0], T, dtype=torch.float32, device=y.device))
+
+
 # ----------------------------------------------------------------------------- project_hash
 
 _L.define("project_hash(Tensor x, Tensor diag, Tensor? bias, int T, float decay, float residual, bool keep_z)"
@@ -454,6 +529,8 @@ fht = torch.ops.lookupffn.fht
 bh4_diag = torch.ops.lookupffn.bh4_diag
 bh4_fold = torch.ops.lookupffn.bh4_fold
 bh4_block = torch.ops.lookupffn.bh4_block
+mix_code_score = torch.ops.lookupffn.mix_code_score
+ln_bh4_block_hash = torch.ops.lookupffn.ln_bh4_block_hash
 project_hash = torch.ops.lookupffn.project_hash
 ln_project_hash = torch.ops.lookupffn.ln_project_hash
 code_score = torch.ops.lookupffn.code_score

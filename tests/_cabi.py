@@ -1,6 +1,8 @@
 """Test helper: call the C ABI of liblookupffn_hip.so directly (ctypes), with
 torch tensors used only as device memory.  Inputs are numpy arrays, outputs come
 back as numpy arrays, so a parity test reads: oracle(numpy) vs cabi(numpy)."""
+import ctypes
+
 import numpy as np
 import torch
 
@@ -65,6 +67,31 @@ def bh4_block(x, w):
     out = torch.full((B, R * NB * bs), float("nan"), dtype=torch.float32, device=DEV)
     _call("lffn_bh4_block_f32", p(xd), p(wf), p(out), B, H, NB * bs, R, J, bs)
     return host(out), host(wf)
+
+
+def ln_bh4_block_hash(x, ln_w, ln_b, eps, w, bias, T, decay=0.7):
+    """fold + the one-kernel front end; w: [R, J, NB, 64, 64]; ln_w None: no LayerNorm."""
+    xd, lw, lb, wd, bd = dev(x), dev(ln_w), dev(ln_b), dev(w), dev(bias)
+    B, H = x.shape
+    R, J, NB, bs, _ = w.shape
+    wf = torch.empty_like(wd)
+    _call("lffn_bh4_fold_f32", p(wd), p(wf), R, J, NB, bs)
+    codes = torch.full((B, T), -1, dtype=torch.int32, device=DEV)
+    scores = torch.full((B, T), float("nan"), dtype=torch.float32, device=DEV)
+    _call("lffn_ln_bh4_block_hash_f32", p(xd), p(lw), p(lb), float(np.float32(eps)), p(wf), p(bd), p(codes), p(scores),
+          B, H, NB * bs, R, J, T, bs, float(np.float32(decay)), float(np.float32(1 - decay)))
+    return host(codes), host(scores)
+
+
+def mix_code_score(y, x, bias, T, k, D, decay=0.7):
+    yd, xd, bd = dev(y), dev(x), dev(bias)
+    B, ldy = y.shape
+    H = x.shape[1]
+    codes = torch.full((B, T), -1, dtype=torch.int32, device=DEV)
+    scores = torch.full((B, T), float("nan"), dtype=torch.float32, device=DEV)
+    _call("lffn_mix_code_score_f32", p(yd), p(xd), p(bd), p(codes), p(scores), B, T, k, H, D, ldy,
+          float(decay), float(1 - decay))
+    return host(codes), host(scores)
 
 
 def project_hash(x, diag, bias, T, decay=0.7, keep_z=True):

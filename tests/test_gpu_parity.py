@@ -161,6 +161,78 @@ def test_bh4_block_exact_on_integers():
     assert np.array_equal(got.astype(np.float64), want)
 
 
+@pytest.mark.parametrize("B,H,D,R,T,k", [(50, 768, 1024, 1, 128, 8), (33, 1024, 1024, 4, 512, 8), (20, 100, 128, 2, 30, 8),
+                                          (17, 256, 256, 1, 21, 12), (9, 64, 64, 3, 48, 4), (5, 30, 32, 1, 3, 7),
+                                          (0, 64, 64, 1, 8, 8)])
+def test_mix_code_score_matches_oracle(B, H, D, R, T, k):
+    rng = np.random.RandomState(B + H + D + R + T + k)
+    y = rng.randn(B, R * D).astype(np.float32)
+    x = rng.randn(B, H).astype(np.float32)
+    bias = (0.05 * rng.randn(T * k)).astype(np.float32)
+    codes, scores = cabi.mix_code_score(y, x, bias, T, k, D)
+    if B == 0:
+        assert codes.shape == (0, T)
+        return
+    xp = np.concatenate([x, np.zeros((B, D - H), np.float32)], axis=1)
+    # PL/lookup.py:36-37 in fp32, operation by operation
+    z = (np.float32(0.7) * y + np.float32(1 - 0.7) * np.tile(xp, (1, R)))[:, :T * k] + bias
+    want_c, want_s = oracle.code_score(z.reshape(B, T, k))
+    assert np.array_equal(codes, want_c)
+    np.testing.assert_allclose(scores, want_s, rtol=2e-6)
+    # without bias
+    codes0, scores0 = cabi.mix_code_score(y, x, None, T, k, D)
+    z0 = (np.float32(0.7) * y + np.float32(1 - 0.7) * np.tile(xp, (1, R)))[:, :T * k]
+    want_c0, want_s0 = oracle.code_score(z0.reshape(B, T, k))
+    assert np.array_equal(codes0, want_c0)
+    np.testing.assert_allclose(scores0, want_s0, rtol=2e-6)
+
+
+@pytest.mark.parametrize("B,H,D,R,T,with_ln", [(100, 768, 1024, 1, 128, True), (70, 1024, 1024, 4, 512, True),
+                                                (45, 256, 256, 1, 32, False), (33, 100, 128, 2, 30, True),
+                                                (64, 512, 512, 2, 100, False), (1, 64, 64, 1, 8, True),
+                                                (0, 64, 64, 1, 8, True)])
+def test_ln_bh4_block_hash_matches_oracle(B, H, D, R, T, with_ln):
+    """(LayerNorm ->) BH4 with 64 x 64 blocks -> mix -> hash in one kernel, against the float64
+    oracle: y is rounded differently from the reference's order (1e-5), so a code may differ
+    only where the true z is that close to 0; scores are compared where the codes agree."""
+    rng = np.random.RandomState(B + H + D + R + T)
+    J, NB = 4, D // 64
+    x = (rng.randn(B, H) * 1.5 + 0.3).astype(np.float32)
+    ln_w = (1 + 0.1 * rng.randn(H)).astype(np.float32) if with_ln else None
+    ln_b = (0.1 * rng.randn(H)).astype(np.float32) if with_ln else None
+    w = (rng.randn(R, J, NB, 64, 64) / math.sqrt(64 * D)).astype(np.float32)
+    bias = (0.05 * rng.randn(T * 8)).astype(np.float32)
+    codes, scores = cabi.ln_bh4_block_hash(x, ln_w, ln_b, 1e-5, w, bias, T)
+    if B == 0:
+        assert codes.shape == (0, T)
+        return
+    h64 = oracle.layernorm(x.astype(np.float64), ln_w, ln_b, 1e-5) if with_ln else x.astype(np.float64)
+    z64 = oracle.projection(h64, w.astype(np.float64), bias.astype(np.float64), T * 8, 0.7).reshape(B, T, 8)
+    code64, score64 = oracle.code_score(z64)
+    scale = np.abs(z64).max()
+    assert (codes >= 0).all() and not np.isnan(scores).any()          # every entry written
+    same = codes == code64
+    assert same.mean() >= 0.995
+    # where a code differs, some z of that group is within rounding of zero
+    assert np.all(np.abs(z64[~same]).min(axis=-1) <= 2e-5 * scale)
+    np.testing.assert_allclose(scores[same], score64[same], rtol=3e-4)
+    # the same codes and scores as the three-step path on the GPU (LayerNorm in torch, the BH4
+    # kernel, the mix + hash kernel) wherever those codes agree with the truth
+    if with_ln:
+        h_gpu = torch.nn.functional.layer_norm(torch.tensor(x, device="cuda:0"), (H,),
+                                               torch.tensor(ln_w, device="cuda:0"),
+                                               torch.tensor(ln_b, device="cuda:0"), 1e-5).cpu().numpy()
+    else:
+        h_gpu = x
+    y, _ = cabi.bh4_block(h_gpu, w)
+    c3, s3 = cabi.mix_code_score(y, h_gpu, bias, T, 8, D)
+    both = same & (c3 == code64)
+    np.testing.assert_allclose(scores[both], s3[both], rtol=1e-4)
+    if not with_ln:
+        # identical inputs to the identical operations: bit for bit
+        assert np.array_equal(codes, c3) and np.array_equal(scores, s3)
+
+
 def test_sign_diagonal_fht_exact():
     # the BASELINE "random +-1 sign diagonal from seed": one round, exact on integers
     rng = np.random.RandomState(8)
