@@ -59,7 +59,8 @@ WORKLOADS = {
 # HBM bytes per launch of the gather kernel measured with rocprofv3 --pmc
 # (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); the summaries
 # are kept under profiles/.  None until measured for that workload.
-MEASURED_TRAFFIC_BYTES = {"cfg2": 477412788, "cfg3": 3169016070, "cfg3bf16": 2250808112, "cfg5": 504127966}
+MEASURED_TRAFFIC_BYTES = {"cfg2": 477559591, "cfg2b64": 477451647, "cfg3": 3156050546, "cfg3bf16": 2252934839,
+                          "cfg5": 504064321}
 
 
 def build_layer(wl, device):
