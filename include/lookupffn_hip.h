@@ -210,6 +210,21 @@ int lffn_lookup_gather_bf16(const int32_t *code, const float *score, const uint1
                             int64_t B, int64_t T, int64_t S, int64_t Do, void *stream);
 
 /*
+ * lffn_lookup_gather_{f32,bf16} with a residual added to the result:
+ *   out[b,:] = residual[b,:] + bias + sum_t score[b,t] * tables[t, code[b,t] & (S-1), :]
+ * residual: [B, Do] fp32 or NULL; it may be the output buffer itself (every element is read
+ * and then written by the same lane).  Replaces, in addition, the residual add of the
+ * encoder layer around the FFN, "self.dropout(self.FFN(x)) + x" (PL/layer.py:77), where
+ * dropout is the identity (eval mode or p == 0).
+ */
+int lffn_lookup_gather_residual_f32(const int32_t *code, const float *score, const float *tables,
+                                    const float *bias, const float *residual, float *out,
+                                    int64_t B, int64_t T, int64_t S, int64_t Do, void *stream);
+int lffn_lookup_gather_residual_bf16(const int32_t *code, const float *score, const uint16_t *tables,
+                                     const float *bias, const float *residual, float *out,
+                                     int64_t B, int64_t T, int64_t S, int64_t Do, void *stream);
+
+/*
  * Which kernel lffn_lookup_gather_{f32,bf16} runs for a shape.  Returns the number
  * of tokens whose accumulators one workgroup keeps in registers while it walks the
  * tables through LDS, or 0 when the token-major kernel is used (small batches,

@@ -45,6 +45,8 @@ SIGNATURES = {
     "lffn_gather_add_bf16": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "lffn_lookup_gather_f32": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "lffn_lookup_gather_bf16": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
+    "lffn_lookup_gather_residual_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
+    "lffn_lookup_gather_residual_bf16": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "lffn_lookup_gather_planned_f32": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
                                        ctypes.c_int32, ctypes.c_int32, _vp],
     "lffn_lookup_gather_planned_bf16": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,

@@ -56,6 +56,7 @@ struct GatherArgs {
     const float *w;       // [B, I]
     const float *g;       // [B, Dv]   (backward kernels)
     const float *bias;    // [Dv] or null (structured forward)
+    const float *residual;// [B, Dv] or null (structured forward): added to the result
     float *out;
     int64_t B;
     int I;
@@ -162,9 +163,15 @@ __global__ __launch_bounds__(256) void gather_add_kernel(GatherArgs a) {
 #pragma unroll
         for (int v = 0; v < NV; ++v)
 #pragma unroll
-            for (int q = 0; q < EPV / 4; ++q)
-                *reinterpret_cast<float4 *>(o + (size_t)(vec0 + v * LPT) * EPV + 4 * q) =
-                    make_float4(acc[v][4 * q + 0], acc[v][4 * q + 1], acc[v][4 * q + 2], acc[v][4 * q + 3]);
+            for (int q = 0; q < EPV / 4; ++q) {
+                const size_t c0 = (size_t)(vec0 + v * LPT) * EPV + 4 * q;
+                float4 r4 = make_float4(acc[v][4 * q + 0], acc[v][4 * q + 1], acc[v][4 * q + 2], acc[v][4 * q + 3]);
+                if (a.residual) {
+                    const float4 rr = *reinterpret_cast<const float4 *>(a.residual + tok * a.Dv + c0);
+                    r4.x += rr.x; r4.y += rr.y; r4.z += rr.z; r4.w += rr.w;
+                }
+                *reinterpret_cast<float4 *>(o + c0) = r4;
+            }
     }
 }
 
@@ -358,14 +365,15 @@ int check_common(const void *idx, int64_t B, int64_t I, int64_t rows, int64_t Dv
 }
 
 template <bool BF16>
-int gather_entry(const int32_t *idx, const void *src, const float *w, const float *bias, float *out,
+int gather_entry(const int32_t *idx, const void *src, const float *w, const float *bias, const float *residual,
+                 float *out,
                  int64_t B, int64_t I, int64_t rows, int64_t Dv, int64_t S, void *stream) {
     int rc = check_common(idx, B, I, rows, Dv);
     if (rc != LFFN_OK) return rc;
     LFFN_REQUIRE(src && out && (w || B * I == 0), LFFN_ERR_BAD_ARG);
     LFFN_REQUIRE(lffn_aligned16(src) && lffn_aligned16(out) && (!bias || lffn_aligned16(bias)), LFFN_ERR_BAD_ARG);
     GatherArgs a{};
-    a.idx = idx; a.src = src; a.w = w; a.g = nullptr; a.bias = bias; a.out = out;
+    a.idx = idx; a.src = src; a.w = w; a.g = nullptr; a.bias = bias; a.residual = residual; a.out = out;
     a.B = B; a.I = (int)I; a.source_size = rows; a.Dv = (int)Dv; a.S = (int)S;
     return launch<BF16, Op::Gather>(a, static_cast<hipStream_t>(stream));
 }
@@ -374,23 +382,23 @@ int gather_entry(const int32_t *idx, const void *src, const float *w, const floa
 
 extern "C" int lffn_gather_add_f32(const int32_t *idx, const float *src, const float *w, float *out,
                                    int64_t B, int64_t I, int64_t source_size, int64_t Dv, void *stream) {
-    return gather_entry<false>(idx, src, w, nullptr, out, B, I, source_size, Dv, 0, stream);
+    return gather_entry<false>(idx, src, w, nullptr, nullptr, out, B, I, source_size, Dv, 0, stream);
 }
 
 extern "C" int lffn_gather_add_bf16(const int32_t *idx, const uint16_t *src, const float *w, float *out,
                                     int64_t B, int64_t I, int64_t source_size, int64_t Dv, void *stream) {
-    return gather_entry<true>(idx, src, w, nullptr, out, B, I, source_size, Dv, 0, stream);
+    return gather_entry<true>(idx, src, w, nullptr, nullptr, out, B, I, source_size, Dv, 0, stream);
 }
 
 // Token-major kernel on table-local codes (offset i*S and bias folded in): the
 // form lookup_gather.hip falls back to for shapes its LDS-tiled kernel is not
 // built for.
 int lffn_internal_lookup_gather_token_major(const int32_t *code, const float *score, const void *tables,
-                                            const float *bias, float *out, int64_t B, int64_t T, int64_t S,
-                                            int64_t Do, bool bf16, void *stream) {
+                                            const float *bias, const float *residual, float *out, int64_t B,
+                                            int64_t T, int64_t S, int64_t Do, bool bf16, void *stream) {
     const int64_t rows = T * S > 0 ? T * S : 1;
-    return bf16 ? gather_entry<true>(code, tables, score, bias, out, B, T, rows, Do, S, stream)
-                : gather_entry<false>(code, tables, score, bias, out, B, T, rows, Do, S, stream);
+    return bf16 ? gather_entry<true>(code, tables, score, bias, residual, out, B, T, rows, Do, S, stream)
+                : gather_entry<false>(code, tables, score, bias, residual, out, B, T, rows, Do, S, stream);
 }
 
 // Atomic scatter-add on table-local codes (row = code & (S-1) + t*S), into a buffer

@@ -27,8 +27,8 @@ static inline int lffn_log2(int64_t v) {
 // gather.hip: token-major gather on table-local codes (not exported)
 __attribute__((visibility("hidden")))
 int lffn_internal_lookup_gather_token_major(const int32_t *code, const float *score, const void *tables,
-                                            const float *bias, float *out, int64_t B, int64_t T, int64_t S,
-                                            int64_t Do, bool bf16, void *stream);
+                                            const float *bias, const float *residual, float *out, int64_t B,
+                                            int64_t T, int64_t S, int64_t Do, bool bf16, void *stream);
 
 // gather.hip: atomic scatter-add on table-local codes (not exported)
 __attribute__((visibility("hidden")))
@@ -44,8 +44,8 @@ int lffn_internal_lookup_inner_token_major(const int32_t *code, const float *g, 
 // lookup_gather_pair.hip: the two-tables-per-buffer LDS gather (not exported)
 __attribute__((visibility("hidden")))
 int lffn_internal_lookup_gather_pair(const int32_t *code, const float *score, const void *tables,
-                                     const float *bias, float *out, int64_t B, int64_t T, int64_t S,
-                                     int64_t Do, bool bf16, int np, void *stream);
+                                     const float *bias, const float *residual, float *out, int64_t B, int64_t T,
+                                     int64_t S, int64_t Do, bool bf16, int np, void *stream);
 
 static inline int lffn_launch_status() {
     return hipGetLastError() == hipSuccess ? LFFN_OK : LFFN_ERR_LAUNCH;

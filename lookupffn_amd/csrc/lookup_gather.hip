@@ -44,6 +44,7 @@ struct LdsGatherArgs {
     const float *score;    // [B, T]
     const char *tables;    // [T, S, Do] fp32 or bf16
     const float *bias;     // [Do] or null
+    const float *residual; // [B, Do] or null: added to the result (may be the output buffer)
     float *out;            // [B, Do]
     int64_t B;
     int T, S, Do;
@@ -223,11 +224,17 @@ __global__ __launch_bounds__(WG) void lookup_gather_lds_kernel(LdsGatherArgs a) 
     for (int p = 0; p < NP; ++p) {
         const int64_t tok = tok0 + p * 64;
         if (tok < a.B) {
-            float *o = a.out + tok * a.Do + (size_t)slice * (SEG_VECS * EPV) + j * EPV;
+            const size_t off = tok * a.Do + (size_t)slice * (SEG_VECS * EPV) + j * EPV;
+            float *o = a.out + off;
 #pragma unroll
-            for (int q = 0; q < EPV / 4; ++q)
-                *reinterpret_cast<float4 *>(o + 4 * q) =
-                    make_float4(acc[p][4 * q], acc[p][4 * q + 1], acc[p][4 * q + 2], acc[p][4 * q + 3]);
+            for (int q = 0; q < EPV / 4; ++q) {
+                float4 v = make_float4(acc[p][4 * q], acc[p][4 * q + 1], acc[p][4 * q + 2], acc[p][4 * q + 3]);
+                if (a.residual) {
+                    const float4 rr = *reinterpret_cast<const float4 *>(a.residual + off + 4 * q);
+                    v.x += rr.x; v.y += rr.y; v.z += rr.z; v.w += rr.w;
+                }
+                *reinterpret_cast<float4 *>(o + 4 * q) = v;
+            }
         }
     }
 }
@@ -311,14 +318,15 @@ bool plan_is_valid(const GatherPlan &p, int64_t B, int64_t T, int64_t S, int64_t
 // requested kernel (kind_req tables per buffer, tokens_req tokens per workgroup).
 template <bool BF16>
 int lookup_gather_entry(const int32_t *code, const float *score, const void *tables, const float *bias,
-                        float *out, int64_t B, int64_t T, int64_t S, int64_t Do, int kind_req, int tokens_req,
+                        const float *residual, float *out, int64_t B, int64_t T, int64_t S, int64_t Do, int kind_req, int tokens_req,
                         void *stream) {
     LFFN_REQUIRE(B >= 0 && T >= 0 && Do >= 1, LFFN_ERR_BAD_ARG);
     LFFN_REQUIRE(lffn_is_pow2(S) && S <= (1 << 24) && T * S <= 0x7fffffff, LFFN_ERR_UNSUPPORTED);
     LFFN_REQUIRE(Do % 64 == 0 && Do <= (1 << 20) && T <= (1 << 24), LFFN_ERR_UNSUPPORTED);
     LFFN_REQUIRE(B <= (int64_t(1) << 31) - 1, LFFN_ERR_UNSUPPORTED);
     LFFN_REQUIRE(tables && out && ((code && score) || B * T == 0), LFFN_ERR_BAD_ARG);
-    LFFN_REQUIRE(lffn_aligned16(tables) && lffn_aligned16(out) && (!bias || lffn_aligned16(bias)), LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_aligned16(tables) && lffn_aligned16(out) && (!bias || lffn_aligned16(bias)) &&
+                     (!residual || lffn_aligned16(residual)), LFFN_ERR_BAD_ARG);
     if (B == 0) return LFFN_OK;
     GatherPlan plan;
     if (kind_req < 0) {
@@ -331,12 +339,12 @@ int lookup_gather_entry(const int32_t *code, const float *score, const void *tab
         LFFN_REQUIRE(plan_is_valid<BF16>(plan, B, T, S, Do), LFFN_ERR_UNSUPPORTED);
     }
     if (plan.kind == 0)
-        return lffn_internal_lookup_gather_token_major(code, score, tables, bias, out, B, T, S, Do, BF16, stream);
+        return lffn_internal_lookup_gather_token_major(code, score, tables, bias, residual, out, B, T, S, Do, BF16, stream);
     if (plan.kind == 2)
-        return lffn_internal_lookup_gather_pair(code, score, tables, bias, out, B, T, S, Do, BF16, plan.np, stream);
+        return lffn_internal_lookup_gather_pair(code, score, tables, bias, residual, out, B, T, S, Do, BF16, plan.np, stream);
     const int np = plan.np;
     LdsGatherArgs a{};
-    a.code = code; a.score = score; a.tables = static_cast<const char *>(tables); a.bias = bias; a.out = out;
+    a.code = code; a.score = score; a.tables = static_cast<const char *>(tables); a.bias = bias; a.residual = residual; a.out = out;
     a.B = B; a.T = (int)T; a.S = (int)S; a.Do = (int)Do;
     a.nslices = (int)(Do / (BF16 ? 128 : 64));
     a.row_bytes = (int)(Do * (BF16 ? 2 : 4));
@@ -358,13 +366,25 @@ int lookup_gather_entry(const int32_t *code, const float *score, const void *tab
 extern "C" int lffn_lookup_gather_f32(const int32_t *code, const float *score, const float *tables,
                                       const float *bias, float *out,
                                       int64_t B, int64_t T, int64_t S, int64_t Do, void *stream) {
-    return lookup_gather_entry<false>(code, score, tables, bias, out, B, T, S, Do, -1, 0, stream);
+    return lookup_gather_entry<false>(code, score, tables, bias, nullptr, out, B, T, S, Do, -1, 0, stream);
 }
 
 extern "C" int lffn_lookup_gather_bf16(const int32_t *code, const float *score, const uint16_t *tables,
                                        const float *bias, float *out,
                                        int64_t B, int64_t T, int64_t S, int64_t Do, void *stream) {
-    return lookup_gather_entry<true>(code, score, tables, bias, out, B, T, S, Do, -1, 0, stream);
+    return lookup_gather_entry<true>(code, score, tables, bias, nullptr, out, B, T, S, Do, -1, 0, stream);
+}
+
+extern "C" int lffn_lookup_gather_residual_f32(const int32_t *code, const float *score, const float *tables,
+                                               const float *bias, const float *residual, float *out,
+                                               int64_t B, int64_t T, int64_t S, int64_t Do, void *stream) {
+    return lookup_gather_entry<false>(code, score, tables, bias, residual, out, B, T, S, Do, -1, 0, stream);
+}
+
+extern "C" int lffn_lookup_gather_residual_bf16(const int32_t *code, const float *score, const uint16_t *tables,
+                                                const float *bias, const float *residual, float *out,
+                                                int64_t B, int64_t T, int64_t S, int64_t Do, void *stream) {
+    return lookup_gather_entry<true>(code, score, tables, bias, residual, out, B, T, S, Do, -1, 0, stream);
 }
 
 extern "C" int lffn_lookup_gather_planned_f32(const int32_t *code, const float *score, const float *tables,
@@ -372,7 +392,7 @@ extern "C" int lffn_lookup_gather_planned_f32(const int32_t *code, const float *
                                               int64_t B, int64_t T, int64_t S, int64_t Do,
                                               int32_t tables_per_buffer, int32_t tokens_per_workgroup, void *stream) {
     LFFN_REQUIRE(tables_per_buffer >= 0, LFFN_ERR_BAD_ARG);
-    return lookup_gather_entry<false>(code, score, tables, bias, out, B, T, S, Do, tables_per_buffer,
+    return lookup_gather_entry<false>(code, score, tables, bias, nullptr, out, B, T, S, Do, tables_per_buffer,
                                       tokens_per_workgroup, stream);
 }
 
@@ -381,7 +401,7 @@ extern "C" int lffn_lookup_gather_planned_bf16(const int32_t *code, const float 
                                                int64_t B, int64_t T, int64_t S, int64_t Do,
                                                int32_t tables_per_buffer, int32_t tokens_per_workgroup, void *stream) {
     LFFN_REQUIRE(tables_per_buffer >= 0, LFFN_ERR_BAD_ARG);
-    return lookup_gather_entry<true>(code, score, tables, bias, out, B, T, S, Do, tables_per_buffer,
+    return lookup_gather_entry<true>(code, score, tables, bias, nullptr, out, B, T, S, Do, tables_per_buffer,
                                      tokens_per_workgroup, stream);
 }
 

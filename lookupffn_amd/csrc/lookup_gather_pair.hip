@@ -42,6 +42,7 @@ struct PairArgs {
     const float *score;    // [B, T]
     const char *tables;    // [T, S, Do] fp32 or bf16
     const float *bias;     // [Do] or null
+    const float *residual; // [B, Do] or null: added to the result (may be the output buffer)
     float *out;            // [B, Do]
     int64_t B;
     int T, S, Do;
@@ -238,11 +239,17 @@ __global__ __launch_bounds__(WG) void lookup_gather_pair_kernel(PairArgs a) {
     for (int p = 0; p < NP; ++p) {
         const int64_t tok = tok0 + p * 128;
         if (tok < a.B) {
-            float *o = a.out + tok * a.Do + (size_t)slice * (8 * EPV) + j * EPV;
+            const size_t off = tok * a.Do + (size_t)slice * (8 * EPV) + j * EPV;
+            float *o = a.out + off;
 #pragma unroll
-            for (int q = 0; q < EPV / 4; ++q)
-                *reinterpret_cast<float4 *>(o + 4 * q) =
-                    make_float4(acc[p][4 * q], acc[p][4 * q + 1], acc[p][4 * q + 2], acc[p][4 * q + 3]);
+            for (int q = 0; q < EPV / 4; ++q) {
+                float4 v = make_float4(acc[p][4 * q], acc[p][4 * q + 1], acc[p][4 * q + 2], acc[p][4 * q + 3]);
+                if (a.residual) {
+                    const float4 rr = *reinterpret_cast<const float4 *>(a.residual + off + 4 * q);
+                    v.x += rr.x; v.y += rr.y; v.z += rr.z; v.w += rr.w;
+                }
+                *reinterpret_cast<float4 *>(o + 4 * q) = v;
+            }
         }
     }
 }
@@ -274,10 +281,11 @@ int launch_pair(const PairArgs &a, hipStream_t stream) {
 // that the shape qualifies: S <= 256, Do a multiple of the 128-byte slice width
 // (32 fp32 / 64 bf16 columns), B*T < 2^31, np one of {4, 8, 13, 16} (fp32) or {4, 8} (bf16).
 int lffn_internal_lookup_gather_pair(const int32_t *code, const float *score, const void *tables,
-                                     const float *bias, float *out, int64_t B, int64_t T, int64_t S,
+                                     const float *bias, const float *residual, float *out, int64_t B, int64_t T,
+                                     int64_t S,
                                      int64_t Do, bool bf16, int np, void *stream) {
     PairArgs a{};
-    a.code = code; a.score = score; a.tables = static_cast<const char *>(tables); a.bias = bias; a.out = out;
+    a.code = code; a.score = score; a.tables = static_cast<const char *>(tables); a.bias = bias; a.residual = residual; a.out = out;
     a.B = B; a.T = (int)T; a.S = (int)S; a.Do = (int)Do;
     a.nslices = (int)(Do / (bf16 ? 64 : 32));
     a.row_bytes = (int)(Do * (bf16 ? 2 : 4));

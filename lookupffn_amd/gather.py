@@ -131,14 +131,17 @@ def gather(indices, weights, tables, training):
 class LookupGather(Function):
     """The gather as the layer issues it (PL/lookup.py:120-130): codes are table-local,
     the offset ``arange(T) * S`` and the output bias (PL/lookup.py:108) are folded
-    into the kernel.  Gradients: tables, scores and bias."""
+    into the kernel, as is an optional residual [B, Do] added to the result.  Gradients: tables,
+    scores, bias and residual."""
 
     @staticmethod
-    def forward(ctx, code, score, tables, bias):
+    def forward(ctx, code, score, tables, bias, residual):
         code, score, tables = code.contiguous(), score.contiguous(), tables.contiguous()
         ctx.save_for_backward(code, score, tables)
         ctx.has_bias = bias is not None
-        return ops.lookup_gather(code, score, tables, None if bias is None else bias.contiguous())
+        ctx.has_residual = residual is not None
+        return ops.lookup_gather(code, score, tables, None if bias is None else bias.contiguous(),
+                                 None if residual is None else residual.contiguous())
 
     @staticmethod
     def backward(ctx, grad_outputs):
@@ -150,10 +153,11 @@ class LookupGather(Function):
         grad_score = ops.lookup_inner(code, grad_outputs, tables) if ctx.needs_input_grad[1] else None
         grad_tables = ops.lookup_scatter(code, score, grad_outputs, S) if ctx.needs_input_grad[2] else None
         grad_bias = grad_outputs.sum(dim=0) if (ctx.has_bias and ctx.needs_input_grad[3]) else None
-        return None, grad_score, grad_tables, grad_bias
+        grad_residual = grad_outputs if (ctx.has_residual and ctx.needs_input_grad[4]) else None
+        return None, grad_score, grad_tables, grad_bias, grad_residual
 
 
-def lookup_gather(code, score, tables, bias=None):
+def lookup_gather(code, score, tables, bias=None, residual=None):
     if not (code.is_cuda and score.is_cuda and tables.is_cuda):
         raise RuntimeError("lookup_gather: lookupffn_amd runs on the GPU only (got a CPU tensor)")
-    return LookupGather.apply(code, score, tables, bias)
+    return LookupGather.apply(code, score, tables, bias, residual)

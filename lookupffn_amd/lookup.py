@@ -174,7 +174,7 @@ class LookupFFN(nn.Module):
         return (f"hidden_size={self.hidden_size}, num_table={self.num_table}, "
                 f"table_size={self.table_size}, output_size={self.output_size}")
 
-    def _forward(self, hidden_states):
+    def _forward(self, hidden_states, residual=None):
         ln = self.LayerNorm
         ln_fusable = (ln.elementwise_affine and ln.weight is not None and ln.bias is not None
                       and ln.weight.dtype == torch.float32
@@ -189,15 +189,20 @@ class LookupFFN(nn.Module):
             code, score = self.hash(hidden_states)
         if self.output_size % 64 == 0 and self.tables.dtype in (torch.float32, torch.bfloat16):
             # table-local codes, offset and bias folded into the gather kernel
-            return lookup_gather(code, score.float(), self.tables, self.bias.float())
+            return lookup_gather(code, score.float(), self.tables, self.bias.float(), residual)
         outputs = self.gather(code, score, self.tables)
-        return outputs + self.bias
+        outputs = outputs + self.bias
+        return outputs if residual is None else outputs + residual
 
-    def forward(self, hidden_states):
+    def forward(self, hidden_states, residual=None):
+        """PL/lookup.py:110-118.  ``residual`` (not in the reference; shape [..., output_size]) is
+        added to the result inside the gather kernel: the encoder layer's "FFN(x) + x"."""
         shape = hidden_states.shape[:-1]
         dim = hidden_states.shape[-1]
         hidden_states = hidden_states.reshape(int(np.prod(shape)), dim)
-        outputs = self._forward(hidden_states)
+        if residual is not None:
+            residual = residual.reshape(int(np.prod(shape)), self.output_size).float()
+        outputs = self._forward(hidden_states, residual)
         return outputs.reshape(*shape, self.output_size)
 
     def gather(self, indexes, weights, tables):

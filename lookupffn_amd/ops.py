@@ -375,11 +375,11 @@ def _(indexes, source, weights):
     return weights.new_empty(indexes.shape[0], source.shape[1])
 
 
-_L.define("lookup_gather(Tensor code, Tensor score, Tensor tables, Tensor? bias) -> Tensor")
+_L.define("lookup_gather(Tensor code, Tensor score, Tensor tables, Tensor? bias, Tensor? residual=None) -> Tensor")
 
 
-def _lookup_gather_impl(code, score, tables, bias):
-    _lib.require_gpu(code, score, tables, bias)
+def _lookup_gather_impl(code, score, tables, bias, residual=None):
+    _lib.require_gpu(code, score, tables, bias, residual)
     assert tables.dim() == 3 and tables.is_contiguous()
     assert score.dtype == torch.float32 and score.is_contiguous()
     assert tuple(score.shape) == tuple(code.shape)
@@ -389,16 +389,18 @@ def _lookup_gather_impl(code, score, tables, bias):
     _check_gather_args(code, T * S, Do)
     if bias is not None:
         assert bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == Do
+    if residual is not None:
+        assert residual.dtype == torch.float32 and residual.is_contiguous() and tuple(residual.shape) == (B, Do)
     out = torch.empty(B, Do, dtype=torch.float32, device=tables.device)
     lib = _lib.load()
     if tables.dtype == torch.float32:
-        fn, name = lib.lffn_lookup_gather_f32, "lffn_lookup_gather_f32"
+        fn, name = lib.lffn_lookup_gather_residual_f32, "lffn_lookup_gather_residual_f32"
     elif tables.dtype == torch.bfloat16:
-        fn, name = lib.lffn_lookup_gather_bf16, "lffn_lookup_gather_bf16"
+        fn, name = lib.lffn_lookup_gather_residual_bf16, "lffn_lookup_gather_residual_bf16"
     else:
         raise NotImplementedError(f"lookup_gather: table dtype {tables.dtype} (float32 and bfloat16 are built)")
     with _dev_guard(tables):
-        rc = fn(_lib.ptr(code), _lib.ptr(score), _lib.ptr(tables), _lib.ptr(bias), _lib.ptr(out),
+        rc = fn(_lib.ptr(code), _lib.ptr(score), _lib.ptr(tables), _lib.ptr(bias), _lib.ptr(residual), _lib.ptr(out),
                 B, T, S, Do, _lib.stream_of(tables))
     _lib.check(rc, f"{name}(B={B}, T={T}, S={S}, Do={Do})")
     return out
@@ -408,7 +410,7 @@ _L.impl("lookup_gather", _lookup_gather_impl, "CUDA")
 
 
 @torch.library.register_fake("lookupffn::lookup_gather")
-def _(code, score, tables, bias):
+def _(code, score, tables, bias, residual=None):
     return score.new_empty(code.shape[0], tables.shape[2])
 
 

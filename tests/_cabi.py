@@ -145,13 +145,21 @@ def gather_add(idx, src, w, bf16=False):
     return host(out)
 
 
-def lookup_gather(code, score, tables, bias=None, bf16=False, plan=None):
-    """plan = (tables_per_buffer, tokens_per_workgroup) runs exactly that kernel."""
+def lookup_gather(code, score, tables, bias=None, bf16=False, plan=None, residual=None, in_place=False):
+    """plan = (tables_per_buffer, tokens_per_workgroup) runs exactly that kernel; residual [B, Do] is
+    added inside the kernel (in_place: the residual buffer is also the output)."""
     cd, sd, td, bd = dev(code), dev(score), dev(tables), dev(bias)
     B, T = code.shape
     _, S, Do = tables.shape
     out = torch.full((B, Do), float("nan"), dtype=torch.float32, device=DEV)
-    if plan is None:
+    if residual is not None:
+        assert plan is None
+        rd = dev(residual)
+        if in_place:
+            out = rd
+        _call("lffn_lookup_gather_residual_bf16" if bf16 else "lffn_lookup_gather_residual_f32",
+              p(cd), p(sd), p(td), p(bd), p(rd), p(out), B, T, S, Do)
+    elif plan is None:
         _call("lffn_lookup_gather_bf16" if bf16 else "lffn_lookup_gather_f32",
               p(cd), p(sd), p(td), p(bd), p(out), B, T, S, Do)
     else:

@@ -195,6 +195,24 @@ def test_reference_call_sequence_of_lookup_gather():
     assert relmax(npf(a), npf(b)) <= 1e-6
 
 
+def test_layer_residual_argument_and_gradients():
+    """LookupFFN(x, residual=r) == LookupFFN(x) + r, and the gradient reaches r unchanged."""
+    torch.manual_seed(11)
+    layer = lookupffn_amd.LookupFFN(_config(hidden_size=256, ffn_num_table=32), 256).to(DEV)
+    x = torch.randn(4, 33, 256, device=DEV)
+    r = torch.randn(4, 33, 256, device=DEV, requires_grad=True)
+    layer.eval()
+    with torch.no_grad():
+        assert torch.equal(layer(x, residual=r), layer(x) + r)
+    layer.train()
+    out = layer(x, residual=r)
+    g = torch.randn_like(out)
+    out.backward(g)
+    assert torch.equal(r.grad, g)
+    ref = layer(x) + r.detach()
+    assert relmax(npf(out), npf(ref)) <= 1e-6
+
+
 def test_encoder_layers_match_float64_composition():
     """The pre-norm encoder with LookupFFN (PL/layer.py:66-78, PL/encoder.py:9-37): each
     layer's output on the GPU against attention evaluated in float64 with the literal

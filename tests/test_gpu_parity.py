@@ -405,6 +405,32 @@ def test_gather_add_matches_oracle(B, T, S, Do):
         assert relmax(cabi.lookup_gather(code, w, tables, bias), want64 + bias) <= 1e-5
 
 
+# (B, T, S, Do, bf16): shapes that the planner sends to the token-major kernel (0 tables per
+# buffer), the one-table LDS kernel (1) and the two-table LDS kernel (2)
+RESIDUAL_CASES = [(300, 20, 256, 256, False, 0), (16384, 8, 256, 768, False, 1), (4000, 12, 256, 768, False, 2),
+                  (8192, 16, 256, 768, True, 2), (500, 6, 64, 128, True, 0)]
+
+
+@pytest.mark.parametrize("B,T,S,Do,bf16,kind", RESIDUAL_CASES)
+def test_lookup_gather_residual(B, T, S, Do, bf16, kind):
+    assert cabi.lookup_gather_plan(B, T, S, Do, bf16)[0] == kind
+    rng = np.random.RandomState(B + T + Do + 5)
+    tables, code, idx, w = _rand_gather(rng, B, T, S, Do)
+    bias = (0.001 * rng.randn(Do)).astype(np.float32)
+    res = rng.randn(B, Do).astype(np.float32)
+    tb = oracle.bf16_round(tables.reshape(T * S, Do)).reshape(T, S, Do) if bf16 else tables
+    plain = cabi.lookup_gather(code, w, tb, bias, bf16=bf16)
+    got = cabi.lookup_gather(code, w, tb, bias, bf16=bf16, residual=res)
+    # the residual is one more fp32 addition on top of the plain result, element by element
+    assert np.array_equal(got, plain + res)
+    # in place: the residual buffer is the output buffer
+    assert np.array_equal(cabi.lookup_gather(code, w, tb, bias, bf16=bf16, residual=res, in_place=True), got)
+    # and the sum against the float64 oracle
+    flat = oracle.bf16_widen(tb.reshape(T * S, Do)) if bf16 else tb.reshape(T * S, Do)
+    want = oracle.gather_add(idx, flat.astype(np.float64), w.astype(np.float64)) + bias + res
+    assert relmax(got, want) <= 1e-5
+
+
 @pytest.mark.parametrize("B,T,S,Do", GATHER_CASES)
 def test_gather_add_bf16_matches_oracle(B, T, S, Do):
     rng = np.random.RandomState(B + T + Do + 1)
