@@ -59,6 +59,17 @@ const char *lffn_error_string(int code);
 int lffn_fht_f32(const float *in, float *out, int64_t B, int64_t D, void *stream);
 
 /*
+ * The same transform on rows stored as IEEE half (f16) or bfloat16 (bf16), raw 16-bit
+ * patterns: values are widened on load, all butterflies run in fp32, the result is
+ * rounded to nearest even once on the store.  in == out is allowed; 8-byte alignment.
+ * Takes the place of fast_hadamard_transform_dim512_fp16 / _dim1024_fp16
+ * (fast_hadamard_transform/extension/cuda_launch.cu:12-54, kernels cuda_kernel.cu:19-216),
+ * which exist for D = 512 and 1024 only and round in half precision after every stage.
+ */
+int lffn_fht_f16(const uint16_t *in, uint16_t *out, int64_t B, int64_t D, void *stream);
+int lffn_fht_bf16(const uint16_t *in, uint16_t *out, int64_t B, int64_t D, void *stream);
+
+/*
  * BH4 mixing with block size 1 (a diagonal scale before every transform):
  *   for r < R:  y = pad(x);  for j < J:  y = FHT(diag[r,j,:] * y);  out[b, r*D:(r+1)*D] = y
  * x: [B, H] with H <= D (zero-padded on load, PL/lookup.py:32-34); diag: [R, J, D];

@@ -29,6 +29,8 @@ _f32 = ctypes.c_float
 # name -> argument types (every entry point returns int except the two below)
 SIGNATURES = {
     "lffn_fht_f32": [_vp, _vp, _i64, _i64, _vp],
+    "lffn_fht_f16": [_vp, _vp, _i64, _i64, _vp],
+    "lffn_fht_bf16": [_vp, _vp, _i64, _i64, _vp],
     "lffn_bh4_diag_f32": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp],
     "lffn_mix_code_score_f32": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64,
                                 ctypes.c_float, ctypes.c_float, _vp],

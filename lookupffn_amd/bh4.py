@@ -34,21 +34,28 @@ def fast_hadamard_transform(X: torch.Tensor) -> torch.Tensor:
     """out = X @ H_D, unnormalised, natural order (fast_hadamard_transform/kernel.py:39-45)."""
     assert X.is_contiguous()
     assert len(X.shape) == 2
-    assert X.dtype == torch.float32
+    assert X.dtype in (torch.float32, torch.float16, torch.bfloat16)
     assert int(2 ** int(math.log2(X.shape[-1]))) == X.shape[-1]
     return ops.fht(X)
 
 
 def fast_hadamard_transform_dim512(X):
-    raise NotImplementedError(
-        "the fp16 dim-512 transform (fast_hadamard_transform/kernel.py:17-22) is not built: "
-        "use float32 inputs")
+    """fast_hadamard_transform/kernel.py:17-22: half rows of 512.  Computed in fp32 with one
+    rounding on the store (the reference rounds in half precision after every stage)."""
+    assert X.is_contiguous()
+    assert len(X.shape) == 2
+    assert X.dtype == torch.float16
+    assert X.shape[-1] == 512
+    return ops.fht(X)
 
 
 def fast_hadamard_transform_dim1024(X):
-    raise NotImplementedError(
-        "the fp16 dim-1024 transform (fast_hadamard_transform/kernel.py:24-29) is not built: "
-        "use float32 inputs")
+    """fast_hadamard_transform/kernel.py:24-29: half rows of 1024; see the 512 form."""
+    assert X.is_contiguous()
+    assert len(X.shape) == 2
+    assert X.dtype == torch.float16
+    assert X.shape[-1] == 1024
+    return ops.fht(X)
 
 
 class FastHadamardTransform(Function):

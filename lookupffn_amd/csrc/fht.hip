@@ -287,6 +287,90 @@ int check_dims(int64_t B, int64_t H, int64_t D, int64_t R, int64_t J) {
     return LFFN_OK;
 }
 
+// The transform on rows stored as 16-bit floats (IEEE half or bfloat16): widened on load,
+// every butterfly in fp32 registers exactly as above, one rounding (to nearest even) on the
+// store.  The reference's half kernels add in half2 after every stage
+// (fast_hadamard_transform/extension/cuda_kernel.cu:47-84); this is the same transform with
+// a single rounding.
+template <bool BF16>
+__device__ __forceinline__ float widen16(uint32_t h) {
+    if constexpr (BF16) return __uint_as_float(h << 16);
+    else return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+}
+
+template <bool BF16>
+__device__ __forceinline__ uint32_t narrow16(float f) {
+    if constexpr (BF16) {
+        const uint32_t u = __float_as_uint(f);
+        if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;      // NaN stays NaN
+        return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+    } else {
+        return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+    }
+}
+
+template <int LOGD, bool BF16>
+__global__ __launch_bounds__(256) void fht16_kernel(const uint16_t *__restrict__ in, uint16_t *__restrict__ out,
+                                                    int64_t B) {
+    using C = FhtCfg<LOGD>;
+    constexpr int D = C::D, NJ = C::NJ, LPR = C::LPR, RPW = C::RPW;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int lr = lane % LPR;
+    const int64_t row = (int64_t(blockIdx.x) * 4 + wave) * RPW + lane / LPR;
+    const bool live = row < B;
+    float v[NJ][4];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        uint2 t = make_uint2(0u, 0u);
+        if (live) t = *reinterpret_cast<const uint2 *>(in + row * D + 256 * j + 4 * lr);
+        v[j][0] = widen16<BF16>(t.x & 0xffffu);
+        v[j][1] = widen16<BF16>(t.x >> 16);
+        v[j][2] = widen16<BF16>(t.y & 0xffffu);
+        v[j][3] = widen16<BF16>(t.y >> 16);
+    }
+    fht_rows<LOGD>(v, lr);
+    if (live) {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            uint2 t;
+            t.x = narrow16<BF16>(v[j][0]) | (narrow16<BF16>(v[j][1]) << 16);
+            t.y = narrow16<BF16>(v[j][2]) | (narrow16<BF16>(v[j][3]) << 16);
+            *reinterpret_cast<uint2 *>(out + row * D + 256 * j + 4 * lr) = t;
+        }
+    }
+}
+
+template <bool BF16>
+int fht16_entry(const uint16_t *in, uint16_t *out, int64_t B, int64_t D, void *stream) {
+    LFFN_REQUIRE(in && out, LFFN_ERR_BAD_ARG);
+    int rc = check_dims(B, D, D, 1, 1);
+    if (rc != LFFN_OK) return rc;
+    LFFN_REQUIRE((reinterpret_cast<uintptr_t>(in) & 7u) == 0 && (reinterpret_cast<uintptr_t>(out) & 7u) == 0,
+                 LFFN_ERR_BAD_ARG);
+    if (B == 0) return LFFN_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    auto go = [&](auto tag) {
+        constexpr int L = decltype(tag)::value;
+        const int64_t rows_per_block = 4 * FhtCfg<L>::RPW;
+        hipLaunchKernelGGL((fht16_kernel<L, BF16>), dim3((unsigned)((B + rows_per_block - 1) / rows_per_block)),
+                           dim3(256), 0, st, in, out, B);
+    };
+    switch (lffn_log2(D)) {
+        case 2: go(std::integral_constant<int, 2>{}); break;
+        case 3: go(std::integral_constant<int, 3>{}); break;
+        case 4: go(std::integral_constant<int, 4>{}); break;
+        case 5: go(std::integral_constant<int, 5>{}); break;
+        case 6: go(std::integral_constant<int, 6>{}); break;
+        case 7: go(std::integral_constant<int, 7>{}); break;
+        case 8: go(std::integral_constant<int, 8>{}); break;
+        case 9: go(std::integral_constant<int, 9>{}); break;
+        case 10: go(std::integral_constant<int, 10>{}); break;
+        default: return LFFN_ERR_UNSUPPORTED;
+    }
+    return lffn_launch_status();
+}
+
 }  // namespace
 
 extern "C" int lffn_fht_f32(const float *in, float *out, int64_t B, int64_t D, void *stream) {
@@ -361,4 +445,12 @@ static int project_hash_impl(const float *x, const float *ln_w, const float *ln_
     a.decay = decay; a.residual = residual; a.mix = 1;
     a.vec_in = (lffn_aligned16(x) && H % 4 == 0) ? 1 : 0;
     return launch_project<true>(a, lffn_log2(D), static_cast<hipStream_t>(stream));
+}
+
+extern "C" int lffn_fht_f16(const uint16_t *in, uint16_t *out, int64_t B, int64_t D, void *stream) {
+    return fht16_entry<false>(in, out, B, D, stream);
+}
+
+extern "C" int lffn_fht_bf16(const uint16_t *in, uint16_t *out, int64_t B, int64_t D, void *stream) {
+    return fht16_entry<true>(in, out, B, D, stream);
 }

@@ -31,13 +31,16 @@ _L.define("fht(Tensor x) -> Tensor")
 
 
 def _fht_impl(x: torch.Tensor) -> torch.Tensor:
+    """float32, float16 or bfloat16 rows; the 16-bit forms compute in fp32 and round once."""
     _lib.require_gpu(x)
-    assert x.dim() == 2 and x.dtype == torch.float32 and x.is_contiguous()
+    assert x.dim() == 2 and x.is_contiguous()
+    assert x.dtype in (torch.float32, torch.float16, torch.bfloat16)
     B, D = x.shape
     out = torch.empty_like(x)
+    name = {torch.float32: "lffn_fht_f32", torch.float16: "lffn_fht_f16", torch.bfloat16: "lffn_fht_bf16"}[x.dtype]
     with _dev_guard(x):
-        rc = _lib.load().lffn_fht_f32(_lib.ptr(x), _lib.ptr(out), B, D, _lib.stream_of(x))
-    _lib.check(rc, f"lffn_fht_f32(B={B}, D={D})")
+        rc = getattr(_lib.load(), name)(_lib.ptr(x), _lib.ptr(out), B, D, _lib.stream_of(x))
+    _lib.check(rc, f"{name}(B={B}, D={D})")
     return out
 
 

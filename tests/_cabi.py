@@ -42,6 +42,14 @@ def fht(x):
     return host(out)
 
 
+def fht16(bits, bf16=False, in_place=False):
+    """bits: uint16 patterns of half (or bfloat16) rows."""
+    xd = dev(bits)
+    out = xd if in_place else torch.full_like(xd, -1)
+    _call("lffn_fht_bf16" if bf16 else "lffn_fht_f16", p(xd), p(out), bits.shape[0], bits.shape[1])
+    return host(out).view(np.uint16)
+
+
 def fht_inplace(x):
     xd = dev(x)
     _call("lffn_fht_f32", p(xd), p(xd), x.shape[0], x.shape[1])

@@ -261,3 +261,18 @@ def test_encoder_layers_match_float64_composition():
             assert (err <= 5e-5).mean() >= 0.9, err
             h = got
         assert relmax(npf(model.encoder.LayerNorm(h)), npf(out)) <= 1e-6
+
+
+def test_hadamard_half_dispatch():
+    """hadamard() on half rows of 512 / 1024 goes to the Dim512 / Dim1024 functions
+    (fast_hadamard_transform/kernel.py:78-89); forward and backward are the same transform."""
+    torch.manual_seed(5)
+    for D in (512, 1024):
+        x = torch.randn(9, D, device=DEV).half().requires_grad_(True)
+        y = lookupffn_amd.hadamard(x)
+        assert y.dtype == torch.float16
+        want = lookupffn_amd.hadamard(x.detach().float())
+        assert relmax(npf(y), npf(want)) <= 1e-3
+        g = torch.randn(9, D, device=DEV).half()
+        y.backward(g)
+        assert relmax(npf(x.grad), npf(lookupffn_amd.hadamard(g.float()))) <= 1e-3

@@ -93,6 +93,37 @@ def test_fht_full_size_properties():
     assert np.array_equal(y[sub], oracle.fht(x[sub]))
 
 
+@pytest.mark.parametrize("D", [4, 16, 64, 256, 512, 1024])
+@pytest.mark.parametrize("bf16", [False, True])
+def test_fht_16bit_storage(D, bf16):
+    """Half / bfloat16 rows: fp32 butterflies, one rounding on the store.  Against the float64
+    transform of the same 16-bit inputs the error is that one rounding (2^-11 resp. 2^-8
+    relative) plus fp32 rounding of the sums; small integers come out exactly."""
+    import scipy.linalg
+    rng = np.random.RandomState(D + int(bf16))
+    B = 37
+    x32 = rng.randn(B, D).astype(np.float32)
+    if bf16:
+        bits = oracle.bf16_round(x32)
+        xin = oracle.bf16_widen(bits).astype(np.float64)
+        widen, eps = (lambda b: oracle.bf16_widen(b).astype(np.float64)), 2.0 ** -8
+    else:
+        h = x32.astype(np.float16)
+        bits = h.view(np.uint16)
+        xin = h.astype(np.float64)
+        widen, eps = (lambda b: b.view(np.float16).astype(np.float64)), 2.0 ** -11
+    want = xin @ scipy.linalg.hadamard(D)
+    got = widen(cabi.fht16(bits, bf16=bf16))
+    scale = np.abs(want).max()
+    assert np.all(np.abs(got - want) <= eps * np.abs(want) + 2e-6 * scale)
+    assert np.array_equal(widen(cabi.fht16(bits, bf16=bf16, in_place=True)), got)
+    # exact on small integers (every sum is representable)
+    xi = rng.randint(-2, 3, size=(B, D)).astype(np.float32)
+    if D <= 64:
+        ib = oracle.bf16_round(xi) if bf16 else xi.astype(np.float16).view(np.uint16)
+        assert np.array_equal(widen(cabi.fht16(ib, bf16=bf16)), xi.astype(np.float64) @ scipy.linalg.hadamard(D))
+
+
 # ----------------------------------------------------------------------------- BH4 diag / projection + hash
 
 @pytest.mark.parametrize("H,D,R,J", [(256, 256, 1, 4), (768, 1024, 1, 4), (1024, 1024, 4, 4), (48, 64, 2, 1),
