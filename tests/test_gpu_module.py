@@ -276,3 +276,30 @@ def test_hadamard_half_dispatch():
         g = torch.randn(9, D, device=DEV).half()
         y.backward(g)
         assert relmax(npf(x.grad), npf(lookupffn_amd.hadamard(g.float()))) <= 1e-3
+
+
+def test_checkpoint_round_trip_and_folded_weight_cache(tmp_path):
+    """A state_dict saved under the reference's key names loads strictly (after the "model."
+    prefix is stripped, roberta_to_hf_checkpoint.py:102-111) and the block-64 layer then
+    computes with the loaded weights: the folded copy of the BH4 weights follows the parameter."""
+    torch.manual_seed(21)
+    cfg = _config(hidden_size=256, ffn_num_table=32, block_size=64)
+    a = lookupffn_amd.LookupFFN(cfg, 256).eval().to(DEV)
+    b = lookupffn_amd.LookupFFN(cfg, 256).eval().to(DEV)
+    x = torch.randn(70, 256, device=DEV)
+    with torch.no_grad():
+        out_a = a(x)
+        out_b_before = b(x)                       # folds b's own weights
+    assert not torch.equal(out_a, out_b_before)
+    path = tmp_path / "ffn.ckpt"
+    torch.save({"state_dict": {"model." + k: v.cpu() for k, v in a.state_dict().items()}}, path)
+    weights = torch.load(path, map_location="cpu", weights_only=True)["state_dict"]
+    weights = {k[len("model."):]: v for k, v in weights.items()}
+    assert set(weights) == {"LayerNorm.weight", "LayerNorm.bias", "hash.projection.weight", "hash.projection.bias",
+                            "tables", "bias"}
+    b.load_state_dict(weights, strict=True)
+    with torch.no_grad():
+        assert torch.equal(b(x), out_a)           # not the stale folded weights
+        # an in-place update (an optimizer step) is seen as well
+        b.hash.projection.weight.mul_(0.5)
+        assert not torch.equal(b(x), out_a)
