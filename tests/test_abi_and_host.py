@@ -64,6 +64,43 @@ def test_argument_validation_needs_no_gpu():
     assert lib.lffn_code_score_f32(256, 256, 256, 0, 8, None) == _lib.LFFN_OK
 
 
+def test_argument_validation_of_the_backward_and_block_entry_points():
+    lib = _lib.load()
+    U, A, OK = _lib.LFFN_ERR_UNSUPPORTED, _lib.LFFN_ERR_BAD_ARG, _lib.LFFN_OK
+    P = 256                                    # a non-null, 16-byte aligned "pointer" that is never dereferenced
+    # indexed inner product on table-local codes
+    assert lib.lffn_lookup_inner_f32(None, None, None, None, 4, 2, 16, 64, None) == A
+    assert lib.lffn_lookup_inner_f32(P, P, P, P, 4, 2, 100, 64, None) == U          # S not a power of two
+    assert lib.lffn_lookup_inner_f32(P, P, P, P, 4, 2, 16, 96, None) == U           # Do % 64
+    assert lib.lffn_lookup_inner_f32(P, P + 4, P, P, 4, 2, 16, 64, None) == A       # misaligned g
+    assert lib.lffn_lookup_inner_f32(P, P, P, P, 0, 2, 16, 64, None) == OK
+    # scatter-add on table-local codes
+    assert lib.lffn_lookup_scatter_f32(P, P, P, P, 4, 2, 100, 64, 0, None) == U
+    # BH4 with 64 x 64 blocks
+    assert lib.lffn_bh4_fold_f32(P, P + 1024, 1, 4, 16, 32, None) == U              # block size other than 64
+    assert lib.lffn_bh4_fold_f32(P, P, 1, 4, 16, 64, None) == A                     # in place
+    assert lib.lffn_bh4_block_f32(P, P, P, 4, 768, 2048, 1, 4, 64, None) == U       # D > 1024
+    assert lib.lffn_bh4_block_f32(P, P, P, 4, 770, 1024, 1, 4, 64, None) == U       # H % 4
+    assert lib.lffn_bh4_block_f32(P, P, P, 4, 2000, 1024, 1, 4, 64, None) == A      # H > D
+    assert lib.lffn_bh4_block_f32(P, P, P, 0, 768, 1024, 1, 4, 64, None) == OK
+    assert lib.lffn_ln_bh4_block_hash_f32(P, None, None, 0.0, P, None, P, P, 4, 768, 1024, 1, 4, 200, 64,
+                                          0.7, 0.3, None) == A                      # T*8 > R*D
+    assert lib.lffn_ln_bh4_block_hash_f32(P, P, None, 1e-5, P, None, P, P, 4, 768, 1024, 1, 4, 128, 64,
+                                          0.7, 0.3, None) == A                      # LayerNorm weight without bias
+    assert lib.lffn_ln_bh4_block_hash_f32(P, None, None, 0.0, P, None, P, P, 0, 768, 1024, 1, 4, 128, 64,
+                                          0.7, 0.3, None) == OK
+    # mix + hash
+    assert lib.lffn_mix_code_score_f32(P, P, None, P, P, 4, 8, 25, 64, 64, 256, 0.7, 0.3, None) == U   # k > 24
+    assert lib.lffn_mix_code_score_f32(P, P, None, P, P, 4, 40, 8, 64, 64, 256, 0.7, 0.3, None) == A   # T*k > ldy
+    assert lib.lffn_mix_code_score_f32(P, P, None, P, P, 0, 8, 8, 64, 64, 256, 0.7, 0.3, None) == OK
+    # 16-bit transform
+    assert lib.lffn_fht_f16(P, P, 4, 2048, None) == U
+    assert lib.lffn_fht_bf16(P, P + 2, 4, 64, None) == A                            # 8-byte alignment
+    assert lib.lffn_fht_f16(P, P, 0, 64, None) == OK
+    # gather with residual
+    assert lib.lffn_lookup_gather_residual_f32(P, P, P, None, P + 4, P, 4, 2, 16, 64, None) == A
+
+
 def _config(**kw):
     base = dict(hidden_size=48, ffn_num_table=8, ffn_table_size=256, layer_norm_eps=1e-5,
                 projection_type="bh4", block_size=1)
