@@ -80,6 +80,25 @@ int lffn_bh4_diag_f32(const float *x, const float *diag, float *out,
                       int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, void *stream);
 
 /*
+ * Backward of lffn_project_hash_f32 (block size 1, 8-bit codes) in one kernel: from x, the
+ * diagonals, the z the forward kept and the gradient of the scores, the gradients of x, of the
+ * diagonals and of the projection bias.  The forward stages are recomputed in registers; the
+ * transform is its own transpose.
+ * x: [B, H], H % 4 == 0; diag: [R, J, D], J <= 4, 256 <= D <= 1024; z: [B, T*8]; g_score: [B, T];
+ * g_x: [R, B, H], one slab per repeat (the caller adds them; R == 1 needs nothing);
+ * part_diag: [num_partials, R, J, D] and part_bias: [num_partials, R*D]: one partial sum per
+ * workgroup, fully written; the caller adds them over the first axis (grad bias = the first
+ * T*8 columns).  num_partials is the number of workgroups per repeat, 1..65535 (512 is a good
+ * value on 256 compute units).  The code has no gradient.
+ * Replaces what autograd records for BH4._forward + compute_code_score_torch
+ * (PL/lookup.py:29-39, PL/bh4/kernel.py:23-36, PL/compute_code_score/kernel.py:47-53).
+ */
+int lffn_project_hash_bwd_f32(const float *x, const float *diag, const float *z, const float *g_score,
+                              float *g_x, float *part_diag, float *part_bias, int64_t B, int64_t H,
+                              int64_t D, int64_t R, int64_t J, int64_t T, int64_t num_partials,
+                              float decay, float residual, void *stream);
+
+/*
  * BH4 mixing with 64 x 64 blocks, all stages of a repeat in one kernel:
  *   for r < R:  y = pad(x);  for j < J:  y = FHT(blockdiag(w[r,j]) y);  out[b, r*D:(r+1)*D] = y
  * x: [B, H], H <= D, H % 4 == 0 (zero-padded on load, PL/lookup.py:32-34);

@@ -36,6 +36,8 @@ SIGNATURES = {
                                 ctypes.c_float, ctypes.c_float, _vp],
     "lffn_ln_bh4_block_hash_f32": [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
                                    _i64, _i64, ctypes.c_float, ctypes.c_float, _vp],
+    "lffn_project_hash_bwd_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
+                                  ctypes.c_float, ctypes.c_float, _vp],
     "lffn_bh4_fold_f32": [_vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "lffn_bh4_block_f32": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp],
     "lffn_project_hash_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _vp],

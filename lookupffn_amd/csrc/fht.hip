@@ -287,6 +287,177 @@ int check_dims(int64_t B, int64_t H, int64_t D, int64_t R, int64_t J) {
     return LFFN_OK;
 }
 
+// Backward of the fused projection + hash for block size 1 and 8-bit codes, one kernel:
+//   z = decay * y + residual * pad(x) (+ bias),  y = FHT(d_{J-1} * ... FHT(d_0 * pad(x)))   per repeat
+// Inputs: x, the diagonals, the z kept by the forward and the gradient of the scores.
+// Per row (one wavefront, D >= 256): the gradient of z from the closed form of the score
+// (PL/compute_code_score/kernel.py:51-53 differentiated; a group of 8 columns sits in a lane
+// pair), the forward stages recomputed in registers (u_0 = pad(x), u_{j+1} = FHT(d_j * u_j)),
+// then backwards t <- FHT(t); grad d_j += t * u_j; t <- d_j * t, the transform being its own
+// transpose.  grad x of this repeat = t + residual * grad z.  The gradients of the diagonals and
+// of the bias are summed over the rows of a wavefront in registers, over the four wavefronts
+// of the workgroup in LDS, and written as one partial per workgroup; the caller adds the
+// partials (and the per-repeat grad x when R > 1).
+struct ProjectBwdArgs {
+    const float *x;        // [B, H]
+    const float *diag;     // [R, J, D]
+    const float *z;        // [B, ncols]  (ncols = T*8)
+    const float *g_score;  // [B, T]
+    float *g_x;            // [R, B, H]
+    float *part_d;         // [nblk, R, J, D]
+    float *part_b;         // [nblk, R*D]   (columns >= ncols are written as zero)
+    int64_t B;
+    int H, R, J, T;
+    float decay, residual;
+};
+
+template <int LOGD>
+__global__ __launch_bounds__(256) void project_hash_bwd_kernel(ProjectBwdArgs a) {
+    using C = FhtCfg<LOGD>;
+    constexpr int D = C::D, NJ = C::NJ;
+    static_assert(C::LPR == 64, "one row per wavefront");
+    constexpr int MAXJ = 4;
+    __shared__ float red[4][64][NJ * 4];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int lr = lane;
+    const int r = blockIdx.y;
+    const int ncols = a.T * 8;
+    const int64_t nwaves = int64_t(gridDim.x) * 4;
+
+    float acc_d[MAXJ][NJ][4], acc_b[NJ][4];
+#pragma unroll
+    for (int s = 0; s < MAXJ; ++s)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) acc_d[s][j][c] = 0.f;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc_b[j][c] = 0.f;
+
+    for (int64_t row = int64_t(blockIdx.x) * 4 + wave; row < a.B; row += nwaves) {
+        // forward stages recomputed: u[s] is the input of stage s
+        float u[MAXJ][NJ][4], t[NJ][4];
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const int e0 = 256 * j + 4 * lr;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (e0 < a.H) v = *reinterpret_cast<const float4 *>(a.x + row * a.H + e0);
+            t[j][0] = v.x; t[j][1] = v.y; t[j][2] = v.z; t[j][3] = v.w;
+        }
+#pragma unroll
+        for (int s = 0; s < MAXJ; ++s) {
+            if (s < a.J) {
+                const float *dg = a.diag + (int64_t(r) * a.J + s) * D;
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    const float4 w = *reinterpret_cast<const float4 *>(dg + 256 * j + 4 * lr);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) u[s][j][c] = t[j][c];
+                    t[j][0] = t[j][0] * w.x; t[j][1] = t[j][1] * w.y; t[j][2] = t[j][2] * w.z; t[j][3] = t[j][3] * w.w;
+                }
+                if (s + 1 < a.J) fht_rows<LOGD>(t, lr);      // the last transform's output is not needed
+            }
+        }
+
+        // gradient of z for this repeat's columns
+        float gz[NJ][4];
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const int col = r * D + 256 * j + 4 * lr;
+            const bool in_cols = col < ncols;
+            float4 zv = make_float4(0.f, 0.f, 0.f, 0.f);
+            float g = 0.f;
+            if (in_cols) {
+                zv = *reinterpret_cast<const float4 *>(a.z + row * ncols + col);
+                g = a.g_score[row * a.T + (col >> 3)];
+            }
+            const float zz[4] = {zv.x, zv.y, zv.z, zv.w};
+            float az[4], ez[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                az[c] = fabsf(zz[c]);
+                ez[c] = expf(-2.0f * az[c]);
+            }
+            // S and P over the 8 values of the group, d ascending: the even lane starts, the odd
+            // lane continues and hands the totals back
+            float s_loc = 0.f, p_loc = 1.f;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) { s_loc = s_loc + az[c]; p_loc = p_loc * (1.0f + ez[c]); }
+            float s_run = lane_xor<1>(s_loc), p_run = lane_xor<1>(p_loc);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) { s_run = s_run + az[c]; p_run = p_run * (1.0f + ez[c]); }
+            const float s_back = lane_xor<1>(s_run), p_back = lane_xor<1>(p_run);
+            const float S = (lr & 1) ? s_run : s_back;
+            const float P = (lr & 1) ? p_run : p_back;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const float sg = zz[c] > 0.f ? 1.f : (zz[c] < 0.f ? -1.f : 0.f);
+                gz[j][c] = in_cols ? g * sg * (1.0f + S * 2.0f * ez[c] / (1.0f + ez[c])) / P : 0.f;
+                acc_b[j][c] += gz[j][c];
+            }
+        }
+
+        // backwards through the stages
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) t[j][c] = a.decay * gz[j][c];
+#pragma unroll
+        for (int s = MAXJ - 1; s >= 0; --s) {
+            if (s < a.J) {
+                fht_rows<LOGD>(t, lr);
+                const float *dg = a.diag + (int64_t(r) * a.J + s) * D;
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    const float4 w = *reinterpret_cast<const float4 *>(dg + 256 * j + 4 * lr);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) acc_d[s][j][c] += t[j][c] * u[s][j][c];
+                    t[j][0] = t[j][0] * w.x; t[j][1] = t[j][1] * w.y; t[j][2] = t[j][2] * w.z; t[j][3] = t[j][3] * w.w;
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const int e0 = 256 * j + 4 * lr;
+            if (e0 < a.H) {
+                float4 o;
+                o.x = t[j][0] + a.residual * gz[j][0];
+                o.y = t[j][1] + a.residual * gz[j][1];
+                o.z = t[j][2] + a.residual * gz[j][2];
+                o.w = t[j][3] + a.residual * gz[j][3];
+                *reinterpret_cast<float4 *>(a.g_x + (int64_t(r) * a.B + row) * a.H + e0) = o;
+            }
+        }
+    }
+
+    // workgroup partials: sum of the four wavefronts, one array at a time through LDS
+    auto flush = [&](const float (&acc)[NJ][4], float *dst) {
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) red[wave][lane][4 * j + c] = acc[j][c];
+        __syncthreads();
+        // thread (wave, lane) adds float4 number `wave`.. of lane `lane` over the four wavefronts
+        for (int j = wave; j < NJ; j += 4) {
+            float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                sum.x += red[w][lane][4 * j + 0]; sum.y += red[w][lane][4 * j + 1];
+                sum.z += red[w][lane][4 * j + 2]; sum.w += red[w][lane][4 * j + 3];
+            }
+            *reinterpret_cast<float4 *>(dst + 256 * j + 4 * lane) = sum;
+        }
+    };
+#pragma unroll
+    for (int s = 0; s < MAXJ; ++s)
+        if (s < a.J) flush(acc_d[s], a.part_d + ((int64_t(blockIdx.x) * a.R + r) * a.J + s) * D);
+    flush(acc_b, a.part_b + (int64_t(blockIdx.x) * a.R + r) * D);
+}
+
 // The transform on rows stored as 16-bit floats (IEEE half or bfloat16): widened on load,
 // every butterfly in fp32 registers exactly as above, one rounding (to nearest even) on the
 // store.  The reference's half kernels add in half2 after every stage
@@ -453,4 +624,28 @@ extern "C" int lffn_fht_f16(const uint16_t *in, uint16_t *out, int64_t B, int64_
 
 extern "C" int lffn_fht_bf16(const uint16_t *in, uint16_t *out, int64_t B, int64_t D, void *stream) {
     return fht16_entry<true>(in, out, B, D, stream);
+}
+
+extern "C" int lffn_project_hash_bwd_f32(const float *x, const float *diag, const float *z, const float *g_score,
+                                         float *g_x, float *part_diag, float *part_bias, int64_t B, int64_t H,
+                                         int64_t D, int64_t R, int64_t J, int64_t T, int64_t num_partials,
+                                         float decay, float residual, void *stream) {
+    int rc = check_dims(B, H, D, R, J);
+    if (rc != LFFN_OK) return rc;
+    LFFN_REQUIRE(D >= 256 && J >= 1 && J <= 4 && H % 4 == 0 && R <= 65535, LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(T >= 1 && T * 8 <= R * D && num_partials >= 1 && num_partials <= 65535, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(x && diag && z && g_score && g_x && part_diag && part_bias, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_aligned16(x) && lffn_aligned16(diag) && lffn_aligned16(z) && lffn_aligned16(g_x) &&
+                     lffn_aligned16(part_diag) && lffn_aligned16(part_bias), LFFN_ERR_BAD_ARG);
+    ProjectBwdArgs a{};
+    a.x = x; a.diag = diag; a.z = z; a.g_score = g_score; a.g_x = g_x; a.part_d = part_diag; a.part_b = part_bias;
+    a.B = B; a.H = (int)H; a.R = (int)R; a.J = (int)J; a.T = (int)T; a.decay = decay; a.residual = residual;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const dim3 grid((unsigned)num_partials, (unsigned)R);
+    switch (lffn_log2(D)) {
+        case 8: hipLaunchKernelGGL((project_hash_bwd_kernel<8>), grid, dim3(256), 0, st, a); break;
+        case 9: hipLaunchKernelGGL((project_hash_bwd_kernel<9>), grid, dim3(256), 0, st, a); break;
+        default: hipLaunchKernelGGL((project_hash_bwd_kernel<10>), grid, dim3(256), 0, st, a); break;
+    }
+    return lffn_launch_status();
 }

@@ -64,6 +64,34 @@ class BH4(nn.Module):
         return outputs.reshape(*shape, self.out_dim)
 
 
+class ProjectHash(torch.autograd.Function):
+    """Diagonal BH4 -> mix -> bias -> 8-bit code + score as one differentiable operator:
+    one kernel forward (z is kept), one kernel backward (the stages are recomputed in
+    registers).  Same mathematics as BH4._forward + compute_code_score under autograd
+    (PL/lookup.py:29-39, PL/compute_code_score/kernel.py:47-53); the code has no gradient."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, T, decay):
+        R, J = weight.shape[0], weight.shape[1]
+        diag = weight.reshape(R, J, -1).contiguous()
+        x = x.contiguous()
+        code, score, z = ops.project_hash(x, diag, bias, T, float(decay), float(1 - decay), True)
+        ctx.save_for_backward(x, diag, z)
+        ctx.weight_shape = weight.shape
+        ctx.has_bias = bias is not None
+        ctx.decay = float(decay)
+        ctx.mark_non_differentiable(code)
+        return code, score
+
+    @staticmethod
+    def backward(ctx, _g_code, g_score):
+        x, diag, z = ctx.saved_tensors
+        g_x, g_diag, g_bias = ops.project_hash_bwd(x, diag, z, g_score.contiguous(), ctx.decay, 1 - ctx.decay)
+        return (g_x if ctx.needs_input_grad[0] else None,
+                g_diag.reshape(ctx.weight_shape) if ctx.needs_input_grad[1] else None,
+                g_bias if (ctx.has_bias and ctx.needs_input_grad[2]) else None, None, None)
+
+
 class Hashing(nn.Module):
     """PL/lookup.py:49-77."""
 
@@ -142,10 +170,21 @@ class Hashing(nn.Module):
         return ops.mix_code_score(y, x, p.bias, self.num_table, self.code_length, p.padded_in_dim,
                                   float(p.decay_coeff), float(1 - p.decay_coeff))
 
+    def can_fuse_training(self, x):
+        """The differentiable one-kernel form: diagonal BH4 with at most 4 stages, 8-bit codes,
+        256 <= D <= 1024, fp32."""
+        p = self.projection
+        return (isinstance(p, BH4) and p.block_size == 1 and self.code_length == 8
+                and 256 <= p.padded_in_dim <= 1024 and p.weight.shape[1] <= 4 and p.in_dim % 4 == 0
+                and x.dtype == torch.float32 and x.is_cuda and p.weight.dtype == torch.float32)
+
     def forward(self, x):
         B, D = x.shape
         if self.can_fuse(x):
             return self.forward_fused(x)
+        if self.can_fuse_training(x):
+            p = self.projection
+            return ProjectHash.apply(x, p.weight, p.bias, self.num_table, p.decay_coeff)
         if self.can_fuse_block(x):
             return self.forward_block(x)
         z = self.projection(x)

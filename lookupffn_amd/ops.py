@@ -246,6 +246,44 @@ def _(x, diag, bias, T, decay, residual, keep_z):
             x.new_empty((B, T * 8) if keep_z else (0,)))
 
 
+_L.define("project_hash_bwd(Tensor x, Tensor diag, Tensor z, Tensor g_score, float decay, float residual)"
+          " -> (Tensor, Tensor, Tensor)")
+
+PROJECT_BWD_PARTIALS = 512      # workgroups per repeat: two per compute unit
+
+
+def _project_hash_bwd_impl(x, diag, z, g_score, decay, residual):
+    """-> (grad x [B,H], grad diag [R,J,D], grad bias [T*8])."""
+    _lib.require_gpu(x, diag, z, g_score)
+    for t in (x, diag, z, g_score):
+        assert t.dtype == torch.float32 and t.is_contiguous()
+    B, H = x.shape
+    R, J, D = diag.shape
+    T = g_score.shape[1]
+    assert tuple(z.shape) == (B, T * 8) and g_score.shape[0] == B
+    nparts = max(1, min(PROJECT_BWD_PARTIALS, (B + 3) // 4))
+    g_x = torch.empty(R, B, H, dtype=torch.float32, device=x.device)
+    part_d = torch.empty(nparts, R, J, D, dtype=torch.float32, device=x.device)
+    part_b = torch.empty(nparts, R * D, dtype=torch.float32, device=x.device)
+    if B > 0:
+        with _dev_guard(x):
+            rc = _lib.load().lffn_project_hash_bwd_f32(
+                _lib.ptr(x), _lib.ptr(diag), _lib.ptr(z), _lib.ptr(g_score), _lib.ptr(g_x), _lib.ptr(part_d),
+                _lib.ptr(part_b), B, H, D, R, J, T, nparts, decay, residual, _lib.stream_of(x))
+        _lib.check(rc, f"lffn_project_hash_bwd_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T})")
+    else:
+        part_d.zero_(); part_b.zero_()
+    return (g_x[0] if R == 1 else g_x.sum(0)), part_d.sum(0), part_b.sum(0)[:T * 8]
+
+
+_L.impl("project_hash_bwd", _project_hash_bwd_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::project_hash_bwd")
+def _(x, diag, z, g_score, decay, residual):
+    return torch.empty_like(x), torch.empty_like(diag), x.new_empty(z.shape[1])
+
+
 _L.define("ln_project_hash(Tensor x, Tensor ln_weight, Tensor ln_bias, float eps, Tensor diag, Tensor? bias, "
           "int T, float decay, float residual, bool keep_z) -> (Tensor, Tensor, Tensor)")
 
@@ -537,6 +575,7 @@ bh4_block = torch.ops.lookupffn.bh4_block
 mix_code_score = torch.ops.lookupffn.mix_code_score
 ln_bh4_block_hash = torch.ops.lookupffn.ln_bh4_block_hash
 project_hash = torch.ops.lookupffn.project_hash
+project_hash_bwd = torch.ops.lookupffn.project_hash_bwd
 ln_project_hash = torch.ops.lookupffn.ln_project_hash
 code_score = torch.ops.lookupffn.code_score
 code_score_bwd = torch.ops.lookupffn.code_score_bwd

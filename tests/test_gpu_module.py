@@ -126,13 +126,19 @@ def test_operator_gradients_match_oracle():
                                rtol=2e-5, atol=1e-6)
 
 
-def test_layer_gradients_match_torch_autograd_of_reference_formulas():
+# (H, T, Do): D = 64 takes the per-operator path; the others the one-kernel differentiable
+# projection + hash (D = 256 with one and with two repeats, D = 512, D = 1024 with zero padding)
+@pytest.mark.parametrize("H,T,Do", [(64, 8, 64), (256, 32, 64), (256, 64, 128), (500, 64, 64), (768, 128, 64)])
+def test_layer_gradients_match_torch_autograd_of_reference_formulas(H, T, Do):
     """Training step through the whole layer vs autograd over the reference's own
     slow formulas (index-multiply-sum gather, compute_code_score_torch, matmul
     Hadamard) evaluated in float64 on the same parameters."""
-    torch.manual_seed(5)
-    H, T, Do, S = 64, 8, 64, 256
+    torch.manual_seed(5 + H + T)
+    S = 256
     layer = lookupffn_amd.LookupFFN(_config(hidden_size=H, ffn_num_table=T), Do).to(DEV).train()
+    with torch.no_grad():
+        layer.hash.projection.bias.normal_(0, 0.05)
+    assert layer.hash.can_fuse_training(torch.empty(1, H, device=DEV)) == (H >= 256)
     x = torch.randn(24, H, device=DEV, requires_grad=True)
     target = torch.randn(24, Do, device=DEV)
     out = layer(x)
@@ -165,6 +171,7 @@ def test_layer_gradients_match_torch_autograd_of_reference_formulas():
         code_g, _ = layer.hash(layer.LayerNorm(x))
     if not np.array_equal(npf(code_g).astype(np.int64), code_r.numpy().astype(np.int64)):
         pytest.skip("a sign flipped between fp32 and fp64 projections for this seed")
+    assert layer.hash.projection.weight.grad.abs().max() > 0 and layer.hash.projection.bias.grad.abs().max() > 0
     assert relmax(npf(out), out_r.detach().numpy()) <= 2e-5
     for k, v in layer.named_parameters():
         assert relmax(npf(v.grad), ref[k].grad.numpy()) <= 2e-4, k
