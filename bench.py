@@ -60,7 +60,7 @@ WORKLOADS = {
 # (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); the summaries
 # are kept under profiles/.  None until measured for that workload.
 MEASURED_TRAFFIC_BYTES = {"cfg2": 477559591, "cfg2b64": 477451647, "cfg3": 3156050546, "cfg3bf16": 2252934839,
-                          "cfg5": 504064321}
+                          "cfg5": 503520831}
 
 
 def build_layer(wl, device):
@@ -158,9 +158,9 @@ def zipf_codes(B, T, S, gen, s=1.1):
 
 def main_backward(args):
     """Backward of the layer's operators at the config-2 shape: gradient w.r.t. the
-    scores (indexed inner product), the tables (atomic scatter-add into a zeroed
-    buffer), z (closed-form score derivative) and the projection input (the four
-    diagonal x Hadamard stages transposed)."""
+    scores (indexed inner product), the tables (scatter-add), and, in one kernel, z
+    (closed-form score derivative), the projection input (the four diagonal x Hadamard
+    stages transposed), the diagonals and the projection bias."""
     import numpy as np
     import torch
 
@@ -177,25 +177,25 @@ def main_backward(args):
     g_out_cpu = torch.randn(B, Do, generator=g)
     score_cpu = 1.0 - torch.rand(B, T, generator=g)
     code, z, g_out, score = code_cpu.to(dev), z_cpu.to(dev), g_out_cpu.to(dev), score_cpu.to(dev)
+    z2 = z.reshape(B, T * 8).contiguous()
     tables = layer.tables.detach()
     flat = tables.reshape(T * S, Do)
     p = layer.hash.projection
     D = p.padded_in_dim
-    diag = p.weight.detach().reshape(1, 4, D)
-    # transpose of x -> FHT(d3*FHT(d2*FHT(d1*FHT(d0*x)))) is g -> d0*FHT(d1*FHT(d2*FHT(d3*FHT(g))))
-    diag_t = torch.stack([torch.ones(D, device=dev), diag[0, 3], diag[0, 2], diag[0, 1]]).reshape(1, 4, D).contiguous()
-    d0 = diag[0, 0].contiguous()
+    diag = p.weight.detach().reshape(1, 4, D).contiguous()
+    h = x_cpu.to(dev)                      # the projection's input (the LayerNorm output in the layer)
 
     def step(events=None):
+        # LookupGather.backward (grad score, grad tables) + ProjectHash.backward (grad of the
+        # projection input, of the diagonals and of the projection bias), as a training step runs them
         g_score = ops.lookup_inner(code, g_out, tables)
         if events is not None:
             events[0].record()
         g_tables = ops.lookup_scatter(code, score, g_out, S)
         if events is not None:
             events[1].record()
-        g_z = ops.code_score_bwd(z, g_score).reshape(B, T * 8)
-        g_h = (ops.bh4_diag((p.decay_coeff * g_z).contiguous(), diag_t) * d0 + (1 - p.decay_coeff) * g_z)[:, :H]
-        return g_score, g_tables, g_z, g_h
+        g_h, g_diag, g_bias = ops.project_hash_bwd(h, diag, z2, g_score, float(p.decay_coeff), float(1 - p.decay_coeff))
+        return g_score, g_tables, g_h, g_diag, g_bias
 
     if args.calibrate_copy:
         calibrate_copy(dev)
@@ -222,7 +222,7 @@ def main_backward(args):
         return a.elapsed_time(b) / n
     inner_ms = timed(lambda: ops.lookup_inner(code, g_out, tables))
     g_score = ops.lookup_inner(code, g_out, tables)
-    bwd_score_ms = timed(lambda: ops.code_score_bwd(z, g_score))
+    bwd_proj_ms = timed(lambda: ops.project_hash_bwd(h, diag, z2, g_score, 0.7, 0.3))
 
     res = {
         "metric": "LookupFFN bwd tokens/s + scatter-add GB/s as % of HBM peak, RoBERTa-base shape, Zipf(1.1) codes",
@@ -230,13 +230,13 @@ def main_backward(args):
         "ms_per_step": sec / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic (seeded; codes Zipf(1.1) through a seeded permutation per table)",
         "config": {"workload": wl["desc"], "tokens": B, "tables": T, "table_size": S, "d_out": Do,
-                   "step": "inner product (grad score) + scatter-add (grad tables) + score "
-                           "derivative + transposed BH4(block 1)x4"},
+                   "step": "inner product (grad score) + scatter-add (grad tables) + one kernel: score "
+                           "derivative, transposed BH4(block 1)x4, grad of diagonals and bias"},
         "roofline": {"bound": "hbm", "kernel": "lookup_scatter", "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get("cfg5"),
                      "algorithmic_bytes": scatter_bytes, "avg_kernel_ms": scatter_ms},
-        "stages_ms": {"lookup_inner": inner_ms, "scatter_add": scatter_ms, "code_score_bwd": bwd_score_ms},
+        "stages_ms": {"lookup_inner": inner_ms, "scatter_add": scatter_ms, "project_hash_bwd": bwd_proj_ms},
     }
     if not args.no_cpu_baseline:
         import oracle
