@@ -91,8 +91,14 @@ struct BlockArgs {
     float decay, residual;
 };
 
-template <int NB, bool HASH>
-__global__ __launch_bounds__(256) void bh4_block_kernel(BlockArgs a) {
+// NH = token halves per wavefront.  NH == 2: 4 wavefronts, each both 16-token halves (a weight
+// fragment is fetched once per workgroup).  NH == 1: 8 wavefronts, wavefront w and w+4 own the
+// same output columns for one half each (the fragment is fetched twice, the second time mostly
+// from the L1), two wavefronts per SIMD: the phases that are not products (tile load and
+// LayerNorm, butterflies, stage hand-over, hash) run on twice the wavefronts.
+template <int NB, bool HASH, int NH>
+__global__ __launch_bounds__(128 * (4 / NH)) void bh4_block_kernel(BlockArgs a) {
+    constexpr int NWAVE = 4 * (2 / NH);
     const float *__restrict__ x = a.x;
     const float *__restrict__ wf = a.wf;
     const int64_t B = a.B;
@@ -109,12 +115,14 @@ __global__ __launch_bounds__(256) void bh4_block_kernel(BlockArgs a) {
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;                    // output columns [16*wave, 16*wave + 16) of each block
+    const int wave = tid >> 6;
+    const int ow = wave & 3;                      // output columns [16*ow, 16*ow + 16) of each block
+    const int hg = wave >> 2;                     // NH == 1: the token half of this wavefront
     const int c = lane & 15;                      // A operand: output column; B operand and result: token
     const int kq = lane >> 4;                     // k index inside an MFMA; result: output columns 4*kq .. 4*kq+3
     const int64_t tok_base = int64_t(blockIdx.x) * TOK;
     if (HASH && a.ln_w) {
-        for (int e = tid * 4; e < D; e += 1024) {
+        for (int e = tid * 4; e < D; e += 256 * NWAVE) {
             const bool in = e < H;
             *reinterpret_cast<float4 *>(lnw_s + e) = in ? *reinterpret_cast<const float4 *>(a.ln_w + e)
                                                         : make_float4(0.f, 0.f, 0.f, 0.f);
@@ -125,11 +133,11 @@ __global__ __launch_bounds__(256) void bh4_block_kernel(BlockArgs a) {
 
     // this lane's weight fragment of block n, quarter q (input columns 16*kq + 4*q .. +3 of output
     // column 16*wave + c): wf[..][n][wave][q][lane][0..3]
-    const int w_lane_off = wave * 1024 + lane * 4;
+    const int w_lane_off = ow * 1024 + lane * 4;
     // this lane's token values of block n, half h: xs[(16*h + c) * LDR + 64*n + 16*kq ..]
     const int x_lane_off = c * LDR + 16 * kq;
     // where this lane's results of block n, half h go: xs[(16*h + c) * LDR + 64*n + 16*wave + 4*kq ..]
-    const int y_lane_off = c * LDR + 16 * wave + 4 * kq;
+    const int y_lane_off = c * LDR + 16 * ow + 4 * kq;
 
     auto load_w = [&](const float *wst, int n, int q) {
         return *reinterpret_cast<const float4 *>(wst + n * (BS * BS) + q * 256);
@@ -141,10 +149,10 @@ __global__ __launch_bounds__(256) void bh4_block_kernel(BlockArgs a) {
     for (int r = 0; r < R; ++r) {
         __syncthreads();                          // the previous repeat's last stage has been read
         {
-            // A wavefront loads 8 rows, 16 bytes per lane and 1 KB of a row per instruction, all
+            // A wavefront loads TOK/NWAVE rows, 16 bytes per lane and 1 KB of a row per instruction, all
             // loads in flight before the first use (one at a time, each would pay the full
             // memory latency).  Columns at or beyond H are zero.
-            constexpr int RPW = TOK / 4;
+            constexpr int RPW = TOK / NWAVE;
             constexpr int NQ = D >= 256 ? D / 256 : 1;
             float4 v[RPW][NQ];
 #pragma unroll
@@ -219,33 +227,29 @@ __global__ __launch_bounds__(256) void bh4_block_kernel(BlockArgs a) {
 #pragma unroll 1
         for (int s = 0; s < J; ++s) {
             const float *wst = wf + (size_t)((r * J + s) * NB) * (BS * BS) + w_lane_off;
-            f32x4 acc[2][NB];
+            f32x4 acc[NH][NB];
 #pragma unroll
-            for (int n = 0; n < NB; ++n) {
-                acc[0][n] = (f32x4){0.f, 0.f, 0.f, 0.f};
-                acc[1][n] = (f32x4){0.f, 0.f, 0.f, 0.f};
-            }
+            for (int n = 0; n < NB; ++n)
+#pragma unroll
+                for (int t = 0; t < NH; ++t) acc[t][n] = (f32x4){0.f, 0.f, 0.f, 0.f};
             if constexpr (!AHEAD) {
 #pragma unroll
                 for (int q = 0; q < 4; ++q)
 #pragma unroll
                     for (int g = 0; g < G; ++g) wq[g][q] = load_w(wst, g, q);
             }
-            float4 xa[NS][4], xb[NS][4];          // token values, halves 0 and 1
+            float4 xv[NH][NS][4];                 // token values of this wavefront's halves
 #pragma unroll
             for (int q = 0; q < 4; ++q)
 #pragma unroll
-                for (int g = 0; g < G; ++g) {
-                    xa[g][q] = read_x(0, g, q);
-                    xb[g][q] = read_x(1, g, q);
-                }
+                for (int g = 0; g < G; ++g)
+#pragma unroll
+                    for (int t = 0; t < NH; ++t) xv[t][g][q] = read_x(hg * NH + t, g, q);
 
-            // A wavefront is alone on its SIMD and issues in order.  Two things keep the matrix
-            // core busy: (1) a product that accumulates into the result of an earlier one waits
-            // for it, and two chains in flight (the two token halves of one block) left the
-            // core idle 45 % of the time, so two blocks are worked on together: four independent
-            // chains; (2) the loads for the next pair of blocks are spread between the products
-            // instead of queueing in a burst at the LDS and the texture unit.
+            // Wavefronts issue in order and there are one or two per SIMD: the loads for the next
+            // pair of blocks are spread between the products instead of queueing in a burst at the
+            // LDS and the texture unit, and two blocks are worked on together (2*NH independent
+            // accumulation chains).
             static_for<NB / G>([&](auto p_c) {
                 constexpr int n0 = decltype(p_c)::value * G;
                 constexpr int n1 = n0 + G - 1;                  // == n0 when G == 1
@@ -254,48 +258,46 @@ __global__ __launch_bounds__(256) void bh4_block_kernel(BlockArgs a) {
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     const float4 w0v = wq[n0 % NS][q], w1v = wq[n1 % NS][q];
-                    const float4 a0 = xa[n0 % NS][q], b0 = xb[n0 % NS][q];
-                    const float4 a1 = xa[n1 % NS][q], b1 = xb[n1 % NS][q];
                     if constexpr (more) wq[m0][q] = load_w(wst, n0 + G, q);
                     __builtin_amdgcn_sched_barrier(0);
-                    LFFN_MFMA(acc[0][n0], w0v.x, a0.x);
-                    LFFN_MFMA(acc[1][n0], w0v.x, b0.x);
+#pragma unroll
+                    for (int t = 0; t < NH; ++t) LFFN_MFMA(acc[t][n0], w0v.x, xv[t][n0 % NS][q].x);
                     if constexpr (G == 2) {
-                        LFFN_MFMA(acc[0][n1], w1v.x, a1.x);
-                        LFFN_MFMA(acc[1][n1], w1v.x, b1.x);
+#pragma unroll
+                        for (int t = 0; t < NH; ++t) LFFN_MFMA(acc[t][n1], w1v.x, xv[t][n1 % NS][q].x);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                     if constexpr (more) {
-                        xa[m0][q] = read_x(0, n0 + G, q);
-                        xb[m0][q] = read_x(1, n0 + G, q);
+#pragma unroll
+                        for (int t = 0; t < NH; ++t) xv[t][m0][q] = read_x(hg * NH + t, n0 + G, q);
                     }
                     __builtin_amdgcn_sched_barrier(0);
-                    LFFN_MFMA(acc[0][n0], w0v.y, a0.y);
-                    LFFN_MFMA(acc[1][n0], w0v.y, b0.y);
+#pragma unroll
+                    for (int t = 0; t < NH; ++t) LFFN_MFMA(acc[t][n0], w0v.y, xv[t][n0 % NS][q].y);
                     if constexpr (G == 2) {
-                        LFFN_MFMA(acc[0][n1], w1v.y, a1.y);
-                        LFFN_MFMA(acc[1][n1], w1v.y, b1.y);
+#pragma unroll
+                        for (int t = 0; t < NH; ++t) LFFN_MFMA(acc[t][n1], w1v.y, xv[t][n1 % NS][q].y);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                     if constexpr (more && G == 2) wq[m1][q] = load_w(wst, n1 + G, q);
                     __builtin_amdgcn_sched_barrier(0);
-                    LFFN_MFMA(acc[0][n0], w0v.z, a0.z);
-                    LFFN_MFMA(acc[1][n0], w0v.z, b0.z);
+#pragma unroll
+                    for (int t = 0; t < NH; ++t) LFFN_MFMA(acc[t][n0], w0v.z, xv[t][n0 % NS][q].z);
                     if constexpr (G == 2) {
-                        LFFN_MFMA(acc[0][n1], w1v.z, a1.z);
-                        LFFN_MFMA(acc[1][n1], w1v.z, b1.z);
+#pragma unroll
+                        for (int t = 0; t < NH; ++t) LFFN_MFMA(acc[t][n1], w1v.z, xv[t][n1 % NS][q].z);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                     if constexpr (more && G == 2) {
-                        xa[m1][q] = read_x(0, n1 + G, q);
-                        xb[m1][q] = read_x(1, n1 + G, q);
+#pragma unroll
+                        for (int t = 0; t < NH; ++t) xv[t][m1][q] = read_x(hg * NH + t, n1 + G, q);
                     }
                     __builtin_amdgcn_sched_barrier(0);
-                    LFFN_MFMA(acc[0][n0], w0v.w, a0.w);
-                    LFFN_MFMA(acc[1][n0], w0v.w, b0.w);
+#pragma unroll
+                    for (int t = 0; t < NH; ++t) LFFN_MFMA(acc[t][n0], w0v.w, xv[t][n0 % NS][q].w);
                     if constexpr (G == 2) {
-                        LFFN_MFMA(acc[0][n1], w1v.w, a1.w);
-                        LFFN_MFMA(acc[1][n1], w1v.w, b1.w);
+#pragma unroll
+                        for (int t = 0; t < NH; ++t) LFFN_MFMA(acc[t][n1], w1v.w, xv[t][n1 % NS][q].w);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -318,7 +320,7 @@ __global__ __launch_bounds__(256) void bh4_block_kernel(BlockArgs a) {
                 for (int n = 0; n < NB; ++n) {
                     if ((n & h) == 0) {
 #pragma unroll
-                        for (int t = 0; t < 2; ++t) {
+                        for (int t = 0; t < NH; ++t) {
                             const f32x4 lo = acc[t][n], hi = acc[t][n + h];
                             acc[t][n] = lo + hi;
                             acc[t][n + h] = lo - hi;
@@ -330,18 +332,18 @@ __global__ __launch_bounds__(256) void bh4_block_kernel(BlockArgs a) {
             __syncthreads();                      // every wavefront has read this stage's input
             if (s + 1 < J) {
 #pragma unroll
-                for (int n = 0; n < NB; ++n) {
-                    *reinterpret_cast<f32x4 *>(xs + y_lane_off + n * BS) = acc[0][n];
-                    *reinterpret_cast<f32x4 *>(xs + 16 * LDR + y_lane_off + n * BS) = acc[1][n];
-                }
+                for (int n = 0; n < NB; ++n)
+#pragma unroll
+                    for (int t = 0; t < NH; ++t)
+                        *reinterpret_cast<f32x4 *>(xs + (hg * NH + t) * 16 * LDR + y_lane_off + n * BS) = acc[t][n];
                 __syncthreads();
             } else if constexpr (!HASH) {
                 const int64_t ld_out = int64_t(R) * D;
 #pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    const int64_t tok = tok_base + 16 * t + c;
+                for (int t = 0; t < NH; ++t) {
+                    const int64_t tok = tok_base + 16 * (hg * NH + t) + c;
                     if (tok < B) {
-                        float *o = a.out + tok * ld_out + (size_t)r * D + 16 * wave + 4 * kq;
+                        float *o = a.out + tok * ld_out + (size_t)r * D + 16 * ow + 4 * kq;
 #pragma unroll
                         for (int n = 0; n < NB; ++n) *reinterpret_cast<f32x4 *>(o + n * BS) = acc[t][n];
                     }
@@ -355,20 +357,21 @@ __global__ __launch_bounds__(256) void bh4_block_kernel(BlockArgs a) {
                 // zero they are formed here instead of being kept in registers through the stages
                 int opq = 0;
                 asm volatile("" : "+v"(opq));
-                int64_t tokv[2];
-                bool livev[2];
-                float meanv[2], rstdv[2];
-                // the two tokens' input values for every block, all requested before the first use
-                float4 xin[2][NB];
+                int64_t tokv[NH];
+                bool livev[NH];
+                float meanv[NH], rstdv[NH];
+                // the tokens' input values for every block, all requested before the first use
+                float4 xin[NH][NB];
 #pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    tokv[t] = tok_base + 16 * t + c + opq;
+                for (int t = 0; t < NH; ++t) {
+                    const int trow = 16 * (hg * NH + t) + c + opq;     // token within the tile
+                    tokv[t] = tok_base + trow;
                     livev[t] = tokv[t] < B;
-                    meanv[t] = a.ln_w ? stats[2 * (16 * t + c + opq)] : 0.f;
-                    rstdv[t] = a.ln_w ? stats[2 * (16 * t + c + opq) + 1] : 1.f;
+                    meanv[t] = a.ln_w ? stats[2 * trow] : 0.f;
+                    rstdv[t] = a.ln_w ? stats[2 * trow + 1] : 1.f;
 #pragma unroll
                     for (int n = 0; n < NB; ++n) {
-                        const int xc = n * BS + 16 * wave + 4 * kq + opq;
+                        const int xc = n * BS + 16 * ow + 4 * kq + opq;
                         xin[t][n] = (livev[t] && xc < H) ? *reinterpret_cast<const float4 *>(x + tokv[t] * H + xc)
                                                          : make_float4(0.f, 0.f, 0.f, 0.f);
                     }
@@ -376,7 +379,7 @@ __global__ __launch_bounds__(256) void bh4_block_kernel(BlockArgs a) {
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int n = 0; n < NB; ++n) {
-                    const int xc = n * BS + 16 * wave + 4 * kq + opq;      // column of the padded input
+                    const int xc = n * BS + 16 * ow + 4 * kq + opq;        // column of the padded input
                     const int col = r * D + xc;                            // column of z
                     const bool in_cols = col < ncols;                      // whole groups of 8: all or nothing
                     float4 lw = make_float4(0.f, 0.f, 0.f, 0.f), lb = lw, bb = lw;
@@ -385,10 +388,9 @@ __global__ __launch_bounds__(256) void bh4_block_kernel(BlockArgs a) {
                         lb = *reinterpret_cast<const float4 *>(lnb_s + xc);
                     }
                     if (a.pbias && in_cols) bb = *reinterpret_cast<const float4 *>(a.pbias + col);
-                    // the two token halves side by side: independent work for a wavefront that has
-                    // its SIMD to itself
+                    // the token halves of this wavefront side by side: independent work
 #pragma unroll
-                    for (int t = 0; t < 2; ++t) {
+                    for (int t = 0; t < NH; ++t) {
                         float4 xv = xin[t][n];
                         if (a.ln_w && xc < H) {
                             xv.x = (xv.x - meanv[t]) * rstdv[t] * lw.x + lb.x;
@@ -426,16 +428,16 @@ __global__ __launch_bounds__(256) void bh4_block_kernel(BlockArgs a) {
                         // staged in LDS (the stage buffer is free now), written out row by row below:
                         // straight from here a store would scatter 4-byte pieces over 32 rows
                         if (kq & 1) {
-                            cs[(16 * t + c) * CROW + (xc >> 3)] = (nib_hi << 4) | nib;
-                            ss[(16 * t + c) * CROW + (xc >> 3)] = s_run / p_run;
+                            cs[(16 * (hg * NH + t) + c) * CROW + (xc >> 3)] = (nib_hi << 4) | nib;
+                            ss[(16 * (hg * NH + t) + c) * CROW + (xc >> 3)] = s_run / p_run;
                         }
                     }
                 }
                 __syncthreads();
-                // wavefront w writes the D/8 codes and scores of tokens 8w .. 8w+7
+                // every wavefront writes the D/8 codes and scores of TOK/NWAVE tokens
 #pragma unroll 1
-                for (int i = 0; i < TOK / 4; ++i) {
-                    const int row = wave * (TOK / 4) + i;
+                for (int i = 0; i < TOK / NWAVE; ++i) {
+                    const int row = wave * (TOK / NWAVE) + i;
                     const int64_t tok = tok_base + row;
                     if (tok >= B) break;
 #pragma unroll
@@ -453,27 +455,30 @@ __global__ __launch_bounds__(256) void bh4_block_kernel(BlockArgs a) {
     }
 }
 
-template <int NB, bool HASH>
+template <int NB, bool HASH, int NH>
 int launch_block(const BlockArgs &a, hipStream_t st) {
     const size_t lds_bytes = (size_t(TOK) * (BS * NB + PAD) + 2 * TOK + (HASH ? 2 * BS * NB : 0)) * sizeof(float);
-    auto kern = bh4_block_kernel<NB, HASH>;
+    auto kern = bh4_block_kernel<NB, HASH, NH>;
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds_bytes) != hipSuccess) {
         (void)hipGetLastError();
         return LFFN_ERR_LAUNCH;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)((a.B + TOK - 1) / TOK)), dim3(256), lds_bytes, st, a);
+    hipLaunchKernelGGL(kern, dim3((unsigned)((a.B + TOK - 1) / TOK)), dim3(128 * (4 / NH)), lds_bytes, st, a);
     return lffn_launch_status();
 }
 
 template <bool HASH>
 int dispatch_block(const BlockArgs &a, int64_t D, hipStream_t st) {
     switch (D / BS) {
-        case 1: return launch_block<1, HASH>(a, st);
-        case 2: return launch_block<2, HASH>(a, st);
-        case 4: return launch_block<4, HASH>(a, st);
-        case 8: return launch_block<8, HASH>(a, st);
-        default: return launch_block<16, HASH>(a, st);
+        case 1: return launch_block<1, HASH, 2>(a, st);
+        case 2: return launch_block<2, HASH, 2>(a, st);
+        case 4: return launch_block<4, HASH, 2>(a, st);
+        case 8: return launch_block<8, HASH, 2>(a, st);
+        // measured at 16384 x 1024: the plain form 110 us with 4 wavefronts, 118 us with 8 (the
+        // second fetch of the weight fragments costs more than the other phases gain); the hash
+        // form 141 us with 4, 133 us with 8 (LayerNorm and the hash are vector-ALU work)
+        default: return HASH ? launch_block<16, HASH, 1>(a, st) : launch_block<16, HASH, 2>(a, st);
     }
 }
 
