@@ -348,6 +348,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--graph", action="store_true",
+                    help="forward workloads: capture the step in a HIP graph and time replays (the launch-bound "
+                         "small configurations); the gather's own duration is then measured in an eager loop")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device-to-device copy, so that a rocprofv3 --pmc run of "
                          "this command holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -405,12 +408,33 @@ def main():
     torch.cuda.synchronize()
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        out = step(evs[i])
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    sec = t1 - t0
+    if args.graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            graph_out = step()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(graph_out, step()), "graph replay and eager step disagree"
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        sec = time.perf_counter() - t0
+        for i in range(args.steps):                       # the gather's duration: eager, with events
+            step(evs[i])
+        torch.cuda.synchronize()
+    else:
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            out = step(evs[i])
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        sec = t1 - t0
     gather_ms = sum(a.elapsed_time(b) for a, b in evs) / args.steps
     achieved = gather_bytes / (gather_ms * 1e-3) / 1e9
 
@@ -452,6 +476,7 @@ def main():
         "stages_ms": {("layernorm_bh4block_hash" if block else "layernorm_project_hash"): hash_ms,
                       "gather_add": gather_ms},
         "gather_tokens_per_s": B / (gather_ms * 1e-3),
+        "launch": "HIP graph replay" if args.graph else "eager",
     }
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(layer, x_cpu, wl)

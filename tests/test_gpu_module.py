@@ -310,3 +310,31 @@ def test_checkpoint_round_trip_and_folded_weight_cache(tmp_path):
         # an in-place update (an optimizer step) is seen as well
         b.hash.projection.weight.mul_(0.5)
         assert not torch.equal(b(x), out_a)
+
+
+def test_layer_forward_under_graph_capture():
+    """The eval forward (two kernels, outputs from torch's allocator) can be captured in a HIP
+    graph and replayed: every replay, with eager work and synchronisations in between, gives
+    the eager result for the inputs then in the static buffer."""
+    torch.manual_seed(31)
+    layer = lookupffn_amd.LookupFFN(_config(hidden_size=256, ffn_num_table=32), 256).eval().to(DEV)
+    static_x = torch.randn(256, 256, device=DEV)
+    with torch.no_grad():
+        for _ in range(3):                                 # warm-up on a side stream, as torch asks
+            s = torch.cuda.Stream()
+            s.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(s):
+                layer(static_x)
+            torch.cuda.current_stream().wait_stream(s)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            static_out = layer(static_x)
+        for i in range(4):
+            x = torch.randn(256, 256, device=DEV)
+            static_x.copy_(x)
+            g.replay()
+            torch.cuda.synchronize()
+            got = static_out.clone()
+            want = layer(x)                                # eager work between the replays
+            torch.cuda.synchronize()
+            assert torch.equal(got, want), i
