@@ -135,6 +135,38 @@ int lffn_ln_bh4_block_hash_f32(const float *x, const float *ln_weight, const flo
                                int64_t block_size, float decay, float residual, void *stream);
 
 /*
+ * Training form of the 64 x 64-block front end and its backward.
+ *
+ * lffn_bh4_block_hash_train_f32: as lffn_ln_bh4_block_hash_f32 without LayerNorm, and keeping
+ * what the backward needs: z [B, T*8] and stage_inputs [R, J-1, B, D], the input of stages
+ * 1 .. J-1 (the input of stage 0 is pad(x)).
+ *
+ * lffn_bh4_fold_mode_f32: the 64-point transform down the output index of num_blocks 64 x 64
+ * blocks, written in one of three orders: mode 0 = what the forward kernels fetch (as
+ * lffn_bh4_fold_f32), mode 1 = what lffn_bh4_block_bwd_f32 fetches (transposed blocks),
+ * mode 2 = natural [o][i] order (applied to a gradient w.r.t. the folded weights it gives the
+ * gradient w.r.t. the weights).
+ *
+ * lffn_bh4_block_bwd_f32: from g_z [B, T*8] (the gradient of z, e.g. from
+ * lffn_code_score_bwd_f32) and the mode-1 folded weights: g_x [R, B, H], one slab per repeat
+ * (the caller adds them), and stage_grads [R, J, B, D], the gradient in front of each stage's
+ * block product after the cross-block part of the transform.  The gradient w.r.t. the folded
+ * weights of block n of stage (r, j) is  sum_b stage_grads[r,j,b,64n+o] * input[r,j,b,64n+i];
+ * the caller forms it (a batched product over the tokens) and applies mode 2.
+ * Replaces what autograd records for bh4_cuda with block_size == 64 (PL/bh4/kernel.py:23-36)
+ * and the mix of BH4._forward (PL/lookup.py:36-37).
+ */
+int lffn_bh4_block_hash_train_f32(const float *x, const float *w_folded, const float *proj_bias,
+                                  int32_t *codes, float *scores, float *z, float *stage_inputs,
+                                  int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
+                                  int64_t block_size, float decay, float residual, void *stream);
+int lffn_bh4_fold_mode_f32(const float *w, float *out, int64_t num_blocks, int64_t block_size,
+                           int32_t mode, void *stream);
+int lffn_bh4_block_bwd_f32(const float *g_z, const float *w_folded_t, float *g_x, float *stage_grads,
+                           int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
+                           int64_t block_size, float decay, float residual, void *stream);
+
+/*
  * The tail of the BH4 module and the hash in one pass, for any block size:
  *   z[b, c] = decay * y[b, c] + residual * pad(x)[b, c % D] + bias[c],  c < T*k
  *   (code, score)[b, t] = code and score of z[b, t*k : (t+1)*k]   (as lffn_code_score_f32)

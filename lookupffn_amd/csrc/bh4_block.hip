@@ -47,6 +47,11 @@ constexpr int PAD = 4;          // floats of padding per LDS row
 // 64-point unnormalised Hadamard transform down the output index o of every block:
 // wf[blk]{o', i} = sum_o H64[o'][o] * w[blk][o][i], stored in the order the product kernel's
 // lanes fetch it.  One lane per (blk, i).
+// MODE 0: the order the forward product fetches (below).  MODE 1: the order the backward
+// product fetches, whose A operand is the transposed block: rows = input index i, k = output
+// index o'.  MODE 2: natural [o'][i] order (turns a gradient w.r.t. the folded weights into the
+// gradient w.r.t. the weights: H64 is symmetric).
+template <int MODE>
 __global__ __launch_bounds__(256) void bh4_fold_kernel(const float *w, float *wf, int64_t nblk) {
     const int64_t gid = int64_t(blockIdx.x) * 256 + threadIdx.x;
     if (gid >= nblk * BS) return;
@@ -67,11 +72,22 @@ __global__ __launch_bounds__(256) void bh4_fold_kernel(const float *w, float *wf
             }
         }
     }
-    // fragment order: [wavefront = o/16][q = (i%16)/4][lane = 16*(i/16) + o%16][i%4], so that a
-    // wavefront's load of (block, q) is 1 KB of contiguous memory, 16 bytes per lane
-    float *dst = wf + blk * (BS * BS) + ((i % 16) / 4) * 256 + (i / 16) * 64 + (i % 4);
+    if constexpr (MODE == 0) {
+        // fragment order: [wavefront = o/16][q = (i%16)/4][lane = 16*(i/16) + o%16][i%4], so that a
+        // wavefront's load of (block, q) is 1 KB of contiguous memory, 16 bytes per lane
+        float *dst = wf + blk * (BS * BS) + ((i % 16) / 4) * 256 + (i / 16) * 64 + (i % 4);
 #pragma unroll
-    for (int o = 0; o < BS; ++o) dst[(o / 16) * 1024 + (o % 16) * 4] = v[o];
+        for (int o = 0; o < BS; ++o) dst[(o / 16) * 1024 + (o % 16) * 4] = v[o];
+    } else if constexpr (MODE == 1) {
+        // the same with the roles of o and i exchanged: [i/16][(o%16)/4][16*(o/16) + i%16][o%4]
+        float *dst = wf + blk * (BS * BS) + (i / 16) * 1024 + (i % 16) * 4;
+#pragma unroll
+        for (int o = 0; o < BS; ++o) dst[((o % 16) / 4) * 256 + (o / 16) * 64 + (o % 4)] = v[o];
+    } else {
+        float *dst = wf + blk * (BS * BS) + i;
+#pragma unroll
+        for (int o = 0; o < BS; ++o) dst[o * BS] = v[o];
+    }
 }
 
 #define LFFN_MFMA(acc, a, b) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc, 0, 0, 0)
@@ -86,6 +102,10 @@ struct BlockArgs {
     const float *pbias;    // [T*8] or null       (hash form)
     int32_t *codes;        // [B, T]              (hash form)
     float *scores;         // [B, T]              (hash form)
+    float *z_out;          // [B, T*8] or null    (hash form: z kept for the backward)
+    float *stage_save;     // forward: [R, J-1, B, D] inputs of stages 1..J-1, or null;
+                           // backward: [R, J, B, D] gradient before the product of each stage
+    const float *gz;       // [B, T*8]            (backward form: gradient of z)
     int64_t B;
     int H, R, J, T;
     float decay, residual;
@@ -96,8 +116,19 @@ struct BlockArgs {
 // same output columns for one half each (the fragment is fetched twice, the second time mostly
 // from the L1), two wavefronts per SIMD: the phases that are not products (tile load and
 // LayerNorm, butterflies, stage hand-over, hash) run on twice the wavefronts.
-template <int NB, bool HASH, int NH>
+//
+// BWD: the backward through the stages with the same machinery.  With G_{s+1} the gradient of a
+// stage's output, the gradient of its input is  W'_s^T (H_NB (x) I_64) G_{s+1}  (H_64 is
+// symmetric and already inside W' = H_64 W): the butterflies across blocks run BEFORE the
+// product, as a pass over the LDS tile, the product takes the folded weights in transposed
+// fragment order (bh4_fold_kernel<1>), and nothing follows it.  The butterflied gradient
+// P_s = (H_NB (x) I) G_{s+1} is also written to memory: the gradient w.r.t. the folded
+// weights is the per-block product P_s^T U_s over all tokens (U_s = the stage's input, which
+// the forward saved), formed by the caller.  Tile load: decay * grad z; result: grad x of
+// this repeat = G_0[:, :H] + residual * grad z[:, :H].
+template <int NB, bool HASH, int NH, bool BWD = false>
 __global__ __launch_bounds__(128 * (4 / NH)) void bh4_block_kernel(BlockArgs a) {
+    static_assert(!(HASH && BWD), "one form at a time");
     constexpr int NWAVE = 4 * (2 / NH);
     const float *__restrict__ x = a.x;
     const float *__restrict__ wf = a.wf;
@@ -161,11 +192,19 @@ __global__ __launch_bounds__(128 * (4 / NH)) void bh4_block_kernel(BlockArgs a) 
 #pragma unroll
                 for (int q = 0; q < NQ; ++q) {
                     const int col = (q * 64 + lane) * 4;
-                    v[i][q] = (tok < B && col < H) ? *reinterpret_cast<const float4 *>(x + tok * H + col)
-                                                   : make_float4(0.f, 0.f, 0.f, 0.f);
+                    if constexpr (BWD) {
+                        const int gcol = r * D + col;
+                        float4 g4 = make_float4(0.f, 0.f, 0.f, 0.f);
+                        if (tok < B && col < D && gcol < a.T * 8)
+                            g4 = *reinterpret_cast<const float4 *>(a.gz + tok * (a.T * 8) + gcol);
+                        v[i][q] = make_float4(a.decay * g4.x, a.decay * g4.y, a.decay * g4.z, a.decay * g4.w);
+                    } else {
+                        v[i][q] = (tok < B && col < H) ? *reinterpret_cast<const float4 *>(x + tok * H + col)
+                                                       : make_float4(0.f, 0.f, 0.f, 0.f);
+                    }
                 }
             }
-            if (a.ln_w) {
+            if (!BWD && a.ln_w) {
                 // LayerNorm over the H valid columns (biased variance, two passes, eps inside the
                 // square root: torch.nn.LayerNorm, PL/lookup.py:84,99)
                 float4 lw[NQ], lb[NQ];
@@ -218,15 +257,45 @@ __global__ __launch_bounds__(128 * (4 / NH)) void bh4_block_kernel(BlockArgs a) 
 
         float4 wq[NS][4];                         // weight fragments
         if constexpr (AHEAD) {
-            const float *w0 = wf + (size_t)(r * J * NB) * (BS * BS) + w_lane_off;
+            const float *w0 = wf + (size_t)((r * J + (BWD ? J - 1 : 0)) * NB) * (BS * BS) + w_lane_off;
 #pragma unroll
             for (int q = 0; q < 4; ++q)
 #pragma unroll
                 for (int g = 0; g < G; ++g) wq[g][q] = load_w(w0, g, q);
         }
 #pragma unroll 1
-        for (int s = 0; s < J; ++s) {
+        for (int si = 0; si < J; ++si) {
+            const int s = BWD ? J - 1 - si : si;                  // the backward walks the stages down
             const float *wst = wf + (size_t)((r * J + s) * NB) * (BS * BS) + w_lane_off;
+            if constexpr (BWD) {
+                // butterflies across the blocks on the LDS tile, 16 bytes of every block per thread;
+                // the result is this stage's P, kept for the weight gradient
+                for (int e = tid; e < TOK * 16; e += 64 * NWAVE) {
+                    const int row = e / 16, c4 = (e % 16) * 4;
+                    f32x4 pv[NB];
+#pragma unroll
+                    for (int n = 0; n < NB; ++n) pv[n] = *reinterpret_cast<const f32x4 *>(xs + row * LDR + n * BS + c4);
+#pragma unroll
+                    for (int h = NB / 2; h >= 1; h >>= 1) {
+#pragma unroll
+                        for (int n = 0; n < NB; ++n) {
+                            if ((n & h) == 0) {
+                                const f32x4 lo = pv[n], hi = pv[n + h];
+                                pv[n] = lo + hi;
+                                pv[n + h] = lo - hi;
+                            }
+                        }
+                    }
+                    const int64_t tok = tok_base + row;
+                    float *ps = a.stage_save + ((size_t(r) * J + s) * B + tok) * D + c4;
+#pragma unroll
+                    for (int n = 0; n < NB; ++n) {
+                        *reinterpret_cast<f32x4 *>(xs + row * LDR + n * BS + c4) = pv[n];
+                        if (tok < B) *reinterpret_cast<f32x4 *>(ps + n * BS) = pv[n];
+                    }
+                }
+                __syncthreads();
+            }
             f32x4 acc[NH][NB];
 #pragma unroll
             for (int n = 0; n < NB; ++n)
@@ -305,7 +374,8 @@ __global__ __launch_bounds__(128 * (4 / NH)) void bh4_block_kernel(BlockArgs a) 
             // the next stage's first blocks (a harmless re-read after the last stage): every product
             // that read slots 0 .. G-1 was issued at least one pair ago
             if constexpr (AHEAD) {
-                const float *wnx = wf + (size_t)((r * J + min(s + 1, J - 1)) * NB) * (BS * BS) + w_lane_off;
+                const int sn = BWD ? max(s - 1, 0) : min(s + 1, J - 1);
+                const float *wnx = wf + (size_t)((r * J + sn) * NB) * (BS * BS) + w_lane_off;
 #pragma unroll
                 for (int q = 0; q < 4; ++q)
 #pragma unroll
@@ -313,30 +383,66 @@ __global__ __launch_bounds__(128 * (4 / NH)) void bh4_block_kernel(BlockArgs a) 
                 __builtin_amdgcn_sched_barrier(0);
             }
 
-            // H_NB across the blocks
+            // H_NB across the blocks (the backward did it before the product)
+            if constexpr (!BWD) {
 #pragma unroll
-            for (int h = NB / 2; h >= 1; h >>= 1) {
+                for (int h = NB / 2; h >= 1; h >>= 1) {
 #pragma unroll
-                for (int n = 0; n < NB; ++n) {
-                    if ((n & h) == 0) {
+                    for (int n = 0; n < NB; ++n) {
+                        if ((n & h) == 0) {
 #pragma unroll
-                        for (int t = 0; t < NH; ++t) {
-                            const f32x4 lo = acc[t][n], hi = acc[t][n + h];
-                            acc[t][n] = lo + hi;
-                            acc[t][n + h] = lo - hi;
+                            for (int t = 0; t < NH; ++t) {
+                                const f32x4 lo = acc[t][n], hi = acc[t][n + h];
+                                acc[t][n] = lo + hi;
+                                acc[t][n + h] = lo - hi;
+                            }
                         }
                     }
                 }
             }
 
             __syncthreads();                      // every wavefront has read this stage's input
-            if (s + 1 < J) {
+            if (si + 1 < J) {
 #pragma unroll
                 for (int n = 0; n < NB; ++n)
 #pragma unroll
                     for (int t = 0; t < NH; ++t)
                         *reinterpret_cast<f32x4 *>(xs + (hg * NH + t) * 16 * LDR + y_lane_off + n * BS) = acc[t][n];
+                if (!BWD && a.stage_save) {
+                    // the input of stage s+1, kept for the weight gradient of the backward
+#pragma unroll
+                    for (int t = 0; t < NH; ++t) {
+                        const int64_t tok = tok_base + 16 * (hg * NH + t) + c;
+                        if (tok < B) {
+                            float *o = a.stage_save + ((size_t(r) * (J - 1) + s) * B + tok) * D + 16 * ow + 4 * kq;
+#pragma unroll
+                            for (int n = 0; n < NB; ++n) *reinterpret_cast<f32x4 *>(o + n * BS) = acc[t][n];
+                        }
+                    }
+                }
                 __syncthreads();
+            } else if constexpr (BWD) {
+                // grad x of this repeat: the first H columns, plus the residual path of the mix
+                const int ncols = a.T * 8;
+#pragma unroll
+                for (int t = 0; t < NH; ++t) {
+                    const int64_t tok = tok_base + 16 * (hg * NH + t) + c;
+                    if (tok < B) {
+#pragma unroll
+                        for (int n = 0; n < NB; ++n) {
+                            const int xc = n * BS + 16 * ow + 4 * kq;
+                            if (xc < H) {
+                                f32x4 o = acc[t][n];
+                                if (r * D + xc < ncols) {
+                                    const f32x4 g4 = *reinterpret_cast<const f32x4 *>(a.gz + tok * ncols + r * D + xc);
+                                    o.x = o.x + a.residual * g4.x; o.y = o.y + a.residual * g4.y;
+                                    o.z = o.z + a.residual * g4.z; o.w = o.w + a.residual * g4.w;
+                                }
+                                *reinterpret_cast<f32x4 *>(a.out + (size_t(r) * B + tok) * H + xc) = o;
+                            }
+                        }
+                    }
+                }
             } else if constexpr (!HASH) {
                 const int64_t ld_out = int64_t(R) * D;
 #pragma unroll
@@ -406,6 +512,8 @@ __global__ __launch_bounds__(128 * (4 / NH)) void bh4_block_kernel(BlockArgs a) 
                         if (a.pbias && in_cols) {
                             z[0] = z[0] + bb.x; z[1] = z[1] + bb.y; z[2] = z[2] + bb.z; z[3] = z[3] + bb.w;
                         }
+                        if (a.z_out && in_cols && livev[t])
+                            *reinterpret_cast<float4 *>(a.z_out + tokv[t] * ncols + col) = make_float4(z[0], z[1], z[2], z[3]);
                         // columns 8g .. 8g+3 sit in the lane with even kq (the high nibble),
                         // 8g+4 .. 8g+7 in lane + 16, which continues the sum and the product
                         // (d = 0..7 in order, compute_code_score/torch_extension.cc:31-37)
@@ -455,10 +563,10 @@ __global__ __launch_bounds__(128 * (4 / NH)) void bh4_block_kernel(BlockArgs a) 
     }
 }
 
-template <int NB, bool HASH, int NH>
+template <int NB, bool HASH, int NH, bool BWD = false>
 int launch_block(const BlockArgs &a, hipStream_t st) {
     const size_t lds_bytes = (size_t(TOK) * (BS * NB + PAD) + 2 * TOK + (HASH ? 2 * BS * NB : 0)) * sizeof(float);
-    auto kern = bh4_block_kernel<NB, HASH, NH>;
+    auto kern = bh4_block_kernel<NB, HASH, NH, BWD>;
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds_bytes) != hipSuccess) {
         (void)hipGetLastError();
@@ -466,6 +574,16 @@ int launch_block(const BlockArgs &a, hipStream_t st) {
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)((a.B + TOK - 1) / TOK)), dim3(128 * (4 / NH)), lds_bytes, st, a);
     return lffn_launch_status();
+}
+
+int dispatch_block_bwd(const BlockArgs &a, int64_t D, hipStream_t st) {
+    switch (D / BS) {
+        case 1: return launch_block<1, false, 2, true>(a, st);
+        case 2: return launch_block<2, false, 2, true>(a, st);
+        case 4: return launch_block<4, false, 2, true>(a, st);
+        case 8: return launch_block<8, false, 2, true>(a, st);
+        default: return launch_block<16, false, 1, true>(a, st);
+    }
 }
 
 template <bool HASH>
@@ -491,8 +609,22 @@ extern "C" int lffn_bh4_fold_f32(const float *w, float *w_folded, int64_t R, int
     LFFN_REQUIRE(w && w_folded && w != w_folded, LFFN_ERR_BAD_ARG);
     const int64_t nblk = R * stages * num_block;
     LFFN_REQUIRE(nblk <= (int64_t(1) << 24), LFFN_ERR_UNSUPPORTED);
-    hipLaunchKernelGGL(bh4_fold_kernel, dim3((unsigned)((nblk * BS + 255) / 256)), dim3(256), 0,
+    hipLaunchKernelGGL(bh4_fold_kernel<0>, dim3((unsigned)((nblk * BS + 255) / 256)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), w, w_folded, nblk);
+    return lffn_launch_status();
+}
+
+extern "C" int lffn_bh4_fold_mode_f32(const float *w, float *out, int64_t num_blocks, int64_t block_size,
+                                      int32_t mode, void *stream) {
+    LFFN_REQUIRE(num_blocks >= 0 && num_blocks <= (int64_t(1) << 24), LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(block_size == BS && mode >= 0 && mode <= 2, LFFN_ERR_UNSUPPORTED);
+    if (num_blocks == 0) return LFFN_OK;
+    LFFN_REQUIRE(w && out && w != out, LFFN_ERR_BAD_ARG);
+    const dim3 grid((unsigned)((num_blocks * BS + 255) / 256));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (mode == 0) hipLaunchKernelGGL(bh4_fold_kernel<0>, grid, dim3(256), 0, st, w, out, num_blocks);
+    else if (mode == 1) hipLaunchKernelGGL(bh4_fold_kernel<1>, grid, dim3(256), 0, st, w, out, num_blocks);
+    else hipLaunchKernelGGL(bh4_fold_kernel<2>, grid, dim3(256), 0, st, w, out, num_blocks);
     return lffn_launch_status();
 }
 
@@ -531,4 +663,43 @@ extern "C" int lffn_ln_bh4_block_hash_f32(const float *x, const float *ln_weight
     a.codes = codes; a.scores = scores; a.B = B; a.H = (int)H; a.R = (int)R; a.J = (int)J; a.T = (int)T;
     a.decay = decay; a.residual = residual;
     return dispatch_block<true>(a, D, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int lffn_bh4_block_hash_train_f32(const float *x, const float *w_folded, const float *proj_bias,
+                                             int32_t *codes, float *scores, float *z, float *stage_inputs,
+                                             int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
+                                             int64_t block_size, float decay, float residual, void *stream) {
+    LFFN_REQUIRE(B >= 0 && R >= 1 && J >= 1 && D >= 1 && H >= 1 && H <= D && T >= 1, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(H % 4 == 0 && J <= 64, LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(block_size == BS && lffn_is_pow2(D) && D >= BS && D <= 1024, LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(R <= 4096 && B <= (int64_t(1) << 31) - 1 && T <= (1 << 24), LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(T * 8 <= R * D, LFFN_ERR_BAD_ARG);
+    if (B == 0) return LFFN_OK;
+    LFFN_REQUIRE(x && w_folded && codes && scores && z && (stage_inputs || J == 1), LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_aligned16(x) && lffn_aligned16(w_folded) && lffn_aligned16(z) &&
+                     (!proj_bias || lffn_aligned16(proj_bias)) && (!stage_inputs || lffn_aligned16(stage_inputs)),
+                 LFFN_ERR_BAD_ARG);
+    BlockArgs a{};
+    a.x = x; a.wf = w_folded; a.pbias = proj_bias; a.codes = codes; a.scores = scores; a.z_out = z;
+    a.stage_save = stage_inputs; a.B = B; a.H = (int)H; a.R = (int)R; a.J = (int)J; a.T = (int)T;
+    a.decay = decay; a.residual = residual;
+    return dispatch_block<true>(a, D, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int lffn_bh4_block_bwd_f32(const float *g_z, const float *w_folded_t, float *g_x, float *stage_grads,
+                                      int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
+                                      int64_t block_size, float decay, float residual, void *stream) {
+    LFFN_REQUIRE(B >= 0 && R >= 1 && J >= 1 && D >= 1 && H >= 1 && H <= D && T >= 1, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(H % 4 == 0 && J <= 64, LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(block_size == BS && lffn_is_pow2(D) && D >= BS && D <= 1024, LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(R <= 4096 && B <= (int64_t(1) << 31) - 1 && T <= (1 << 24), LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(T * 8 <= R * D, LFFN_ERR_BAD_ARG);
+    if (B == 0) return LFFN_OK;
+    LFFN_REQUIRE(g_z && w_folded_t && g_x && stage_grads, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_aligned16(g_z) && lffn_aligned16(w_folded_t) && lffn_aligned16(g_x) &&
+                     lffn_aligned16(stage_grads), LFFN_ERR_BAD_ARG);
+    BlockArgs a{};
+    a.gz = g_z; a.wf = w_folded_t; a.out = g_x; a.stage_save = stage_grads;
+    a.B = B; a.H = (int)H; a.R = (int)R; a.J = (int)J; a.T = (int)T; a.decay = decay; a.residual = residual;
+    return dispatch_block_bwd(a, D, static_cast<hipStream_t>(stream));
 }

@@ -92,6 +92,57 @@ class ProjectHash(torch.autograd.Function):
                 g_bias if (ctx.has_bias and ctx.needs_input_grad[2]) else None, None, None)
 
 
+class BlockProjectHash(torch.autograd.Function):
+    """BH4 with 64 x 64 blocks -> mix -> bias -> 8-bit code + score as one differentiable
+    operator.  Forward: one matrix-core kernel that also keeps z and the input of every stage.
+    Backward: the score derivative, one matrix-core kernel walking the stages down (grad x and
+    the gradient in front of every block product), then the weight gradient as a batched product
+    over the tokens of those gradients with the saved stage inputs, taken back through the
+    64-point transform.  Same mathematics as bh4_cuda + BH4._forward + compute_code_score under
+    autograd (PL/bh4/kernel.py:23-36, PL/lookup.py:29-39)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, T, decay):
+        x = x.contiguous()
+        w = weight.contiguous()
+        folded = ops.bh4_fold_mode(w, 0)
+        code, score, z, stage_in = ops.bh4_block_hash_train(x, folded, bias, T, float(decay), float(1 - decay))
+        ctx.save_for_backward(x, w, z, stage_in)
+        ctx.has_bias = bias is not None
+        ctx.decay = float(decay)
+        ctx.mark_non_differentiable(code)
+        return code, score
+
+    @staticmethod
+    def backward(ctx, _g_code, g_score):
+        x, w, z, stage_in = ctx.saved_tensors
+        R, J, NB, bs, _ = w.shape
+        B, H = x.shape
+        T = g_score.shape[1]
+        g_z = ops.code_score_bwd(z.reshape(B, T, 8), g_score.contiguous()).reshape(B, T * 8)
+        g_x, stage_g = ops.bh4_block_bwd(g_z, ops.bh4_fold_mode(w, 1), H, ctx.decay, 1 - ctx.decay)
+        g_w = None
+        if ctx.needs_input_grad[1]:
+            g_folded = torch.empty_like(w)
+            for r in range(R):
+                for j in range(J):
+                    p = stage_g[r, j].view(B, NB, bs)
+                    if j == 0:        # the input of stage 0 is x, zero beyond its H columns
+                        full, rem = H // bs, H % bs
+                        g_folded[r, j].zero_()
+                        if full:
+                            g_folded[r, j, :full] = torch.einsum(
+                                "bno,bni->noi", p[:, :full], x[:, :full * bs].reshape(B, full, bs))
+                        if rem:
+                            g_folded[r, j, full, :, :rem] = p[:, full].t() @ x[:, full * bs:]
+                    else:
+                        g_folded[r, j] = torch.einsum("bno,bni->noi", p, stage_in[r, j - 1].view(B, NB, bs))
+            g_w = ops.bh4_fold_mode(g_folded, 2)
+        g_x = g_x[0] if R == 1 else g_x.sum(0)
+        g_bias = g_z.sum(0) if (ctx.has_bias and ctx.needs_input_grad[2]) else None
+        return (g_x if ctx.needs_input_grad[0] else None, g_w, g_bias, None, None)
+
+
 class Hashing(nn.Module):
     """PL/lookup.py:49-77."""
 
@@ -178,15 +229,25 @@ class Hashing(nn.Module):
                 and 256 <= p.padded_in_dim <= 1024 and p.weight.shape[1] <= 4 and p.in_dim % 4 == 0
                 and x.dtype == torch.float32 and x.is_cuda and p.weight.dtype == torch.float32)
 
+    def can_fuse_block_training(self, x):
+        """The differentiable matrix-core form: 64 x 64 blocks, 8-bit codes, D <= 1024, fp32."""
+        p = self.projection
+        return (isinstance(p, BH4) and p.block_size == 64 and self.code_length == 8
+                and 64 <= p.padded_in_dim <= 1024 and p.in_dim % 4 == 0
+                and x.dtype == torch.float32 and x.is_cuda and p.weight.dtype == torch.float32)
+
     def forward(self, x):
         B, D = x.shape
-        if self.can_fuse(x):
+        if self.can_fuse(x):                      # no gradient needed: the inference kernels
             return self.forward_fused(x)
+        if self.can_fuse_block(x):
+            return self.forward_block(x)
         if self.can_fuse_training(x):
             p = self.projection
             return ProjectHash.apply(x, p.weight, p.bias, self.num_table, p.decay_coeff)
-        if self.can_fuse_block(x):
-            return self.forward_block(x)
+        if self.can_fuse_block_training(x):
+            p = self.projection
+            return BlockProjectHash.apply(x, p.weight, p.bias, self.num_table, p.decay_coeff)
         z = self.projection(x)
         z = z.reshape(B, self.num_table, self.code_length)
         code, score = compute_code_score(z, training=self.training)

@@ -174,6 +174,102 @@ def _(x, ln_weight, ln_bias, ln_eps, w_folded, bias, T, decay, residual):
             torch.empty(x.shape[0], T, dtype=torch.float32, device=x.device))
 
 
+# ----------------------------------------------------------------------------- bh4_block training
+
+_L.define("bh4_fold_mode(Tensor w, int mode) -> Tensor")
+
+
+def _bh4_fold_mode_impl(w: torch.Tensor, mode: int) -> torch.Tensor:
+    """w: [..., 64, 64] blocks.  mode 0 / 1: the forward / backward kernels' fetch order,
+    mode 2: natural order (gradient w.r.t. folded weights -> gradient w.r.t. weights)."""
+    _lib.require_gpu(w)
+    assert w.dim() >= 2 and w.shape[-1] == w.shape[-2] and w.dtype == torch.float32 and w.is_contiguous()
+    bs = w.shape[-1]
+    nblk = w.numel() // (bs * bs)
+    out = torch.empty_like(w)
+    with _dev_guard(w):
+        rc = _lib.load().lffn_bh4_fold_mode_f32(_lib.ptr(w), _lib.ptr(out), nblk, bs, mode, _lib.stream_of(w))
+    _lib.check(rc, f"lffn_bh4_fold_mode_f32(num_blocks={nblk}, block_size={bs}, mode={mode})")
+    return out
+
+
+_L.impl("bh4_fold_mode", _bh4_fold_mode_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::bh4_fold_mode")
+def _(w, mode):
+    return torch.empty_like(w)
+
+
+_L.define("bh4_block_hash_train(Tensor x, Tensor w_folded, Tensor? bias, int T, float decay, float residual)"
+          " -> (Tensor, Tensor, Tensor, Tensor)")
+
+
+def _bh4_block_hash_train_impl(x, w_folded, bias, T, decay, residual):
+    """-> (codes [B,T], scores [B,T], z [B,T*8], stage_inputs [R,J-1,B,D])."""
+    _lib.require_gpu(x, w_folded, bias)
+    assert x.dim() == 2 and w_folded.dim() == 5
+    assert x.dtype == torch.float32 and w_folded.dtype == torch.float32
+    assert x.is_contiguous() and w_folded.is_contiguous()
+    B, H = x.shape
+    R, J, NB, bs, _ = w_folded.shape
+    D = NB * bs
+    assert H <= D and T * 8 <= R * D
+    if bias is not None:
+        assert bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == T * 8
+    codes = torch.empty(B, T, dtype=torch.int32, device=x.device)
+    scores = torch.empty(B, T, dtype=torch.float32, device=x.device)
+    z = torch.empty(B, T * 8, dtype=torch.float32, device=x.device)
+    stage_in = torch.empty(R, max(J - 1, 0), B, D, dtype=torch.float32, device=x.device)
+    with _dev_guard(x):
+        rc = _lib.load().lffn_bh4_block_hash_train_f32(
+            _lib.ptr(x), _lib.ptr(w_folded), _lib.ptr(bias), _lib.ptr(codes), _lib.ptr(scores), _lib.ptr(z),
+            _lib.ptr(stage_in) if J > 1 else None, B, H, D, R, J, T, bs, decay, residual, _lib.stream_of(x))
+    _lib.check(rc, f"lffn_bh4_block_hash_train_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T})")
+    return codes, scores, z, stage_in
+
+
+_L.impl("bh4_block_hash_train", _bh4_block_hash_train_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::bh4_block_hash_train")
+def _(x, w_folded, bias, T, decay, residual):
+    B = x.shape[0]
+    R, J, NB, bs, _ = w_folded.shape
+    return (torch.empty(B, T, dtype=torch.int32, device=x.device), x.new_empty(B, T), x.new_empty(B, T * 8),
+            x.new_empty(R, max(J - 1, 0), B, NB * bs))
+
+
+_L.define("bh4_block_bwd(Tensor g_z, Tensor w_folded_t, int H, float decay, float residual) -> (Tensor, Tensor)")
+
+
+def _bh4_block_bwd_impl(g_z, w_folded_t, H, decay, residual):
+    """-> (g_x [R,B,H], stage_grads [R,J,B,D])."""
+    _lib.require_gpu(g_z, w_folded_t)
+    assert g_z.dim() == 2 and g_z.dtype == torch.float32 and g_z.is_contiguous() and g_z.shape[1] % 8 == 0
+    assert w_folded_t.dim() == 5 and w_folded_t.dtype == torch.float32 and w_folded_t.is_contiguous()
+    B = g_z.shape[0]
+    T = g_z.shape[1] // 8
+    R, J, NB, bs, _ = w_folded_t.shape
+    D = NB * bs
+    g_x = torch.empty(R, B, H, dtype=torch.float32, device=g_z.device)
+    stage_g = torch.empty(R, J, B, D, dtype=torch.float32, device=g_z.device)
+    with _dev_guard(g_z):
+        rc = _lib.load().lffn_bh4_block_bwd_f32(_lib.ptr(g_z), _lib.ptr(w_folded_t), _lib.ptr(g_x), _lib.ptr(stage_g),
+                                                B, H, D, R, J, T, bs, decay, residual, _lib.stream_of(g_z))
+    _lib.check(rc, f"lffn_bh4_block_bwd_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T})")
+    return g_x, stage_g
+
+
+_L.impl("bh4_block_bwd", _bh4_block_bwd_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::bh4_block_bwd")
+def _(g_z, w_folded_t, H, decay, residual):
+    R, J, NB, bs, _ = w_folded_t.shape
+    return g_z.new_empty(R, g_z.shape[0], H), g_z.new_empty(R, J, g_z.shape[0], NB * bs)
+
+
 # ----------------------------------------------------------------------------- mix_code_score
 
 _L.define("mix_code_score(Tensor y, Tensor x, Tensor? bias, int T, int k, int D, float decay, float residual)"
@@ -573,6 +669,9 @@ bh4_diag = torch.ops.lookupffn.bh4_diag
 bh4_fold = torch.ops.lookupffn.bh4_fold
 bh4_block = torch.ops.lookupffn.bh4_block
 mix_code_score = torch.ops.lookupffn.mix_code_score
+bh4_fold_mode = torch.ops.lookupffn.bh4_fold_mode
+bh4_block_hash_train = torch.ops.lookupffn.bh4_block_hash_train
+bh4_block_bwd = torch.ops.lookupffn.bh4_block_bwd
 ln_bh4_block_hash = torch.ops.lookupffn.ln_bh4_block_hash
 project_hash = torch.ops.lookupffn.project_hash
 project_hash_bwd = torch.ops.lookupffn.project_hash_bwd

@@ -128,17 +128,20 @@ def test_operator_gradients_match_oracle():
 
 # (H, T, Do): D = 64 takes the per-operator path; the others the one-kernel differentiable
 # projection + hash (D = 256 with one and with two repeats, D = 512, D = 1024 with zero padding)
-@pytest.mark.parametrize("H,T,Do", [(64, 8, 64), (256, 32, 64), (256, 64, 128), (500, 64, 64), (768, 128, 64)])
-def test_layer_gradients_match_torch_autograd_of_reference_formulas(H, T, Do):
+@pytest.mark.parametrize("H,T,Do,bs", [(64, 8, 64, 1), (256, 32, 64, 1), (256, 64, 128, 1), (500, 64, 64, 1),
+                                        (768, 128, 64, 1), (256, 32, 64, 64), (256, 64, 128, 64), (500, 64, 64, 64),
+                                        (768, 128, 64, 64), (64, 8, 64, 64), (192, 32, 64, 16)])
+def test_layer_gradients_match_torch_autograd_of_reference_formulas(H, T, Do, bs):
     """Training step through the whole layer vs autograd over the reference's own
     slow formulas (index-multiply-sum gather, compute_code_score_torch, matmul
     Hadamard) evaluated in float64 on the same parameters."""
     torch.manual_seed(5 + H + T)
     S = 256
-    layer = lookupffn_amd.LookupFFN(_config(hidden_size=H, ffn_num_table=T), Do).to(DEV).train()
+    layer = lookupffn_amd.LookupFFN(_config(hidden_size=H, ffn_num_table=T, block_size=bs), Do).to(DEV).train()
     with torch.no_grad():
         layer.hash.projection.bias.normal_(0, 0.05)
-    assert layer.hash.can_fuse_training(torch.empty(1, H, device=DEV)) == (H >= 256)
+    assert layer.hash.can_fuse_training(torch.empty(1, H, device=DEV)) == (bs == 1 and H >= 256)
+    assert layer.hash.can_fuse_block_training(torch.empty(1, H, device=DEV)) == (bs == 64)
     x = torch.randn(24, H, device=DEV, requires_grad=True)
     target = torch.randn(24, Do, device=DEV)
     out = layer(x)
@@ -157,7 +160,10 @@ def test_layer_gradients_match_torch_autograd_of_reference_formulas(H, T, Do):
     for i in range(w.shape[0]):
         y = hp
         for j in range(w.shape[1]):
-            y = (y * w[i, j].reshape(1, D)) @ Hm
+            if bs == 1:
+                y = (y * w[i, j].reshape(1, D)) @ Hm
+            else:
+                y = torch.einsum("bni,noi->bno", y.reshape(24, D // bs, bs), w[i, j]).reshape(24, D) @ Hm
         ys.append(y)
     z = 0.7 * torch.cat(ys, -1) + (1 - 0.7) * hp.repeat(1, w.shape[0])
     z = (z[:, :T * 8] + ref["hash.projection.bias"]).reshape(24, T, 8)
