@@ -91,6 +91,46 @@ def ln_bh4_block_hash(x, ln_w, ln_b, eps, w, bias, T, decay=0.7):
     return host(codes), host(scores)
 
 
+def bh4_fold_mode(w, mode):
+    wd = dev(w)
+    out = torch.full_like(wd, float("nan"))
+    _call("lffn_bh4_fold_mode_f32", p(wd), p(out), w.size // (64 * 64), 64, mode)
+    return host(out)
+
+
+def bh4_block_train(x, w, bias, T, decay=0.7):
+    """-> codes, scores, z, stage_inputs [R, J-1, B, D]"""
+    xd, wd, bd = dev(x), dev(w), dev(bias)
+    B, H = x.shape
+    R, J, NB, bs, _ = w.shape
+    D = NB * bs
+    wf = torch.empty_like(wd)
+    _call("lffn_bh4_fold_mode_f32", p(wd), p(wf), R * J * NB, bs, 0)
+    codes = torch.full((B, T), -1, dtype=torch.int32, device=DEV)
+    scores = torch.full((B, T), float("nan"), dtype=torch.float32, device=DEV)
+    z = torch.full((B, T * 8), float("nan"), dtype=torch.float32, device=DEV)
+    st = torch.full((R, max(J - 1, 1), B, D), float("nan"), dtype=torch.float32, device=DEV)
+    _call("lffn_bh4_block_hash_train_f32", p(xd), p(wf), p(bd), p(codes), p(scores), p(z), p(st), B, H, D, R, J, T, bs,
+          float(np.float32(decay)), float(np.float32(1 - decay)))
+    return host(codes), host(scores), host(z), host(st)[:, :J - 1]
+
+
+def bh4_block_bwd(g_z, w, H, decay=0.7):
+    """-> g_x [R, B, H], stage_grads [R, J, B, D]"""
+    gd, wd = dev(g_z), dev(w)
+    B = g_z.shape[0]
+    T = g_z.shape[1] // 8
+    R, J, NB, bs, _ = w.shape
+    D = NB * bs
+    wt = torch.empty_like(wd)
+    _call("lffn_bh4_fold_mode_f32", p(wd), p(wt), R * J * NB, bs, 1)
+    g_x = torch.full((R, B, H), float("nan"), dtype=torch.float32, device=DEV)
+    sg = torch.full((R, J, B, D), float("nan"), dtype=torch.float32, device=DEV)
+    _call("lffn_bh4_block_bwd_f32", p(gd), p(wt), p(g_x), p(sg), B, H, D, R, J, T, bs,
+          float(np.float32(decay)), float(np.float32(1 - decay)))
+    return host(g_x), host(sg)
+
+
 def mix_code_score(y, x, bias, T, k, D, decay=0.7):
     yd, xd, bd = dev(y), dev(x), dev(bias)
     B, ldy = y.shape

@@ -97,6 +97,16 @@ def test_argument_validation_of_the_backward_and_block_entry_points():
     assert lib.lffn_fht_f16(P, P, 4, 2048, None) == U
     assert lib.lffn_fht_bf16(P, P + 2, 4, 64, None) == A                            # 8-byte alignment
     assert lib.lffn_fht_f16(P, P, 0, 64, None) == OK
+    # block-64 training kernels
+    assert lib.lffn_bh4_fold_mode_f32(P, P + 1 << 20, 4, 64, 3, None) == U                 # mode
+    assert lib.lffn_bh4_fold_mode_f32(P, P, 4, 64, 1, None) == A                           # in place
+    assert lib.lffn_bh4_fold_mode_f32(P, P + 4096, 0, 64, 1, None) == OK
+    assert lib.lffn_bh4_block_hash_train_f32(P, P, None, P, P, None, P, 4, 768, 1024, 1, 4, 128, 64,
+                                             0.7, 0.3, None) == A                          # z is required
+    assert lib.lffn_bh4_block_bwd_f32(P, P, P, P, 4, 768, 1024, 1, 4, 200, 64, 0.7, 0.3, None) == A   # T*8 > R*D
+    assert lib.lffn_bh4_block_bwd_f32(P, P, P, P, 0, 768, 1024, 1, 4, 128, 64, 0.7, 0.3, None) == OK
+    assert lib.lffn_project_hash_bwd_f32(P, P, P, P, P, P, P, 4, 64, 64, 1, 4, 8, 1, 0.7, 0.3, None) == U   # D < 256
+    assert lib.lffn_project_hash_bwd_f32(P, P, P, P, P, P, P, 4, 768, 1024, 1, 5, 128, 1, 0.7, 0.3, None) == U  # J > 4
     # gather with residual
     assert lib.lffn_lookup_gather_residual_f32(P, P, P, None, P + 4, P, 4, 2, 16, 64, None) == A
 

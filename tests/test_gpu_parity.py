@@ -264,6 +264,69 @@ def test_ln_bh4_block_hash_matches_oracle(B, H, D, R, T, with_ln):
         assert np.array_equal(codes, c3) and np.array_equal(scores, s3)
 
 
+def test_bh4_fold_modes():
+    import scipy.linalg
+    rng = np.random.RandomState(77)
+    w = rng.randn(3, 2, 64, 64).astype(np.float32)
+    want = np.einsum("po,rnoi->rnpi", scipy.linalg.hadamard(64).astype(np.float64), w.astype(np.float64))
+    f0 = cabi.bh4_fold_mode(w, 0).reshape(3, 2, 4, 4, 4, 16, 4).transpose(0, 1, 2, 5, 4, 3, 6).reshape(3, 2, 64, 64)
+    assert relmax(f0, want) <= 1e-6                        # [o/16][(i%16)/4][i/16][o%16][i%4]
+    f1 = cabi.bh4_fold_mode(w, 1).reshape(3, 2, 4, 4, 4, 16, 4)      # [i/16][(o%16)/4][o/16][i%16][o%4]
+    f1 = f1.transpose(0, 1, 4, 3, 6, 2, 5).reshape(3, 2, 64, 64)     # -> [o/16, (o%16)/4, o%4][i/16, i%16]
+    assert relmax(f1, want) <= 1e-6
+    assert relmax(cabi.bh4_fold_mode(w, 2), want) <= 1e-6
+
+
+@pytest.mark.parametrize("B,H,D,R,T", [(70, 768, 1024, 1, 128), (33, 256, 256, 2, 64), (40, 500, 512, 1, 64),
+                                        (17, 64, 64, 1, 8), (50, 1024, 1024, 4, 512)])
+def test_bh4_block_training_kernels_match_float64(B, H, D, R, T):
+    """Forward with saved stage inputs, and the backward kernel, against the chain written out in
+    float64: u_{s+1} = (W_s u_s) H_D per block; backwards q = G H_D, G <- W_s^T q."""
+    import scipy.linalg
+    rng = np.random.RandomState(B + H + D + R + T)
+    J, NB = 4, D // 64
+    x = rng.randn(B, H).astype(np.float32)
+    w = (rng.randn(R, J, NB, 64, 64) / math.sqrt(64 * D)).astype(np.float32)
+    bias = (0.05 * rng.randn(T * 8)).astype(np.float32)
+    codes, scores, z, stage_in = cabi.bh4_block_train(x, w, bias, T)
+    HD = scipy.linalg.hadamard(D).astype(np.float64)
+    HN = scipy.linalg.hadamard(NB).astype(np.float64) if NB > 1 else np.ones((1, 1))
+    xp = np.concatenate([x.astype(np.float64), np.zeros((B, D - H))], axis=1)
+    w64 = w.astype(np.float64)
+    us = np.zeros((R, J + 1, B, D))
+    for r in range(R):
+        us[r, 0] = xp
+        for j in range(J):
+            v = np.einsum("bni,noi->bno", us[r, j].reshape(B, NB, 64), w64[r, j]).reshape(B, D)
+            us[r, j + 1] = v @ HD
+    z64 = (0.7 * np.concatenate([us[r, J] for r in range(R)], axis=1) + 0.3 * np.tile(xp, (1, R)))[:, :T * 8] + bias
+    scale = np.abs(z64).max()
+    assert np.abs(z - z64).max() <= 1e-5 * scale
+    for r in range(R):
+        for j in range(1, J):
+            assert relmax(stage_in[r, j - 1], us[r, j]) <= 1e-5
+    # the codes and scores of the kernel's own z, exactly
+    code_z, score_z = oracle.code_score(z.reshape(B, T, 8))
+    assert np.array_equal(codes, code_z)
+    np.testing.assert_allclose(scores, score_z, rtol=2e-6)
+    # same codes and scores as the inference form
+    c2, s2 = cabi.ln_bh4_block_hash(x, None, None, 0.0, w, bias, T)
+    assert np.array_equal(codes, c2) and np.array_equal(scores, s2)
+
+    g_z = rng.randn(B, T * 8).astype(np.float32)
+    g_x, stage_g = cabi.bh4_block_bwd(g_z, w, H)
+    gzp = np.concatenate([g_z.astype(np.float64), np.zeros((B, R * D - T * 8))], axis=1)
+    for r in range(R):
+        G = 0.7 * gzp[:, r * D:(r + 1) * D]
+        for j in range(J - 1, -1, -1):
+            P = np.einsum("mn,bno->bmo", HN, G.reshape(B, NB, 64)).reshape(B, D)
+            assert relmax(stage_g[r, j], P) <= 1e-5, (r, j)
+            q = G @ HD
+            G = np.einsum("bno,noi->bni", q.reshape(B, NB, 64), w64[r, j]).reshape(B, D)
+        want_x = G[:, :H] + 0.3 * gzp[:, r * D:r * D + H]
+        assert relmax(g_x[r], want_x) <= 1e-5, r
+
+
 def test_sign_diagonal_fht_exact():
     # the BASELINE "random +-1 sign diagonal from seed": one round, exact on integers
     rng = np.random.RandomState(8)
