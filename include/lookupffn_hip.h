@@ -167,6 +167,20 @@ int lffn_bh4_block_bwd_f32(const float *g_z, const float *w_folded_t, float *g_x
                            int64_t block_size, float decay, float residual, void *stream);
 
 /*
+ * Weight gradient of the BH4 module with 64 x 64 blocks, all stages in one launch, in the
+ * folded basis: for stage s = r * J + j and block n
+ *   g_folded[s][n][o][i] += sum_b stage_grads[s][b][64n + o] * u_s[b][64n + i]
+ * stage_grads: [R*J, B, D] as lffn_bh4_block_bwd_f32 writes it; u_s is x [B, H] (zero from
+ * column H on) for j = 0, else stage_inputs[r][j-1] of lffn_bh4_block_hash_train_f32
+ * ([R, J-1, B, D], may be null when J = 1); g_folded: [R*J, D/64, 64, 64], natural order,
+ * accumulated into with atomics (zero it first for a plain result).
+ * lffn_bh4_fold_mode_f32(mode 2) turns the sum into the gradient of the weights.  Replaces
+ * the einsum "bno,bni->noi" autograd records for PL/bh4/kernel.py:32.
+ */
+int lffn_bh4_block_wgrad_f32(const float *stage_grads, const float *x, const float *stage_inputs, float *g_folded,
+                             int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t block_size, void *stream);
+
+/*
  * The tail of the BH4 module and the hash in one pass, for any block size:
  *   z[b, c] = decay * y[b, c] + residual * pad(x)[b, c % D] + bias[c],  c < T*k
  *   (code, score)[b, t] = code and score of z[b, t*k : (t+1)*k]   (as lffn_code_score_f32)

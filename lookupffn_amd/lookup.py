@@ -96,9 +96,9 @@ class BlockProjectHash(torch.autograd.Function):
     """BH4 with 64 x 64 blocks -> mix -> bias -> 8-bit code + score as one differentiable
     operator.  Forward: one matrix-core kernel that also keeps z and the input of every stage.
     Backward: the score derivative, one matrix-core kernel walking the stages down (grad x and
-    the gradient in front of every block product), then the weight gradient as a batched product
-    over the tokens of those gradients with the saved stage inputs, taken back through the
-    64-point transform.  Same mathematics as bh4_cuda + BH4._forward + compute_code_score under
+    the gradient in front of every block product), then the weight gradient: a matrix-core
+    kernel summing, per block, those gradients against the saved stage inputs over the tokens,
+    taken back through the 64-point transform.  Same mathematics as bh4_cuda + BH4._forward + compute_code_score under
     autograd (PL/bh4/kernel.py:23-36, PL/lookup.py:29-39)."""
 
     @staticmethod
@@ -123,20 +123,8 @@ class BlockProjectHash(torch.autograd.Function):
         g_x, stage_g = ops.bh4_block_bwd(g_z, ops.bh4_fold_mode(w, 1), H, ctx.decay, 1 - ctx.decay)
         g_w = None
         if ctx.needs_input_grad[1]:
-            g_folded = torch.empty_like(w)
-            for r in range(R):
-                for j in range(J):
-                    p = stage_g[r, j].view(B, NB, bs)
-                    if j == 0:        # the input of stage 0 is x, zero beyond its H columns
-                        full, rem = H // bs, H % bs
-                        g_folded[r, j].zero_()
-                        if full:
-                            g_folded[r, j, :full] = torch.einsum(
-                                "bno,bni->noi", p[:, :full], x[:, :full * bs].reshape(B, full, bs))
-                        if rem:
-                            g_folded[r, j, full, :, :rem] = p[:, full].t() @ x[:, full * bs:]
-                    else:
-                        g_folded[r, j] = torch.einsum("bno,bni->noi", p, stage_in[r, j - 1].view(B, NB, bs))
+            # stage 0 reads x (zero beyond its H columns), stage j the saved input of that stage
+            g_folded = ops.bh4_block_wgrad(stage_g.reshape(R * J, B, NB * bs), x, stage_in, R, J).view_as(w)
             g_w = ops.bh4_fold_mode(g_folded, 2)
         g_x = g_x[0] if R == 1 else g_x.sum(0)
         g_bias = g_z.sum(0) if (ctx.has_bias and ctx.needs_input_grad[2]) else None

@@ -270,6 +270,34 @@ def _(g_z, w_folded_t, H, decay, residual):
     return g_z.new_empty(R, g_z.shape[0], H), g_z.new_empty(R, J, g_z.shape[0], NB * bs)
 
 
+_L.define("bh4_block_wgrad(Tensor stage_grads, Tensor x, Tensor stage_inputs, int R, int J) -> Tensor")
+
+
+def _bh4_block_wgrad_impl(stage_grads, x, stage_inputs, R, J):
+    """[R*J, D/64, 64, 64]: per stage and block, the sum over the tokens of (stage gradient)^T (stage input),
+    in the folded basis.  stage_grads [R*J, B, D]; x [B, H]; stage_inputs [R, J-1, B, D]."""
+    _lib.require_gpu(stage_grads, x, stage_inputs)
+    for t in (stage_grads, x, stage_inputs):
+        assert t.dtype == torch.float32 and t.is_contiguous()
+    S, B, D = stage_grads.shape
+    assert S == R * J and x.shape[0] == B and stage_inputs.numel() == R * (J - 1) * B * D
+    g = torch.zeros(S, D // 64, 64, 64, dtype=torch.float32, device=x.device)
+    with _dev_guard(x):
+        rc = _lib.load().lffn_bh4_block_wgrad_f32(_lib.ptr(stage_grads), _lib.ptr(x), _lib.ptr(stage_inputs), _lib.ptr(g), B,
+                                                  x.shape[1], D, R, J, 64, _lib.stream_of(x))
+    _lib.check(rc, f"lffn_bh4_block_wgrad_f32(B={B}, H={x.shape[1]}, D={D}, R={R}, J={J})")
+    return g
+
+
+_L.impl("bh4_block_wgrad", _bh4_block_wgrad_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::bh4_block_wgrad")
+def _(stage_grads, x, stage_inputs, R, J):
+    S, B, D = stage_grads.shape
+    return x.new_empty(S, D // 64, 64, 64)
+
+
 # ----------------------------------------------------------------------------- mix_code_score
 
 _L.define("mix_code_score(Tensor y, Tensor x, Tensor? bias, int T, int k, int D, float decay, float residual)"
@@ -672,6 +700,7 @@ mix_code_score = torch.ops.lookupffn.mix_code_score
 bh4_fold_mode = torch.ops.lookupffn.bh4_fold_mode
 bh4_block_hash_train = torch.ops.lookupffn.bh4_block_hash_train
 bh4_block_bwd = torch.ops.lookupffn.bh4_block_bwd
+bh4_block_wgrad = torch.ops.lookupffn.bh4_block_wgrad
 ln_bh4_block_hash = torch.ops.lookupffn.ln_bh4_block_hash
 project_hash = torch.ops.lookupffn.project_hash
 project_hash_bwd = torch.ops.lookupffn.project_hash_bwd

@@ -131,6 +131,14 @@ def bh4_block_bwd(g_z, w, H, decay=0.7):
     return host(g_x), host(sg)
 
 
+def bh4_block_wgrad(stage_grads, x, stage_inputs, R, J, init=None):
+    sg, xd, si = dev(stage_grads), dev(x), dev(stage_inputs)
+    S, B, D = stage_grads.shape
+    g = torch.zeros(S, D // 64, 64, 64, dtype=torch.float32, device=DEV) if init is None else dev(init)
+    _call("lffn_bh4_block_wgrad_f32", p(sg), p(xd), p(si), p(g), B, x.shape[1], D, R, J, 64)
+    return host(g)
+
+
 def mix_code_score(y, x, bias, T, k, D, decay=0.7):
     yd, xd, bd = dev(y), dev(x), dev(bias)
     B, ldy = y.shape

@@ -105,6 +105,11 @@ def test_argument_validation_of_the_backward_and_block_entry_points():
                                              0.7, 0.3, None) == A                          # z is required
     assert lib.lffn_bh4_block_bwd_f32(P, P, P, P, 4, 768, 1024, 1, 4, 200, 64, 0.7, 0.3, None) == A   # T*8 > R*D
     assert lib.lffn_bh4_block_bwd_f32(P, P, P, P, 0, 768, 1024, 1, 4, 128, 64, 0.7, 0.3, None) == OK
+    assert lib.lffn_bh4_block_wgrad_f32(P, P, P, P, 4, 768, 1024, 1, 4, 32, None) == U       # block size
+    assert lib.lffn_bh4_block_wgrad_f32(P, P, P, P, 4, 770, 1024, 1, 4, 64, None) == U       # H % 4
+    assert lib.lffn_bh4_block_wgrad_f32(P, P, None, P, 4, 768, 1024, 1, 4, 64, None) == A    # stage inputs needed
+    assert lib.lffn_bh4_block_wgrad_f32(P, P, P, P, 4, 1088, 1024, 1, 4, 64, None) == A      # H > D
+    assert lib.lffn_bh4_block_wgrad_f32(P, P, P, P, 0, 768, 1024, 1, 4, 64, None) == OK
     assert lib.lffn_project_hash_bwd_f32(P, P, P, P, P, P, P, 4, 64, 64, 1, 4, 8, 1, 0.7, 0.3, None) == U   # D < 256
     assert lib.lffn_project_hash_bwd_f32(P, P, P, P, P, P, P, 4, 768, 1024, 1, 5, 128, 1, 0.7, 0.3, None) == U  # J > 4
     # gather with residual

@@ -327,6 +327,27 @@ def test_bh4_block_training_kernels_match_float64(B, H, D, R, T):
         assert relmax(g_x[r], want_x) <= 1e-5, r
 
 
+@pytest.mark.parametrize("B,H,D,R,J", [(1000, 1024, 1024, 1, 2), (515, 768, 1024, 2, 2), (70, 100, 256, 1, 3),
+                                       (2050, 512, 512, 1, 1), (3, 64, 64, 2, 1), (0, 64, 64, 1, 2)])
+def test_bh4_block_wgrad_matches_float64(B, H, D, R, J):
+    rng = np.random.RandomState(B + D + H)
+    NB = D // 64
+    sg = rng.randn(R * J, B, D).astype(np.float32)
+    x = rng.randn(B, H).astype(np.float32)
+    si = rng.randn(R, max(J - 1, 1), B, D).astype(np.float32)[:, :J - 1]
+    xp = np.concatenate([x.astype(np.float64), np.zeros((B, D - H))], axis=1)
+    want = np.stack([np.einsum("bno,bni->noi", sg[r * J + j].astype(np.float64).reshape(B, NB, 64),
+                               (xp if j == 0 else si[r, j - 1].astype(np.float64)).reshape(B, NB, 64))
+                     for r in range(R) for j in range(J)])
+    got = cabi.bh4_block_wgrad(sg, x, np.ascontiguousarray(si), R, J)
+    if B == 0:
+        assert not got.any()
+        return
+    assert relmax(got, want) <= 1e-5
+    init = rng.randn(R * J, NB, 64, 64).astype(np.float32)
+    assert relmax(cabi.bh4_block_wgrad(sg, x, np.ascontiguousarray(si), R, J, init=init), want + init) <= 1e-5   # accumulates
+
+
 def test_sign_diagonal_fht_exact():
     # the BASELINE "random +-1 sign diagonal from seed": one round, exact on integers
     rng = np.random.RandomState(8)
