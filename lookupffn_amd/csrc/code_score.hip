@@ -98,24 +98,54 @@ __global__ __launch_bounds__(256) void mix_code_score_kernel(const float *__rest
     scores[n] = num / den;
 }
 
+// K > 0: k == K, z and g_z 16-byte aligned with K % 4 == 0: one hash per lane, its K values in
+// registers (one exponential per value).  K == 0: any k, scalar loads.
+template <int K>
 __global__ __launch_bounds__(256) void code_score_bwd_kernel(const float *__restrict__ z, const float *__restrict__ g_score,
                                                              float *__restrict__ g_z, int64_t N, int k) {
     const int64_t n = int64_t(blockIdx.x) * 256 + threadIdx.x;
     if (n >= N) return;
-    const float *p = z + n * k;
-    float S = 0.f, P = 1.f;
-    for (int d = 0; d < k; ++d) {
-        const float a = fabsf(p[d]);
-        S = S + a;
-        P = P * (1.0f + expf(-2.0f * a));
-    }
-    const float g = g_score[n];
-    for (int d = 0; d < k; ++d) {
-        const float v = p[d];
-        const float a = fabsf(v);
-        const float e = expf(-2.0f * a);
-        const float sg = v > 0.f ? 1.f : (v < 0.f ? -1.f : 0.f);
-        g_z[n * k + d] = g * sg * (1.0f + S * 2.0f * e / (1.0f + e)) / P;
+    if constexpr (K > 0) {
+        float v[K], e[K];
+#pragma unroll
+        for (int q = 0; q < K / 4; ++q) {
+            const float4 t = reinterpret_cast<const float4 *>(z + n * K)[q];
+            v[4 * q] = t.x, v[4 * q + 1] = t.y, v[4 * q + 2] = t.z, v[4 * q + 3] = t.w;
+        }
+        float S = 0.f, P = 1.f;
+#pragma unroll
+        for (int d = 0; d < K; ++d) {
+            const float a = fabsf(v[d]);
+            e[d] = expf(-2.0f * a);
+            S = S + a;
+            P = P * (1.0f + e[d]);
+        }
+        const float gp = g_score[n] / P;
+        float o[K];
+#pragma unroll
+        for (int d = 0; d < K; ++d) {
+            const float sg = v[d] > 0.f ? gp : (v[d] < 0.f ? -gp : 0.f);
+            o[d] = sg * (1.0f + S * 2.0f * e[d] / (1.0f + e[d]));
+        }
+#pragma unroll
+        for (int q = 0; q < K / 4; ++q)
+            reinterpret_cast<float4 *>(g_z + n * K)[q] = make_float4(o[4 * q], o[4 * q + 1], o[4 * q + 2], o[4 * q + 3]);
+    } else {
+        const float *p = z + n * k;
+        float S = 0.f, P = 1.f;
+        for (int d = 0; d < k; ++d) {
+            const float a = fabsf(p[d]);
+            S = S + a;
+            P = P * (1.0f + expf(-2.0f * a));
+        }
+        const float g = g_score[n];
+        for (int d = 0; d < k; ++d) {
+            const float v = p[d];
+            const float a = fabsf(v);
+            const float e = expf(-2.0f * a);
+            const float sg = v > 0.f ? 1.f : (v < 0.f ? -1.f : 0.f);
+            g_z[n * k + d] = g * sg * (1.0f + S * 2.0f * e / (1.0f + e)) / P;
+        }
     }
 }
 
@@ -176,7 +206,17 @@ extern "C" int lffn_code_score_bwd_f32(const float *z, const float *g_score, flo
     if (N == 0) return LFFN_OK;
     const int64_t blocks = (N + 255) / 256;
     LFFN_REQUIRE(blocks <= 0x7fffffff, LFFN_ERR_UNSUPPORTED);
-    hipLaunchKernelGGL(code_score_bwd_kernel, dim3((unsigned)blocks), dim3(256), 0,
-                       static_cast<hipStream_t>(stream), z, g_score, g_z, N, (int)k);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool vec = lffn_aligned16(z) && lffn_aligned16(g_z);
+    if (vec && k == 8)
+        hipLaunchKernelGGL((code_score_bwd_kernel<8>), dim3((unsigned)blocks), dim3(256), 0, s, z, g_score, g_z, N, 8);
+    else if (vec && k == 4)
+        hipLaunchKernelGGL((code_score_bwd_kernel<4>), dim3((unsigned)blocks), dim3(256), 0, s, z, g_score, g_z, N, 4);
+    else if (vec && k == 12)
+        hipLaunchKernelGGL((code_score_bwd_kernel<12>), dim3((unsigned)blocks), dim3(256), 0, s, z, g_score, g_z, N, 12);
+    else if (vec && k == 16)
+        hipLaunchKernelGGL((code_score_bwd_kernel<16>), dim3((unsigned)blocks), dim3(256), 0, s, z, g_score, g_z, N, 16);
+    else
+        hipLaunchKernelGGL((code_score_bwd_kernel<0>), dim3((unsigned)blocks), dim3(256), 0, s, z, g_score, g_z, N, (int)k);
     return lffn_launch_status();
 }

@@ -458,7 +458,7 @@ def test_code_score_matches_oracle(k):
 
 def test_code_score_bwd_matches_oracle():
     rng = np.random.RandomState(12)
-    for k in (3, 8):
+    for k in (3, 4, 8, 12, 16):                       # 4, 8, 12, 16 take the vector kernel
         z = rng.randn(300, 9, k).astype(np.float32)
         z[0, 0, 0] = 0.0
         g = rng.randn(300, 9).astype(np.float32)
