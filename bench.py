@@ -19,6 +19,7 @@ One GPU only: this path has no multi-GPU form in this build.
 from __future__ import annotations
 
 import argparse
+import statistics
 import json
 import math
 import os
@@ -59,8 +60,8 @@ WORKLOADS = {
 # HBM bytes per launch of the gather kernel measured with rocprofv3 --pmc
 # (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); the summaries
 # are kept under profiles/.  None until measured for that workload.
-MEASURED_TRAFFIC_BYTES = {"cfg2": 477559591, "cfg2b64": 477451647, "cfg3": 3156050546, "cfg3bf16": 2252934839,
-                          "cfg5": 503520831}
+MEASURED_TRAFFIC_BYTES = {"cfg2": 478224292, "cfg2b64": 478392534, "cfg3": 3166744484, "cfg3bf16": 2259132035,
+                          "cfg5": 503558258}
 
 
 def build_layer(wl, device):
@@ -450,6 +451,27 @@ def main():
     with torch.no_grad():
         hash_ms = timed(hash_front)
 
+    # Warm and cold medians of single launches (outside the timed region).  Warm: back to
+    # back, the tables still in the caches from the launch before.  Cold: a 1 GiB fill
+    # between the launches pushes the tables out of the L2s and the 256 MB Infinity Cache.
+    def single(fn, reps, flush=None):
+        ts = []
+        for _ in range(reps):
+            if flush is not None:
+                flush.add_(1.0)
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(); fn(); b.record()
+            torch.cuda.synchronize()
+            ts.append(a.elapsed_time(b))
+        return statistics.median(ts)
+    with torch.no_grad():
+        code, score = hash_front()
+        gather_only = lambda: ops.lookup_gather(code, score, layer.tables, layer.bias)
+        warm_gather, warm_step = single(gather_only, 25), single(step, 25)
+        flush = torch.zeros(1 << 28, dtype=torch.float32, device=dev)
+        cold_gather, cold_step = single(gather_only, 15, flush), single(step, 15, flush)
+        del flush
+
     res = {
         "metric": "LookupFFN fwd tokens/s + gather-add GB/s as % of HBM peak, RoBERTa-base",
         "value": B * args.steps / sec,
@@ -476,6 +498,9 @@ def main():
         "stages_ms": {("layernorm_bh4block_hash" if block else "layernorm_project_hash"): hash_ms,
                       "gather_add": gather_ms},
         "gather_tokens_per_s": B / (gather_ms * 1e-3),
+        "single_launch_median_ms": {"gather_warm": warm_gather, "gather_cold": cold_gather,
+                                    "step_warm": warm_step, "step_cold": cold_step,
+                                    "cold": "1 GiB fill between launches (tables evicted from L2 and Infinity Cache)"},
         "launch": "HIP graph replay" if args.graph else "eager",
     }
     if not args.no_cpu_baseline:
