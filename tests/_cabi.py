@@ -261,6 +261,28 @@ def lookup_scatter(code, score, g, S, accumulate=False, init=None):
     return host(out)
 
 
+def lookup_scatter_workspace_bytes(B, T, S, Do):
+    n = ctypes.c_int64(-1)
+    rc = _lib.load().lffn_lookup_scatter_workspace_bytes(B, T, S, Do, ctypes.byref(n))
+    assert rc == 0
+    return n.value
+
+
+def lookup_scatter_sorted(code, score, g, S, accumulate=False, init=None):
+    cd, sd, gd = dev(code), dev(score), dev(g)
+    B, T = code.shape
+    Do = g.shape[1]
+    nbytes = lookup_scatter_workspace_bytes(B, T, S, Do)
+    assert nbytes > 0
+    ws = torch.full((nbytes // 4,), 0x7f7f7f7f, dtype=torch.int32, device=DEV)      # scratch: any contents
+    if init is None:
+        out = torch.full((T, S, Do), float("nan"), dtype=torch.float32, device=DEV)   # must be fully overwritten
+    else:
+        out = dev(init)
+    _call("lffn_lookup_scatter_sorted_f32", p(cd), p(sd), p(gd), p(out), p(ws), nbytes, B, T, S, Do, 1 if accumulate else 0)
+    return host(out)
+
+
 def lookup_inner(code, g, tables):
     cd, gd, td = dev(code), dev(g), dev(tables)
     B, T = code.shape

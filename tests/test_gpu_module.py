@@ -184,6 +184,30 @@ def test_layer_gradients_match_torch_autograd_of_reference_formulas(H, T, Do, bs
     assert relmax(npf(x.grad), xr.grad.numpy()) <= 2e-4
 
 
+@pytest.mark.gpu
+def test_table_gradient_of_a_large_batch_takes_the_sorted_scatter():
+    # 16384 tokens x 32 tables x 768 columns is above ops.SORTED_SCATTER_MIN_WORK: the backward of
+    # the layer's gather sorts the tokens by code; checked against index_add_ in float64 and for reproducibility
+    from lookupffn_amd import ops
+    B, T, S, Do = 16384, 32, 256, 768
+    assert B * T * Do >= ops.SORTED_SCATTER_MIN_WORK
+    gen = torch.Generator().manual_seed(5)
+    code = torch.randint(0, S, (B, T), generator=gen, dtype=torch.int32).cuda()
+    score = torch.rand(B, T, generator=gen).cuda()
+    tables = (0.02 * torch.randn(T, S, Do, generator=gen)).cuda().requires_grad_(True)
+    go = torch.randn(B, Do, generator=gen).cuda()
+    out = lookupffn_amd.lookup_gather(code, score, tables)
+    out.backward(go)
+    flat = (code.long() + torch.arange(T, device="cuda") * S).reshape(-1)
+    contrib = (score.double().reshape(-1, 1) * go.double().repeat_interleave(T, dim=0))
+    want = torch.zeros(T * S, Do, dtype=torch.float64, device="cuda").index_add_(0, flat, contrib).reshape(T, S, Do)
+    assert relmax(npf(tables.grad), npf(want)) <= 1e-5
+    first = tables.grad.clone()
+    tables.grad = None
+    lookupffn_amd.lookup_gather(code, score, tables).backward(go)
+    assert torch.equal(first, tables.grad)
+
+
 def test_bf16_tables_inference():
     torch.manual_seed(6)
     layer = lookupffn_amd.LookupFFN(_config(), 128).eval().to(DEV)

@@ -717,6 +717,55 @@ def test_lookup_scatter_matches_oracle(B, T, S, Do):
         assert relmax(cabi.lookup_scatter(dirty, w, g, S), want) <= 1e-5
 
 
+# the sorted form: ragged token counts around the 8-entry steps, the 64-entry batches and the
+# per-wavefront pieces, one code only (S = 1: every piece cuts the same bucket), few tokens in
+# many codes (most buckets empty), 32-column slices beyond and below the eight XCDs
+SORTED_CASES = [(256, 32, 256, 256), (1, 2, 4, 64), (63, 3, 16, 128), (65, 5, 256, 192), (1025, 7, 8, 64),
+                (2100, 6, 256, 128), (300, 1, 2, 64), (500, 4, 512, 96), (4099, 3, 1, 32), (7, 2, 512, 32),
+                (5000, 9, 64, 352), (16384 + 16384 + 100, 2, 16, 32)]      # the last: three chunks of tokens
+
+
+@pytest.mark.parametrize("B,T,S,Do", SORTED_CASES)
+def test_lookup_scatter_sorted_matches_oracle(B, T, S, Do):
+    rng = np.random.RandomState(B + T + S + Do)
+    tables, code, idx, w = _rand_gather(rng, B, T, S, Do)
+    g = rng.randn(B, Do).astype(np.float32)
+    want = oracle.scatter_add(idx, g.astype(np.float64), w.astype(np.float64), T * S).reshape(T, S, Do)
+    got = cabi.lookup_scatter_sorted(code, w, g, S)
+    assert not np.isnan(got).any()                      # every row written, touched or not
+    assert relmax(got, want) <= 1e-5
+    assert np.array_equal(got, cabi.lookup_scatter_sorted(code, w, g, S))        # fixed order of additions
+    init = rng.randn(T, S, Do).astype(np.float32)
+    assert relmax(cabi.lookup_scatter_sorted(code, w, g, S, accumulate=True, init=init), want + init) <= 1e-5
+    dirty = (code + S * rng.randint(0, 4, size=code.shape)).astype(np.int32)      # codes are masked into their table
+    assert np.array_equal(cabi.lookup_scatter_sorted(dirty, w, g, S), got)
+
+
+def test_lookup_scatter_sorted_workspace_query():
+    assert cabi.lookup_scatter_workspace_bytes(16384, 128, 256, 768) >= 16384 * 128 * 8
+    assert cabi.lookup_scatter_workspace_bytes(1 << 20, 128, 256, 768) == cabi.lookup_scatter_workspace_bytes(16384, 128, 256, 768)
+    for shape in ((0, 4, 16, 64), (16, 0, 16, 64), (16, 4, 1024, 64), (16, 4, 16, 48)):
+        assert cabi.lookup_scatter_workspace_bytes(*shape) == 0
+
+
+def test_lookup_scatter_sorted_full_size_zipf():
+    # BASELINE config 5: config-2 shape, codes Zipf(1.1) over 256 entries (the hottest code takes ~18 % of the tokens)
+    rng = np.random.RandomState(41)
+    B, T, S, Do = 16384, 128, 256, 768
+    p = 1.0 / np.arange(1, S + 1) ** 1.1
+    p /= p.sum()
+    code = rng.choice(S, size=(B, T), p=p).astype(np.int32)
+    w = (1.0 - rng.rand(B, T)).astype(np.float32)
+    g = rng.randn(B, Do).astype(np.float32)
+    got = cabi.lookup_scatter_sorted(code, w, g, S)
+    want_sum = w.astype(np.float64).T @ g.astype(np.float64)
+    assert relmax(got.astype(np.float64).sum(1), want_sum) <= 1e-5
+    for t in (0, 77, 127):
+        want_t = oracle.scatter_add(code[:, t:t + 1], g.astype(np.float64), w[:, t:t + 1].astype(np.float64), S)
+        assert relmax(got[t], want_t) <= 1e-5
+    assert relmax(got, cabi.lookup_scatter(code, w, g, S)) <= 1e-5                # the LDS form
+
+
 def test_lookup_scatter_full_size_zipf_properties():
     # BASELINE config 5: config-2 shape, codes Zipf(1.1) over 256 entries
     rng = np.random.RandomState(41)
