@@ -61,7 +61,7 @@ WORKLOADS = {
 # (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); the summaries
 # are kept under profiles/.  None until measured for that workload.
 MEASURED_TRAFFIC_BYTES = {"cfg2": 478224292, "cfg2b64": 478392534, "cfg3": 3166744484, "cfg3bf16": 2259132035,
-                          "cfg5": 503558258}
+                          "cfg5": 949215733}
 
 
 def build_layer(wl, device):
@@ -233,7 +233,7 @@ def main_backward(args):
         "config": {"workload": wl["desc"], "tokens": B, "tables": T, "table_size": S, "d_out": Do,
                    "step": "inner product (grad score) + scatter-add (grad tables) + one kernel: score "
                            "derivative, transposed BH4(block 1)x4, grad of diagonals and bias"},
-        "roofline": {"bound": "hbm", "kernel": "lookup_scatter", "achieved": achieved,
+        "roofline": {"bound": "hbm", "kernel": "lookup_scatter (three launches: transpose/pack, sort, sorted accumulate)", "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get("cfg5"),
                      "algorithmic_bytes": scatter_bytes, "avg_kernel_ms": scatter_ms},
