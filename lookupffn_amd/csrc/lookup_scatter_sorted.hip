@@ -236,15 +236,26 @@ struct SortedArgs {
 
 __device__ __forceinline__ float4 add4(float4 a, float4 b) { return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); }
 
+// v + (v of the lane 16 / 32 positions away): gfx950's row and half-wave swaps, no LDS traffic
+__device__ __forceinline__ float add_xor16(float v) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float add_xor32(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+// v + (v of lane ^ 8): a DPP rotation by eight inside the 16-lane row
+__device__ __forceinline__ float add_xor8(float v) {
+    return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xF, 0xF, true));
+}
+
 // sum over the eight lane groups; afterwards every lane holds the total of its column group
 __device__ __forceinline__ float4 sum_groups(float4 v) {
-#pragma unroll
-    for (int d = 8; d < 64; d <<= 1) {
-        v.x += __shfl_xor(v.x, d);
-        v.y += __shfl_xor(v.y, d);
-        v.z += __shfl_xor(v.z, d);
-        v.w += __shfl_xor(v.w, d);
-    }
+    v.x = add_xor32(add_xor16(add_xor8(v.x)));
+    v.y = add_xor32(add_xor16(add_xor8(v.y)));
+    v.z = add_xor32(add_xor16(add_xor8(v.z)));
+    v.w = add_xor32(add_xor16(add_xor8(v.w)));
     return v;
 }
 
