@@ -352,6 +352,9 @@ def main():
     ap.add_argument("--graph", action="store_true",
                     help="forward workloads: capture the step in a HIP graph and time replays (the launch-bound "
                          "small configurations); the gather's own duration is then measured in an eager loop")
+    ap.add_argument("--two-kernels", action="store_true",
+                    help="small forward workloads: keep the projection+hash kernel and the gather kernel apart "
+                         "instead of the one-launch form of the layer (for comparison)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device-to-device copy, so that a rocprofv3 --pmc run of "
                          "this command holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -386,10 +389,22 @@ def main():
             return layer.hash.forward_block(x, layer_norm=layer.LayerNorm)
         return layer.hash.forward_fused(x, layer_norm=layer.LayerNorm)
 
+    if args.two_kernels:
+        type(layer).FUSED_LAYER_MAX_TOKENS = 0
+    with torch.no_grad():
+        fused_layer = layer.can_fuse_layer(x)      # few tokens: the layer is one launch, gather included
+
     def step(events=None):
         # exactly what LookupFFN.forward runs in eval mode (checked below), with an
         # event pair around the gather launch
         with torch.no_grad():
+            if fused_layer:
+                if events is not None:
+                    events[0].record()
+                out = layer._forward(x)
+                if events is not None:
+                    events[1].record()
+                return out
             code, score = hash_front()
             if events is not None:
                 events[0].record()
@@ -449,7 +464,7 @@ def main():
         b.record(); torch.cuda.synchronize()
         return a.elapsed_time(b) / n
     with torch.no_grad():
-        hash_ms = timed(hash_front)
+        hash_ms = None if fused_layer else timed(hash_front)
 
     # Warm and cold medians of single launches (outside the timed region).  Warm: back to
     # back, the tables still in the caches from the launch before.  Cold: a 1 GiB fill
@@ -465,8 +480,11 @@ def main():
             ts.append(a.elapsed_time(b))
         return statistics.median(ts)
     with torch.no_grad():
-        code, score = hash_front()
-        gather_only = lambda: ops.lookup_gather(code, score, layer.tables, layer.bias)
+        if fused_layer:
+            gather_only = step
+        else:
+            code, score = hash_front()
+            gather_only = lambda: ops.lookup_gather(code, score, layer.tables, layer.bias)
         warm_gather, warm_step = single(gather_only, 25), single(step, 25)
         flush = torch.zeros(1 << 28, dtype=torch.float32, device=dev)
         cold_gather, cold_step = single(gather_only, 15, flush), single(step, 15, flush)
@@ -490,13 +508,16 @@ def main():
                    "tables": T, "table_size": S, "d_out": Do,
                    "step": ("one kernel: LayerNorm + BH4(block 64)x4 on fp32 MFMA + mix + hash (weights folded once, "
                             "outside the step); one kernel: gather-add + bias") if block else
-                           "one kernel: LayerNorm + BH4(block 1)x4 + mix + hash; one kernel: gather-add + bias"},
-        "roofline": {"bound": "hbm", "kernel": "lookup_gather", "achieved": achieved, "peak": HBM_PEAK_GBS,
+                           ("one kernel: LayerNorm + BH4(block 1)x4 + mix + hash + gather-add + bias" if fused_layer else
+                            "one kernel: LayerNorm + BH4(block 1)x4 + mix + hash; one kernel: gather-add + bias")},
+        "roofline": {"bound": "hbm", "kernel": "lookup_ffn_fused (the whole layer)" if fused_layer else "lookup_gather",
+                     "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
                      "algorithmic_bytes": gather_bytes, "avg_kernel_ms": gather_ms},
-        "stages_ms": {("layernorm_bh4block_hash" if block else "layernorm_project_hash"): hash_ms,
-                      "gather_add": gather_ms},
+        "stages_ms": ({"whole_layer": gather_ms} if fused_layer else
+                      {("layernorm_bh4block_hash" if block else "layernorm_project_hash"): hash_ms,
+                       "gather_add": gather_ms}),
         "gather_tokens_per_s": B / (gather_ms * 1e-3),
         "single_launch_median_ms": {"gather_warm": warm_gather, "gather_cold": cold_gather,
                                     "step_warm": warm_step, "step_cold": cold_step,

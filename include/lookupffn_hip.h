@@ -167,6 +167,27 @@ int lffn_bh4_block_bwd_f32(const float *g_z, const float *w_folded_t, float *g_x
                            int64_t block_size, float decay, float residual, void *stream);
 
 /*
+ * The whole layer in one launch, for small batches without gradient (PL/lookup.py:99-108):
+ *   out[b, :] = sum_t score[b,t] * tables[t, code[b,t], :] + out_bias (+ residual_in[b, :])
+ * with (code, score) the 8-bit hash of 0.7 * BH4(LayerNorm(x)) + 0.3 * tile(LayerNorm(x)) +
+ * proj_bias as lffn_ln_project_hash_f32 computes it (same kernel body: the codes and scores
+ * are bit-identical), kept in LDS instead of written out.  One wavefront per token; each
+ * token reads its own T rows from memory, so from a few hundred tokens on the two-kernel
+ * form (lffn_ln_project_hash_f32 + lffn_lookup_gather_f32), which shares table slices
+ * through LDS, is the faster one.
+ * ln_weight/ln_bias: [H], both null for no LayerNorm; diag: [R, J, D]; proj_bias: [T*8] or
+ * null; tables: [T, S, Do] with S >= 256; out_bias: [Do] or null; residual_in: [B, Do] or
+ * null; out: [B, Do].  D in {256, 512, 1024}, T <= 512, Do % 4 == 0.
+ * Replaces, in one call, LookupFFN.forward's LayerNorm, hash and gather (PL/lookup.py:99-108,
+ * 120-130) for the diagonal BH4 projection (PL/lookup.py:29-39 with block_size 1).
+ */
+int lffn_lookup_ffn_fused_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
+                              const float *diag, const float *proj_bias, const float *tables,
+                              const float *out_bias, const float *residual_in, float *out, int64_t B, int64_t H,
+                              int64_t D, int64_t R, int64_t J, int64_t T, int64_t S, int64_t Do, float decay,
+                              float residual, void *stream);
+
+/*
  * Weight gradient of the BH4 module with 64 x 64 blocks, all stages in one launch, in the
  * folded basis: for stage s = r * J + j and block n
  *   g_folded[s][n][o][i] += sum_b stage_grads[s][b][64n + o] * u_s[b][64n + i]

@@ -110,7 +110,15 @@ struct ProjectArgs {
     float decay, residual;
     int mix;              // 1: out = decay*y + residual*x (+ bias); 0: out = y
     int vec_in;           // x rows are 16-byte aligned and H % 4 == 0
+    // GATHER only: the table rows the codes select are added up in the same kernel
+    const float *tables;  // [T, S, Do]
+    const float *obias;   // [Do] or null
+    const float *gres;    // [B, Do] or null: added to the result
+    float *gout;          // [B, Do]
+    int S, Do;
 };
+
+constexpr int FUSED_MAX_T = 512;   // (code, score) pairs a wavefront keeps in LDS for its token
 
 // Part of the score recurrence over the four values of one float4:
 // s <- s + a_c, p <- p * f_c with a_c = |z_c| and f_c = 1 + exp(-2|z_c|), c ascending.
@@ -122,14 +130,16 @@ __device__ __forceinline__ void score_chain(const float (&a)[4], const float (&f
     }
 }
 
-template <int LOGD, bool HASH>
+template <int LOGD, bool HASH, bool GATHER = false>
 __global__ __launch_bounds__(256) void project_kernel(ProjectArgs a) {
     using C = FhtCfg<LOGD>;
     constexpr int D = C::D, NJ = C::NJ, LPR = C::LPR, RPW = C::RPW;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int lr = lane % LPR;
-    const int64_t row = (int64_t(blockIdx.x) * 4 + wave) * RPW + lane / LPR;
+    // GATHER: one token per workgroup; its four wavefronts each compute the token's codes (no
+    // hand-over needed) and then share the gather, a quarter of the tables each
+    const int64_t row = GATHER ? int64_t(blockIdx.x) : (int64_t(blockIdx.x) * 4 + wave) * RPW + lane / LPR;
     const bool live = row < a.B;
 
     float orig[NJ][4];
@@ -245,7 +255,68 @@ __global__ __launch_bounds__(256) void project_kernel(ProjectArgs a) {
                 const int nib_hi = __float_as_int(lane_xor<1>(__int_as_float(nib)));
                 score_chain(az, fz, s_run, p_run);                 // an odd lane continues from there
                 const int t = col >> 3;
-                if (live && (lr & 1) && t < a.T) {
+                if constexpr (GATHER) {
+                    __shared__ uint2 pairs[4][FUSED_MAX_T];
+                    static_assert(RPW == 1, "one token per wavefront");
+                    if ((lr & 1) && t < a.T)
+                        pairs[wave][t] = make_uint2((unsigned)((nib_hi << 4) | nib), __float_as_uint(s_run / p_run));
+                    if (r == a.R - 1 && j == NJ - 1) {
+                        // Small batches: the gather-add of the token's T rows follows in the same
+                        // workgroup (PL/lookup.py:120-130, 108): wavefront w takes tables
+                        // [w*T/4, (w+1)*T/4), 256 columns per pass, eight row loads in flight; the
+                        // four partial sums meet in LDS.  No codes or scores go to memory and
+                        // nothing else is launched.
+                        __shared__ float4 part[4][64];
+                        __syncthreads();                         // the odd lanes' pairs are visible to the whole wavefront
+                        const uint2 *mine = pairs[wave];         // this wavefront's own copy
+                        const int tq = (a.T + 3) / 4;
+                        const int t_lo = min(wave * tq, a.T), t_hi = min(t_lo + tq, a.T);
+                        for (int c0 = 0; c0 < a.Do; c0 += 256) {
+                            const int gc = c0 + 4 * lane;
+                            const bool on = gc < a.Do;
+                            float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+                            for (int t0 = t_lo; t0 < t_hi; t0 += 8) {
+                                float4 rv[8];
+                                float sv[8];
+#pragma unroll
+                                for (int u = 0; u < 8; ++u) {
+                                    const int tt = min(t0 + u, t_hi - 1);
+                                    const uint2 pr = mine[tt];
+                                    sv[u] = t0 + u < t_hi ? __uint_as_float(pr.y) : 0.f;
+                                    const float *rowp = a.tables + ((size_t)tt * a.S + pr.x) * a.Do;
+                                    rv[u] = on ? *reinterpret_cast<const float4 *>(rowp + gc) : make_float4(0.f, 0.f, 0.f, 0.f);
+                                }
+#pragma unroll
+                                for (int u = 0; u < 8; ++u) {
+                                    acc.x = fmaf(sv[u], rv[u].x, acc.x);
+                                    acc.y = fmaf(sv[u], rv[u].y, acc.y);
+                                    acc.z = fmaf(sv[u], rv[u].z, acc.z);
+                                    acc.w = fmaf(sv[u], rv[u].w, acc.w);
+                                }
+                            }
+                            part[wave][lane] = acc;
+                            __syncthreads();
+                            if (wave == 0 && on) {
+                                float4 o = part[0][lane];
+#pragma unroll
+                                for (int w = 1; w < 4; ++w) {
+                                    const float4 q = part[w][lane];
+                                    o.x += q.x; o.y += q.y; o.z += q.z; o.w += q.w;
+                                }
+                                if (a.obias) {
+                                    const float4 bb = *reinterpret_cast<const float4 *>(a.obias + gc);
+                                    o.x += bb.x; o.y += bb.y; o.z += bb.z; o.w += bb.w;
+                                }
+                                if (a.gres) {
+                                    const float4 rr = *reinterpret_cast<const float4 *>(a.gres + row * a.Do + gc);
+                                    o.x += rr.x; o.y += rr.y; o.z += rr.z; o.w += rr.w;
+                                }
+                                *reinterpret_cast<float4 *>(a.gout + row * a.Do + gc) = o;
+                            }
+                            __syncthreads();
+                        }
+                    }
+                } else if (live && (lr & 1) && t < a.T) {
                     a.codes[row * a.T + t] = (nib_hi << 4) | nib;
                     a.scores[row * a.T + t] = s_run / p_run;
                 }
@@ -616,6 +687,40 @@ static int project_hash_impl(const float *x, const float *ln_w, const float *ln_
     a.decay = decay; a.residual = residual; a.mix = 1;
     a.vec_in = (lffn_aligned16(x) && H % 4 == 0) ? 1 : 0;
     return launch_project<true>(a, lffn_log2(D), static_cast<hipStream_t>(stream));
+}
+
+extern "C" int lffn_lookup_ffn_fused_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
+                                         const float *diag, const float *proj_bias, const float *tables,
+                                         const float *out_bias, const float *residual_in, float *out, int64_t B,
+                                         int64_t H, int64_t D, int64_t R, int64_t J, int64_t T, int64_t S,
+                                         int64_t Do, float decay, float residual, void *stream) {
+    LFFN_REQUIRE(x && diag && tables && out, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE((ln_weight != nullptr) == (ln_bias != nullptr) && ln_eps >= 0.f, LFFN_ERR_BAD_ARG);
+    int rc = check_dims(B, H, D, R, J);
+    if (rc != LFFN_OK) return rc;
+    LFFN_REQUIRE(D >= 256 && T <= FUSED_MAX_T && S >= 256 && S * T <= 0x7fffffff, LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(Do >= 4 && Do % 4 == 0 && Do <= (1 << 20), LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(T >= 1 && T * 8 <= R * D, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_aligned16(diag) && (!proj_bias || lffn_aligned16(proj_bias)) && lffn_aligned16(tables) &&
+                     (!out_bias || lffn_aligned16(out_bias)) && (!residual_in || lffn_aligned16(residual_in)) &&
+                     lffn_aligned16(out),
+                 LFFN_ERR_BAD_ARG);
+    if (B == 0) return LFFN_OK;
+    ProjectArgs a{};
+    a.x = x; a.diag = diag; a.pbias = proj_bias; a.ln_w = ln_weight; a.ln_b = ln_bias; a.ln_eps = ln_eps;
+    a.B = B; a.H = (int)H; a.R = (int)R; a.J = (int)J;
+    a.out_stride = (int)(T * 8); a.out_cols = (int)(T * 8); a.T = (int)T;
+    a.decay = decay; a.residual = residual; a.mix = 1;
+    a.vec_in = (lffn_aligned16(x) && H % 4 == 0) ? 1 : 0;
+    a.tables = tables; a.obias = out_bias; a.gres = residual_in; a.gout = out; a.S = (int)S; a.Do = (int)Do;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const dim3 grid((unsigned)B);                       // one token per workgroup
+    switch (lffn_log2(D)) {
+        case 8: hipLaunchKernelGGL((project_kernel<8, true, true>), grid, dim3(256), 0, st, a); break;
+        case 9: hipLaunchKernelGGL((project_kernel<9, true, true>), grid, dim3(256), 0, st, a); break;
+        default: hipLaunchKernelGGL((project_kernel<10, true, true>), grid, dim3(256), 0, st, a); break;
+    }
+    return lffn_launch_status();
 }
 
 extern "C" int lffn_fht_f16(const uint16_t *in, uint16_t *out, int64_t B, int64_t D, void *stream) {

@@ -262,11 +262,31 @@ class LookupFFN(nn.Module):
         return (f"hidden_size={self.hidden_size}, num_table={self.num_table}, "
                 f"table_size={self.table_size}, output_size={self.output_size}")
 
+    # Up to this many tokens the one-launch form of the layer (a wavefront per token: LayerNorm,
+    # projection, hash and the token's gather-add) beats the projection kernel followed by the
+    # table-major gather, which stages every table slice in LDS and needs many tokens to pay for it.
+    FUSED_LAYER_MAX_TOKENS = 512
+
+    def can_fuse_layer(self, x):
+        p = self.hash.projection
+        no_grad = not (torch.is_grad_enabled() and (self.tables.requires_grad or self.bias.requires_grad))
+        return (x.shape[0] <= self.FUSED_LAYER_MAX_TOKENS and self.hash.can_fuse(x) and no_grad
+                and p.padded_in_dim >= 256 and self.num_table <= 512 and self.table_size == 256
+                and self.output_size % 4 == 0 and self.tables.dtype == torch.float32
+                and self.bias.dtype == torch.float32)
+
     def _forward(self, hidden_states, residual=None):
         ln = self.LayerNorm
         ln_fusable = (ln.elementwise_affine and ln.weight is not None and ln.bias is not None
                       and ln.weight.dtype == torch.float32
                       and not (torch.is_grad_enabled() and (ln.weight.requires_grad or ln.bias.requires_grad)))
+        if ln_fusable and self.can_fuse_layer(hidden_states):
+            # small batches without gradient: the whole layer in one launch
+            p = self.hash.projection
+            diag = p.weight.reshape(p.num_repeat, p.weight.shape[1], p.padded_in_dim).contiguous()
+            return ops.lookup_ffn_fused(hidden_states.contiguous(), ln.weight, ln.bias, float(ln.eps), diag, p.bias,
+                                        self.tables, self.bias, None if residual is None else residual.contiguous(),
+                                        float(p.decay_coeff), float(1 - p.decay_coeff))
         if ln_fusable and self.hash.can_fuse(hidden_states):
             # inference: LayerNorm runs inside the projection kernel
             code, score = self.hash.forward_fused(hidden_states, layer_norm=ln)

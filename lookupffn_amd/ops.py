@@ -300,6 +300,41 @@ def _(stage_grads, x, stage_inputs, R, J):
     return x.new_empty(S, D // 64, 64, 64)
 
 
+_L.define("lookup_ffn_fused(Tensor x, Tensor ln_w, Tensor ln_b, float eps, Tensor diag, Tensor? pbias, Tensor tables, "
+          "Tensor? obias, Tensor? residual, float decay, float residual_coef) -> Tensor")
+
+
+def _lookup_ffn_fused_impl(x, ln_w, ln_b, eps, diag, pbias, tables, obias, residual, decay, residual_coef):
+    """The whole layer in one launch (PL/lookup.py:99-108): LayerNorm, diagonal BH4, mix, bias, 8-bit
+    code + score, gather-add of the T rows, output bias, optional residual [B, Do]."""
+    _lib.require_gpu(x, ln_w, ln_b, diag, tables)
+    B, H = x.shape
+    R, J, D = diag.shape
+    T, S, Do = tables.shape
+    for t in (x, ln_w, ln_b, diag, tables, pbias, obias, residual):
+        assert t is None or (t.dtype == torch.float32 and t.is_contiguous())
+    assert ln_w.numel() == H and ln_b.numel() == H
+    assert pbias is None or pbias.numel() == T * 8
+    assert obias is None or obias.numel() == Do
+    assert residual is None or tuple(residual.shape) == (B, Do)
+    out = torch.empty(B, Do, dtype=torch.float32, device=x.device)
+    with _dev_guard(x):
+        rc = _lib.load().lffn_lookup_ffn_fused_f32(
+            _lib.ptr(x), _lib.ptr(ln_w), _lib.ptr(ln_b), eps, _lib.ptr(diag), _lib.ptr(pbias), _lib.ptr(tables),
+            _lib.ptr(obias), _lib.ptr(residual), _lib.ptr(out), B, H, D, R, J, T, S, Do, decay, residual_coef,
+            _lib.stream_of(x))
+    _lib.check(rc, f"lffn_lookup_ffn_fused_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T}, S={S}, Do={Do})")
+    return out
+
+
+_L.impl("lookup_ffn_fused", _lookup_ffn_fused_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::lookup_ffn_fused")
+def _(x, ln_w, ln_b, eps, diag, pbias, tables, obias, residual, decay, residual_coef):
+    return x.new_empty(x.shape[0], tables.shape[2])
+
+
 # ----------------------------------------------------------------------------- mix_code_score
 
 _L.define("mix_code_score(Tensor y, Tensor x, Tensor? bias, int T, int k, int D, float decay, float residual)"
@@ -717,6 +752,7 @@ bh4_fold_mode = torch.ops.lookupffn.bh4_fold_mode
 bh4_block_hash_train = torch.ops.lookupffn.bh4_block_hash_train
 bh4_block_bwd = torch.ops.lookupffn.bh4_block_bwd
 bh4_block_wgrad = torch.ops.lookupffn.bh4_block_wgrad
+lookup_ffn_fused = torch.ops.lookupffn.lookup_ffn_fused
 ln_bh4_block_hash = torch.ops.lookupffn.ln_bh4_block_hash
 project_hash = torch.ops.lookupffn.project_hash
 project_hash_bwd = torch.ops.lookupffn.project_hash_bwd

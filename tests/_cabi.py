@@ -139,6 +139,21 @@ def bh4_block_wgrad(stage_grads, x, stage_inputs, R, J, init=None):
     return host(g)
 
 
+def lookup_ffn_fused(x, ln_w, ln_b, eps, diag, pbias, tables, obias, residual, decay=0.7):
+    xd, dd, td = dev(x), dev(diag), dev(tables)
+    lw, lb = (None, None) if ln_w is None else (dev(ln_w), dev(ln_b))
+    pb = None if pbias is None else dev(pbias)
+    ob = None if obias is None else dev(obias)
+    rs = None if residual is None else dev(residual)
+    B, H = x.shape
+    R, J, D = diag.shape
+    T, S, Do = tables.shape
+    out = torch.full((B, Do), float("nan"), dtype=torch.float32, device=DEV)
+    _call("lffn_lookup_ffn_fused_f32", p(xd), p(lw), p(lb), float(np.float32(eps)), p(dd), p(pb), p(td), p(ob), p(rs),
+          p(out), B, H, D, R, J, T, S, Do, float(np.float32(decay)), float(np.float32(1 - decay)))
+    return host(out)
+
+
 def mix_code_score(y, x, bias, T, k, D, decay=0.7):
     yd, xd, bd = dev(y), dev(x), dev(bias)
     B, ldy = y.shape

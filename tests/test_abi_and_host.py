@@ -117,6 +117,13 @@ def test_argument_validation_of_the_backward_and_block_entry_points():
     assert lib.lffn_lookup_scatter_sorted_f32(P, P, P, P, P, 64, 16, 4, 16, 64, 0, None) == A           # workspace too small
     assert lib.lffn_lookup_scatter_sorted_f32(P, P, P, P, None, 1 << 30, 16, 4, 16, 64, 0, None) == A
     assert lib.lffn_lookup_scatter_workspace_bytes(16, 4, 16, 64, None) == A
+    # whole layer in one launch
+    assert lib.lffn_lookup_ffn_fused_f32(P, P, P, 1e-5, P, P, P, P, P, P, 4, 64, 64, 1, 4, 8, 256, 64, 0.7, 0.3, None) == U   # D < 256
+    assert lib.lffn_lookup_ffn_fused_f32(P, P, P, 1e-5, P, P, P, P, P, P, 4, 256, 256, 1, 4, 32, 128, 64, 0.7, 0.3, None) == U  # S < 256
+    assert lib.lffn_lookup_ffn_fused_f32(P, P, P, 1e-5, P, P, P, P, P, P, 4, 256, 256, 1, 4, 32, 256, 66, 0.7, 0.3, None) == U  # Do % 4
+    assert lib.lffn_lookup_ffn_fused_f32(P, P, None, 1e-5, P, P, P, P, P, P, 4, 256, 256, 1, 4, 32, 256, 64, 0.7, 0.3, None) == A
+    assert lib.lffn_lookup_ffn_fused_f32(P, P, P, 1e-5, P, P, P, P, P, P, 4, 256, 256, 1, 4, 40, 256, 64, 0.7, 0.3, None) == A  # T*8 > R*D
+    assert lib.lffn_lookup_ffn_fused_f32(P, P, P, 1e-5, P, P, P, P, P, P, 0, 256, 256, 1, 4, 32, 256, 64, 0.7, 0.3, None) == OK
     # gather with residual
     assert lib.lffn_lookup_gather_residual_f32(P, P, P, None, P + 4, P, 4, 2, 16, 64, None) == A
 

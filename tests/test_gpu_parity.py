@@ -348,6 +348,45 @@ def test_bh4_block_wgrad_matches_float64(B, H, D, R, J):
     assert relmax(cabi.bh4_block_wgrad(sg, x, np.ascontiguousarray(si), R, J, init=init), want + init) <= 1e-5   # accumulates
 
 
+# (B, H, D, R, J, T, Do): the whole layer in one launch; ragged token counts around the four tokens
+# of a workgroup, H < D, several repeats, table counts around the eight loads in flight, output
+# widths below, at and above the 256 columns of a pass
+FUSED_LAYER_CASES = [(256, 256, 256, 1, 4, 32, 256), (5, 200, 256, 1, 4, 30, 64), (131, 768, 1024, 1, 4, 128, 768),
+                     (9, 512, 512, 2, 3, 100, 260), (1, 300, 512, 1, 1, 7, 4)]
+
+
+@pytest.mark.parametrize("B,H,D,R,J,T,Do", FUSED_LAYER_CASES)
+@pytest.mark.parametrize("with_ln", [True, False])
+def test_lookup_ffn_fused_matches_the_two_kernel_form(B, H, D, R, J, T, Do, with_ln):
+    rng = np.random.RandomState(B + H + T + Do)
+    S = 256
+    x = rng.randn(B, H).astype(np.float32)
+    ln_w = (1.0 + 0.1 * rng.randn(H)).astype(np.float32) if with_ln else None
+    ln_b = (0.1 * rng.randn(H)).astype(np.float32) if with_ln else None
+    diag = (rng.choice([-1.0, 1.0], size=(R, J, D)) / np.sqrt(D)).astype(np.float32)
+    pbias = (0.01 * rng.randn(T * 8)).astype(np.float32)
+    tables = (0.02 * rng.randn(T, S, Do)).astype(np.float32)
+    obias = (0.001 * rng.randn(Do)).astype(np.float32)
+    res = rng.randn(B, Do).astype(np.float32)
+    if with_ln:
+        code, score, _ = cabi.ln_project_hash(x, ln_w, ln_b, 1e-5, diag, pbias, T)
+    else:
+        code, score, _ = cabi.project_hash(x, diag, pbias, T)
+    idx = code + (np.arange(T, dtype=np.int32) * S)[None]
+    want = oracle.gather_add(idx, tables.reshape(T * S, Do).astype(np.float64), score.astype(np.float64))
+    got = cabi.lookup_ffn_fused(x, ln_w, ln_b, 1e-5, diag, pbias, tables, obias, res)
+    assert not np.isnan(got).any()
+    assert relmax(got, want + obias + res) <= 1e-5       # same codes and scores (same kernel body), fp32 row sums
+    got = cabi.lookup_ffn_fused(x, ln_w, ln_b, 1e-5, diag, None, tables, None, None)
+    if with_ln:
+        code, score, _ = cabi.ln_project_hash(x, ln_w, ln_b, 1e-5, diag, np.zeros(T * 8, np.float32), T)
+    else:
+        code, score, _ = cabi.project_hash(x, diag, np.zeros(T * 8, np.float32), T)
+    idx = code + (np.arange(T, dtype=np.int32) * S)[None]
+    want = oracle.gather_add(idx, tables.reshape(T * S, Do).astype(np.float64), score.astype(np.float64))
+    assert relmax(got, want) <= 1e-5
+
+
 def test_sign_diagonal_fht_exact():
     # the BASELINE "random +-1 sign diagonal from seed": one round, exact on integers
     rng = np.random.RandomState(8)
