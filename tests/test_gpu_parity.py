@@ -634,6 +634,25 @@ def _check_lds_gather(B, T, S, Do, bf16, plan):
     assert relmax(got_nb[sub], want - bias) <= 1e-5
 
 
+@pytest.mark.parametrize("bf16", [False, True])
+def test_lookup_gather_takes_many_tokens_in_pieces(bf16):
+    # from 32768 tokens on (tables that fit the cache) the entry point runs one launch per ~16384 tokens;
+    # 40001 tokens: pieces of 20032 and 19969, with a residual and a bias, every token against the oracle
+    rng = np.random.RandomState(77)
+    B, T, S, Do = 40001, 6, 16, 128
+    tables, code, idx, w = _rand_gather(rng, B, T, S, Do)
+    bias = (0.001 * rng.randn(Do)).astype(np.float32)
+    res = rng.randn(B, Do).astype(np.float32)
+    flat = tables.reshape(T * S, Do)
+    src = oracle.bf16_round(flat) if bf16 else flat
+    got = cabi.lookup_gather(code, w, src.reshape(T, S, Do), bias, bf16=bf16, residual=res)
+    if bf16:
+        want = oracle.gather_add_bf16(idx, src, w.astype(np.float64))
+    else:
+        want = oracle.gather_add(idx, flat.astype(np.float64), w.astype(np.float64))
+    assert relmax(got, want + bias + res) <= 1e-5
+
+
 @pytest.mark.parametrize("plan", F32_PLANS)
 @pytest.mark.parametrize("B,T,S,Do", LDS_SHAPES)
 def test_lookup_gather_lds_kernels_match_oracle(B, T, S, Do, plan):
