@@ -111,7 +111,14 @@ def cpu_baseline(layer, x, wl, budget_s=12.0):
         oracle.lookup_ffn(xs, *args, decay=np.float32(p.decay_coeff))
         t_total += time.perf_counter() - t0
         reps += 1
+    cpu_model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            cpu_model = next(l.split(":", 1)[1].strip() for l in f if l.startswith("model name"))
+    except (OSError, StopIteration):
+        pass
     out = {"value": n * reps / t_total, "unit": "tokens/s", "cores": oracle.num_threads(), "kind": "port",
+           "cpu_model": cpu_model,
            "sample": f"first {n} of {wl['B']} tokens, full tables, {reps} passes of the OpenMP C oracle "
                      f"(whole layer, fp32{' on bf16-rounded tables' if wl['bf16'] else ''}), {t_total:.1f} s"}
     # the reference's own x86 kernels (compiled from its sources), gather + code/score legs only
