@@ -73,7 +73,9 @@ constexpr int DPP_ROW_NEWBCAST0 = 0x150;   // + n: every lane of a 16-lane row <
 template <int N>
 __device__ __forceinline__ int row_broadcast(int v) {
     static_assert(N >= 0 && N < 16, "row_broadcast: lane within the row");
-    return __builtin_amdgcn_update_dpp(v, v, DPP_ROW_NEWBCAST0 + N, 0xF, 0xF, false);
+    // every lane has a source inside its row, so `old` is never used: 0 with bound_ctrl lets the
+    // compiler emit the bare v_mov_b32_dpp without first copying v into the destination
+    return __builtin_amdgcn_update_dpp(0, v, DPP_ROW_NEWBCAST0 + N, 0xF, 0xF, true);
 }
 
 // f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>)

@@ -60,23 +60,48 @@ struct LdsGatherArgs {
 // wait for the copy before the next LDS read of ANY address (it cannot tell the two
 // buffers apart), which would serialise the copy with the pass loop.  The caller
 // waits with vmcnt(0) before the barrier that publishes the buffer.
-__device__ __forceinline__ void lds_dma16(const char *gptr, uint32_t lds_byte_addr) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+__device__ __forceinline__ void lds_dma16(const char *table, uint32_t lane_offset, uint32_t lds_byte_addr) {
+    // scalar base + 32-bit lane offset: the lane offsets are the same for every table, so they
+    // stay in registers and a table costs no address arithmetic on the vector unit
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
-                 : "v"(gptr), "s"(lds_byte_addr)
+                 : "v"(lane_offset), "s"(table), "s"(lds_byte_addr)
                  : "memory");
 }
 
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) const u32x4 *lds_vec_ptr;
+
+// acc += (sc of lane N of the 16-lane row) * r in one instruction: the DPP row broadcast rides
+// on the multiply-add's first operand instead of costing a move of its own (the compiler
+// keeps the two apart when the broadcast value has several uses).
+template <int N>
+__device__ __forceinline__ void fmac_row_bcast(float &acc, float sc, float r) {
+    asm("v_fmac_f32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(sc), "v"(r), "n"(N));
+}
+
+// Byte offsets, from the start of a table's slice, of the four vectors this lane copies.
+struct CopyLanes {
+    uint32_t off[4];
+    uint32_t wbase;      // LDS byte offset of this wavefront's first vector inside a buffer
+};
+
+__device__ __forceinline__ CopyLanes copy_lanes(int row_bytes, int tid) {
+    CopyLanes c;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        c.off[i] = (uint32_t)((tid >> 4) + i * (WG / SEG_VECS)) * (uint32_t)row_bytes + (tid & 15) * 16;
+    c.wbase = (uint32_t)__builtin_amdgcn_readfirstlane(tid >> 6) * (64 * 16);      // scalar: never spilled with the vectors
+    return c;
+}
+
 template <bool FULL>
-__device__ __forceinline__ void copy_slice_to_lds(const char *tb, int row_bytes, int tid, int buf_vecs, uint4 *dst) {
-    const char *p = tb + (size_t)(tid >> 4) * row_bytes + (tid & 15) * 16;
-    const size_t step = (size_t)(WG / SEG_VECS) * row_bytes;   // 64 rows further down
-    // LDS byte address of this wavefront's first vector in `dst`, made scalar
-    const uint32_t wbase = __builtin_amdgcn_readfirstlane(
-        (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint4 *)(dst + (tid & ~63)));
+__device__ __forceinline__ void copy_slice_to_lds(const char *tb, const CopyLanes &c, int tid, int buf_vecs,
+                                                  uint32_t dst_byte_addr) {
+    const uint32_t wbase = dst_byte_addr + c.wbase;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        if (FULL || tid + i * WG < buf_vecs) lds_dma16(p + i * step, wbase + i * (WG * 16));
+        if (FULL || tid + i * WG < buf_vecs) lds_dma16(tb, c.off[i], wbase + i * (WG * 16));
     }
 }
 
@@ -119,11 +144,19 @@ __global__ __launch_bounds__(WG) void lookup_gather_lds_kernel(LdsGatherArgs a) 
     const char *slice_base = a.tables + (size_t)slice * (SEG_VECS * 16);
     const size_t table_bytes = (size_t)a.S * a.row_bytes;
 
-    copy_slice_to_lds<FULL>(slice_base, a.row_bytes, tid, buf_vecs, lds);
+    const CopyLanes cl = copy_lanes(a.row_bytes, tid);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint4 *)lds;
+    copy_slice_to_lds<FULL>(slice_base, cl, tid, buf_vecs, lds0);
     __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0): this lane's copies have landed in LDS
     __syncthreads();
 
-    constexpr int NQ = (NP + 3) / 4;     // codes are 8 bits (S <= 256): four passes' codes per register
+    // Codes are 8 bits (S <= 256).  bf16: four passes' codes per register.  fp32: two per
+    // register, each already shifted to bits 8..15 of its 16-bit half, which is where a row
+    // number sits in an LDS byte address (row * 256 + vector * 16 + buffer offset; S is a power
+    // of two and the codes are masked, so the fields do not overlap): an address is then one
+    // OR of a half-word with the lane's base, a single SDWA or AND-OR instruction.
+    constexpr int NQ = BF16 ? (NP + 3) / 4 : (NP + 1) / 2;
+    const unsigned lds_base = lds0 + j * 16;
     for (int t0 = 0; t0 < a.T; t0 += CHUNK) {
         // Lane j of a token group holds (code, score) of table t0 + j for each of
         // its NP tokens.  Addresses are clamped into range and the loads are
@@ -146,7 +179,10 @@ __global__ __launch_bounds__(WG) void lookup_gather_lds_kernel(LdsGatherArgs a) 
 #pragma unroll
             for (int p = 0; p < NP; ++p) {
                 const bool ok = (tok0 + p * 64 < a.B) && (tt < a.T);
-                cd[p / 4] |= unsigned(craw[p] & (a.S - 1)) << (8 * (p % 4));
+                if constexpr (BF16)
+                    cd[p / 4] |= unsigned(craw[p] & (a.S - 1)) << (8 * (p % 4));
+                else
+                    cd[p / 2] |= unsigned(craw[p] & (a.S - 1)) << (8 + 16 * (p % 2));
                 sc[p] = ok ? sc[p] : 0.f;
             }
         }
@@ -169,33 +205,34 @@ __global__ __launch_bounds__(WG) void lookup_gather_lds_kernel(LdsGatherArgs a) 
                 // next table's slice goes straight into the other buffer, which was last
                 // read one table ago, before the previous barrier (the last iteration
                 // re-copies the last table: harmless)
-                copy_slice_to_lds<FULL>(slice_base + (size_t)min(t + 1, a.T - 1) * table_bytes, a.row_bytes, tid,
-                                        buf_vecs, lds + ((t + 1) & 1) * buf_vecs);
+                copy_slice_to_lds<FULL>(slice_base + (size_t)min(t + 1, a.T - 1) * table_bytes, cl, tid, buf_vecs,
+                                        lds0 + (uint32_t)(((t + 1) & 1) * buf_vecs) * 16u);
                 const uint4 *buf = lds + (t & 1) * buf_vecs + j;
+                const unsigned buf_addr = lds_base + (unsigned)((t & 1) * buf_vecs) * 16u;
                 unsigned packed[NQ];
 #pragma unroll
                 for (int q = 0; q < NQ; ++q) packed[q] = (unsigned)row_broadcast<TT>((int)cd[q]);
                 // passes in groups of at most GRP: a group's row reads are issued together
                 // (GRP rows in flight per lane), then its fmas; the scheduling barriers keep
                 // the compiler from merging groups, which would not fit the register file
-                constexpr int GRP = BF16 ? 4 : (NP >= 16 ? 4 : (NP > 8 ? 5 : NP));
+                constexpr int GRP = BF16 ? 4 : (NP > 8 ? 4 : NP);
 #pragma unroll
                 for (int g0 = 0; g0 < NP; g0 += GRP) {
-                    uint4 r[GRP];
+                    if constexpr (BF16) {
+                        uint4 r[GRP];
 #pragma unroll
-                    for (int i = 0; i < GRP; ++i) {
-                        const int p = g0 + i;
-                        if (p < NP) {
-                            const unsigned row = (packed[p / 4] >> (8 * (p % 4))) & 0xFFu;
-                            r[i] = buf[row * SEG_VECS];
+                        for (int i = 0; i < GRP; ++i) {
+                            const int p = g0 + i;
+                            if (p < NP) {
+                                const unsigned row = (packed[p / 4] >> (8 * (p % 4))) & 0xFFu;
+                                r[i] = buf[row * SEG_VECS];
+                            }
                         }
-                    }
 #pragma unroll
-                    for (int i = 0; i < GRP; ++i) {
-                        const int p = g0 + i;
-                        if (p < NP) {
-                            const float w = __int_as_float(row_broadcast<TT>(__float_as_int(sc[p])));
-                            if constexpr (BF16) {
+                        for (int i = 0; i < GRP; ++i) {
+                            const int p = g0 + i;
+                            if (p < NP) {
+                                const float w = __int_as_float(row_broadcast<TT>(__float_as_int(sc[p])));
                                 acc[p][0] = fmaf(bf16_lo(r[i].x), w, acc[p][0]);
                                 acc[p][1] = fmaf(bf16_hi(r[i].x), w, acc[p][1]);
                                 acc[p][2] = fmaf(bf16_lo(r[i].y), w, acc[p][2]);
@@ -204,11 +241,26 @@ __global__ __launch_bounds__(WG) void lookup_gather_lds_kernel(LdsGatherArgs a) 
                                 acc[p][5] = fmaf(bf16_hi(r[i].z), w, acc[p][5]);
                                 acc[p][6] = fmaf(bf16_lo(r[i].w), w, acc[p][6]);
                                 acc[p][7] = fmaf(bf16_hi(r[i].w), w, acc[p][7]);
-                            } else {
-                                acc[p][0] = fmaf(__uint_as_float(r[i].x), w, acc[p][0]);
-                                acc[p][1] = fmaf(__uint_as_float(r[i].y), w, acc[p][1]);
-                                acc[p][2] = fmaf(__uint_as_float(r[i].z), w, acc[p][2]);
-                                acc[p][3] = fmaf(__uint_as_float(r[i].w), w, acc[p][3]);
+                            }
+                        }
+                    } else {
+                        u32x4 r[GRP];
+#pragma unroll
+                        for (int i = 0; i < GRP; ++i) {
+                            const int p = g0 + i;
+                            if (p < NP) {
+                                const unsigned half = (p % 2) ? (packed[p / 2] >> 16) : (packed[p / 2] & 0xFFFFu);
+                                r[i] = *(lds_vec_ptr)(uintptr_t)(half | buf_addr);
+                            }
+                        }
+#pragma unroll
+                        for (int i = 0; i < GRP; ++i) {
+                            const int p = g0 + i;
+                            if (p < NP) {
+                                fmac_row_bcast<TT>(acc[p][0], sc[p], __uint_as_float(r[i].x));
+                                fmac_row_bcast<TT>(acc[p][1], sc[p], __uint_as_float(r[i].y));
+                                fmac_row_bcast<TT>(acc[p][2], sc[p], __uint_as_float(r[i].z));
+                                fmac_row_bcast<TT>(acc[p][3], sc[p], __uint_as_float(r[i].w));
                             }
                         }
                     }
