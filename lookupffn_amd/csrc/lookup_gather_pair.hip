@@ -82,14 +82,23 @@ __device__ __forceinline__ void copy_pair_to_lds(const char *slice_base, size_t 
 // of row lane 8 + NHI: each 8-lane token group reads one of its own lanes.
 template <int NLO, int NHI>
 __device__ __forceinline__ int half_row_broadcast(int v) {
-    const int lo = __builtin_amdgcn_update_dpp(v, v, DPP_ROW_NEWBCAST0 + NLO, 0xF, 0x3, false);
+    // all 16 lanes <- lane NLO (every lane has a source, so no `old` value is needed: a bare
+    // v_mov_b32_dpp), then banks 2-3 (lanes 8-15) <- lane 8 + NHI on top of that
+    const int lo = __builtin_amdgcn_update_dpp(0, v, DPP_ROW_NEWBCAST0 + NLO, 0xF, 0xF, true);
     return __builtin_amdgcn_update_dpp(lo, v, DPP_ROW_NEWBCAST0 + 8 + NHI, 0xF, 0xC, false);
 }
+
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) const u32x4 *lds_vec_ptr;
 
 template <bool BF16, int NP, bool FULL>
 __global__ __launch_bounds__(WG) void lookup_gather_pair_kernel(PairArgs a) {
     constexpr int EPV = BF16 ? 8 : 4;
-    constexpr int NQ = (NP + 3) / 4;              // four 8-bit codes per register
+    // bf16: four 8-bit codes per register.  fp32: two per register, each at bits 8..15 of its
+    // 16-bit half, where a row number sits in an LDS byte address (row * 256 + ...): an address
+    // is then one OR of a half-word with the lane's base (S is a power of two and the codes are
+    // masked, so the buffer offset never overlaps the row field)
+    constexpr int NQ = BF16 ? (NP + 3) / 4 : (NP + 1) / 2;
     extern __shared__ uint4 lds[];                // 2 buffers of S * ROW_VECS vectors
 
     const int xcd = blockIdx.x % XCDS;
@@ -123,6 +132,7 @@ __global__ __launch_bounds__(WG) void lookup_gather_pair_kernel(PairArgs a) {
     }
 
     const int buf_vecs = a.S * ROW_VECS;
+    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) uint4 *)lds;
     const char *slice_base = a.tables + (size_t)slice * 128;
     const size_t table_bytes = (size_t)a.S * a.row_bytes;
     const int npairs = (a.T + 1) / 2;
@@ -146,7 +156,10 @@ __global__ __launch_bounds__(WG) void lookup_gather_pair_kernel(PairArgs a) {
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
             const bool ok = (tok0 + p * 128 < a.B) && (tt < a.T);
-            cd[p / 4] |= unsigned(craw[p] & (a.S - 1)) << (8 * (p % 4));
+            if constexpr (BF16)
+                cd[p / 4] |= unsigned(craw[p] & (a.S - 1)) << (8 * (p % 4));
+            else
+                cd[p / 2] |= unsigned(craw[p] & (a.S - 1)) << (8 + 16 * (p % 2));
             sc[p] = ok ? sc[p] : 0.f;
         }
     };
@@ -189,27 +202,28 @@ __global__ __launch_bounds__(WG) void lookup_gather_pair_kernel(PairArgs a) {
                     // (row lanes 8-15) table 2*KQ + 1 - HALF; table 2k sits in the left 128 bytes
                     constexpr int NLO = 2 * KQ + HALF, NHI = 2 * KQ + 1 - HALF;
                     const uint4 *hbuf = buf + (HALF ^ par) * 8;
+                    const unsigned haddr = lds0 + (unsigned)(((k & 1) * buf_vecs + (HALF ^ par) * 8 + j) * 16);
                     unsigned packed[NQ];
 #pragma unroll
                     for (int q = 0; q < NQ; ++q) packed[q] = (unsigned)half_row_broadcast<NLO, NHI>((int)cd[q]);
-                    constexpr int GRP = BF16 ? 4 : (NP >= 16 ? 4 : (NP > 8 ? 5 : NP));
+                    constexpr int GRP = BF16 ? 4 : (NP > 8 ? 4 : NP);
 #pragma unroll
                     for (int g0 = 0; g0 < NP; g0 += GRP) {
-                        uint4 r[GRP];
+                        if constexpr (BF16) {
+                            uint4 r[GRP];
 #pragma unroll
-                        for (int i = 0; i < GRP; ++i) {
-                            const int p = g0 + i;
-                            if (p < NP) {
-                                const unsigned row = (packed[p / 4] >> (8 * (p % 4))) & 0xFFu;
-                                r[i] = hbuf[row * ROW_VECS];
+                            for (int i = 0; i < GRP; ++i) {
+                                const int p = g0 + i;
+                                if (p < NP) {
+                                    const unsigned row = (packed[p / 4] >> (8 * (p % 4))) & 0xFFu;
+                                    r[i] = hbuf[row * ROW_VECS];
+                                }
                             }
-                        }
 #pragma unroll
-                        for (int i = 0; i < GRP; ++i) {
-                            const int p = g0 + i;
-                            if (p < NP) {
-                                const float w = __int_as_float(half_row_broadcast<NLO, NHI>(__float_as_int(sc[p])));
-                                if constexpr (BF16) {
+                            for (int i = 0; i < GRP; ++i) {
+                                const int p = g0 + i;
+                                if (p < NP) {
+                                    const float w = __int_as_float(half_row_broadcast<NLO, NHI>(__float_as_int(sc[p])));
                                     acc[p][0] = fmaf(bf16_lo(r[i].x), w, acc[p][0]);
                                     acc[p][1] = fmaf(bf16_hi(r[i].x), w, acc[p][1]);
                                     acc[p][2] = fmaf(bf16_lo(r[i].y), w, acc[p][2]);
@@ -218,7 +232,23 @@ __global__ __launch_bounds__(WG) void lookup_gather_pair_kernel(PairArgs a) {
                                     acc[p][5] = fmaf(bf16_hi(r[i].z), w, acc[p][5]);
                                     acc[p][6] = fmaf(bf16_lo(r[i].w), w, acc[p][6]);
                                     acc[p][7] = fmaf(bf16_hi(r[i].w), w, acc[p][7]);
-                                } else {
+                                }
+                            }
+                        } else {
+                            u32x4 r[GRP];
+#pragma unroll
+                            for (int i = 0; i < GRP; ++i) {
+                                const int p = g0 + i;
+                                if (p < NP) {
+                                    const unsigned half = (p % 2) ? (packed[p / 2] >> 16) : (packed[p / 2] & 0xFFFFu);
+                                    r[i] = *(lds_vec_ptr)(uintptr_t)(half | haddr);
+                                }
+                            }
+#pragma unroll
+                            for (int i = 0; i < GRP; ++i) {
+                                const int p = g0 + i;
+                                if (p < NP) {
+                                    const float w = __int_as_float(half_row_broadcast<NLO, NHI>(__float_as_int(sc[p])));
                                     acc[p][0] = fmaf(__uint_as_float(r[i].x), w, acc[p][0]);
                                     acc[p][1] = fmaf(__uint_as_float(r[i].y), w, acc[p][1]);
                                     acc[p][2] = fmaf(__uint_as_float(r[i].z), w, acc[p][2]);
