@@ -60,6 +60,7 @@ WORKLOADS = {
 # HBM bytes per launch of the gather kernel measured with rocprofv3 --pmc
 # (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); the summaries
 # are kept under profiles/.  None until measured for that workload.
+LDS_READ_PEAK_GBS = 76700.0     # microbenchmark: 125 bytes per clock per CU, 256 CUs
 MEASURED_TRAFFIC_BYTES = {"cfg2": 478224292, "cfg2b64": 478392534, "cfg3": 3166744484, "cfg3bf16": 2259132035,
                           "cfg5": 949215733}
 
@@ -521,7 +522,11 @@ def main():
                      "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-                     "algorithmic_bytes": gather_bytes, "avg_kernel_ms": gather_ms},
+                     "algorithmic_bytes": gather_bytes, "avg_kernel_ms": gather_ms,
+                     # the rows are read from LDS, whose measured read rate (conflict-free ds_read_b128 on
+                     # every CU) is 76.7 TB/s on this part: the bound that actually applies to this kernel
+                     "lds": {"row_read_bytes": B * T * Do * esz, "peak": LDS_READ_PEAK_GBS, "unit": "GB/s",
+                             "frac": B * T * Do * esz / (gather_ms * 1e-3) / 1e9 / LDS_READ_PEAK_GBS}},
         "stages_ms": ({"whole_layer": gather_ms} if fused_layer else
                       {("layernorm_bh4block_hash" if block else "layernorm_project_hash"): hash_ms,
                        "gather_add": gather_ms}),

@@ -15,7 +15,7 @@ _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 # LOOKUPFFN_HIP_LIB points at another build of the same ABI (e.g. a tuning build)
 LIB_PATH = os.environ.get("LOOKUPFFN_HIP_LIB") or os.path.join(_PKG_DIR, "liblookupffn_hip.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 LFFN_OK = 0
 LFFN_ERR_BAD_ARG = -1
