@@ -799,6 +799,26 @@ def test_lookup_scatter_sorted_matches_oracle(B, T, S, Do):
     assert np.array_equal(cabi.lookup_scatter_sorted(dirty, w, g, S), got)
 
 
+def test_lookup_scatter_sorted_random_shapes():
+    # seeded sweep: token counts around the 8-entry steps and the per-wavefront pieces, skewed and
+    # uniform codes, one to many 32-column slices
+    rng = np.random.RandomState(2024)
+    for _ in range(16):
+        B = int(rng.choice([1, 7, 8, 9, 63, 64, 65, 511, 513, 1000, 2047, 3001]))
+        T = int(rng.randint(1, 8))
+        S = int(rng.choice([1, 2, 8, 64, 256, 512]))
+        Do = 32 * int(rng.randint(1, 10))
+        code = (rng.zipf(1.3, size=(B, T)) % S).astype(np.int32) if rng.rand() < 0.5 else \
+            rng.randint(0, S, size=(B, T)).astype(np.int32)
+        w = rng.randn(B, T).astype(np.float32)
+        g = rng.randn(B, Do).astype(np.float32)
+        idx = code + (np.arange(T, dtype=np.int32) * S)[None]
+        want = oracle.scatter_add(idx, g.astype(np.float64), w.astype(np.float64), T * S).reshape(T, S, Do)
+        got = cabi.lookup_scatter_sorted(code, w, g, S)
+        assert not np.isnan(got).any(), (B, T, S, Do)
+        assert relmax(got, want) <= 1e-5, (B, T, S, Do)
+
+
 def test_lookup_scatter_sorted_workspace_query():
     assert cabi.lookup_scatter_workspace_bytes(16384, 128, 256, 768) >= 16384 * 128 * 8
     assert cabi.lookup_scatter_workspace_bytes(1 << 20, 128, 256, 768) == cabi.lookup_scatter_workspace_bytes(16384, 128, 256, 768)
