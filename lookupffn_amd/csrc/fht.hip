@@ -36,9 +36,51 @@ struct FhtCfg {
     static_assert(LOGD >= 2 && LOGD <= 10, "FHT dims 4..1024");
 };
 
-template <int M, int LPR, int NJ>
+// Butterflies across lanes 16 or 32 apart, two values at a time, with the gfx950 row / half-wave
+// swaps: swap(a, b) hands every lane one of the two values together with that value's partner,
+// so a plain add and subtract give both results, and a second swap puts them back in place.
+// Four vector-ALU instructions per pair of values, no LDS permute and no sign multiply; the
+// sums are the same additions as in the one-value form (a + b and a - b are commutative up to
+// the sign of b), so results are unchanged bit for bit.
+template <int M>
+__device__ __forceinline__ void butterfly_swap_pair(float &e0, float &e1) {
+    static_assert(M == 16 || M == 32, "swap butterflies: rows (16) or half-waves (32)");
+    unsigned a = __float_as_uint(e0), b = __float_as_uint(e1);
+    if constexpr (M == 32) {
+        const auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+        a = r[0]; b = r[1];
+    } else {
+        const auto r = __builtin_amdgcn_permlane16_swap(a, b, false, false);
+        a = r[0]; b = r[1];
+    }
+    const float s = __uint_as_float(a) + __uint_as_float(b);
+    const float d = __uint_as_float(a) - __uint_as_float(b);
+    unsigned su = __float_as_uint(s), du = __float_as_uint(d);
+    if constexpr (M == 32) {
+        const auto r = __builtin_amdgcn_permlane32_swap(su, du, false, false);
+        su = r[0]; du = r[1];
+    } else {
+        const auto r = __builtin_amdgcn_permlane16_swap(su, du, false, false);
+        su = r[0]; du = r[1];
+    }
+    e0 = __uint_as_float(su);
+    e1 = __uint_as_float(du);
+}
+
+// SWAP: lane distances 16 and 32 with the swap butterflies instead of LDS permutes.  The swaps
+// cost more vector-ALU time than a permute plus a multiply-add: the forward kernels, which run
+// many wavefronts per SIMD and are bound by ALU issue, are faster with the permutes (59 against
+// 66 us at 16384 x 1024, four stages); the backward kernel, two wavefronts per SIMD and waiting
+// on every permute, is faster with the swaps (178 -> 130 us).
+template <int M, int LPR, int NJ, bool SWAP>
 __device__ __forceinline__ void lane_stage(float (&v)[NJ][4], int lr) {
-    if constexpr (M >= 1 && M < LPR) {
+    if constexpr (SWAP && (M == 16 || M == 32) && M < LPR) {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            butterfly_swap_pair<M>(v[j][0], v[j][1]);
+            butterfly_swap_pair<M>(v[j][2], v[j][3]);
+        }
+    } else if constexpr (M >= 1 && M < LPR) {
         const float sgn = (lr & M) ? -1.0f : 1.0f;
 #pragma unroll
         for (int j = 0; j < NJ; ++j)
@@ -47,7 +89,7 @@ __device__ __forceinline__ void lane_stage(float (&v)[NJ][4], int lr) {
     }
 }
 
-template <int LOGD>
+template <int LOGD, bool SWAP = false>
 __device__ __forceinline__ void fht_rows(float (&v)[FhtCfg<LOGD>::NJ][4], int lr) {
     using C = FhtCfg<LOGD>;
     constexpr int NJ = C::NJ;
@@ -73,12 +115,12 @@ __device__ __forceinline__ void fht_rows(float (&v)[FhtCfg<LOGD>::NJ][4], int lr
             }
     }
     // strides 4*32 .. 4*1: across lanes
-    lane_stage<32, C::LPR, NJ>(v, lr);
-    lane_stage<16, C::LPR, NJ>(v, lr);
-    lane_stage<8, C::LPR, NJ>(v, lr);
-    lane_stage<4, C::LPR, NJ>(v, lr);
-    lane_stage<2, C::LPR, NJ>(v, lr);
-    lane_stage<1, C::LPR, NJ>(v, lr);
+    lane_stage<32, C::LPR, NJ, SWAP>(v, lr);
+    lane_stage<16, C::LPR, NJ, SWAP>(v, lr);
+    lane_stage<8, C::LPR, NJ, SWAP>(v, lr);
+    lane_stage<4, C::LPR, NJ, SWAP>(v, lr);
+    lane_stage<2, C::LPR, NJ, SWAP>(v, lr);
+    lane_stage<1, C::LPR, NJ, SWAP>(v, lr);
     // strides 2 and 1: inside a float4
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
@@ -429,7 +471,7 @@ __global__ __launch_bounds__(256) void project_hash_bwd_kernel(ProjectBwdArgs a)
                     for (int c = 0; c < 4; ++c) u[s][j][c] = t[j][c];
                     t[j][0] = t[j][0] * w.x; t[j][1] = t[j][1] * w.y; t[j][2] = t[j][2] * w.z; t[j][3] = t[j][3] * w.w;
                 }
-                if (s + 1 < a.J) fht_rows<LOGD>(t, lr);      // the last transform's output is not needed
+                if (s + 1 < a.J) fht_rows<LOGD, true>(t, lr);      // the last transform's output is not needed
             }
         }
 
@@ -479,7 +521,7 @@ __global__ __launch_bounds__(256) void project_hash_bwd_kernel(ProjectBwdArgs a)
 #pragma unroll
         for (int s = MAXJ - 1; s >= 0; --s) {
             if (s < a.J) {
-                fht_rows<LOGD>(t, lr);
+                fht_rows<LOGD, true>(t, lr);
                 const float *dg = a.diag + (int64_t(r) * a.J + s) * D;
 #pragma unroll
                 for (int j = 0; j < NJ; ++j) {

@@ -87,18 +87,25 @@ __device__ __forceinline__ void static_for(F &&f) {
     }
 }
 
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov_all(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+
 // Value held by lane (lane ^ M), for M a power of two below 64.
 template <int M>
 __device__ __forceinline__ float lane_xor(float v) {
+    // Where every lane has a source, `old` is never used: 0 with bound_ctrl gives the bare
+    // v_mov_b32_dpp, without a copy of v into the destination first.
     if constexpr (M == 1) {
-        return dpp_mov<DPP_QUAD_XOR1>(v, v);
+        return dpp_mov_all<DPP_QUAD_XOR1>(v);
     } else if constexpr (M == 2) {
-        return dpp_mov<DPP_QUAD_XOR2>(v, v);
+        return dpp_mov_all<DPP_QUAD_XOR2>(v);
     } else if constexpr (M == 4) {
-        float r = dpp_mov<DPP_ROW_SHL4, 0xF, 0x5>(v, v);   // banks 0,2 take lane+4
+        float r = dpp_mov_all<DPP_ROW_SHL4>(v);            // lane+4 (banks 0,2 keep it; lanes 12-15 read 0)
         return dpp_mov<DPP_ROW_SHR4, 0xF, 0xA>(r, v);      // banks 1,3 take lane-4
     } else if constexpr (M == 8) {
-        return dpp_mov<DPP_ROW_ROR8>(v, v);
+        return dpp_mov_all<DPP_ROW_ROR8>(v);
     } else if constexpr (M == 16) {
         // ds_swizzle, bit-mask mode inside 32 lanes: and 0x1F, or 0, xor 0x10
         return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401F));
@@ -110,9 +117,8 @@ __device__ __forceinline__ float lane_xor(float v) {
 
 // One butterfly across lanes: the lane whose M bit is clear gets own + partner,
 // the other gets partner - own.  `sgn` is +1 / -1 for the two cases.
-// (The gfx950 v_permlane16_swap / v_permlane32_swap instructions can do the M = 16
-// and M = 32 exchanges on the vector ALU; measured on the projection kernel they
-// were 15 % slower than ds_swizzle / ds_bpermute, so they are not used.)
+// (The gfx950 v_permlane16_swap / v_permlane32_swap instructions can do the M = 16 and M = 32
+// exchanges on the vector ALU; the kernels that wait on LDS permutes use them, see fht.hip.)
 template <int M>
 __device__ __forceinline__ float butterfly_xor(float v, float sgn) {
     return fmaf(v, sgn, lane_xor<M>(v));   // (+-1)*v is exact: one rounding, like a plain add
