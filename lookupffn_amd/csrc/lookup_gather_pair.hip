@@ -98,7 +98,9 @@ __global__ __launch_bounds__(WG) void lookup_gather_pair_kernel(PairArgs a) {
     // 16-bit half, where a row number sits in an LDS byte address (row * 256 + ...): an address
     // is then one OR of a half-word with the lane's base (S is a power of two and the codes are
     // masked, so the buffer offset never overlaps the row field)
-    constexpr int NQ = BF16 ? (NP + 3) / 4 : (NP + 1) / 2;
+    // (at 16 passes the extra code registers of the two-per-register form would spill: four per register there)
+    constexpr bool WIDE = !BF16 && NP <= 13;
+    constexpr int NQ = WIDE ? (NP + 1) / 2 : (NP + 3) / 4;
     extern __shared__ uint4 lds[];                // 2 buffers of S * ROW_VECS vectors
 
     const int xcd = blockIdx.x % XCDS;
@@ -156,10 +158,10 @@ __global__ __launch_bounds__(WG) void lookup_gather_pair_kernel(PairArgs a) {
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
             const bool ok = (tok0 + p * 128 < a.B) && (tt < a.T);
-            if constexpr (BF16)
-                cd[p / 4] |= unsigned(craw[p] & (a.S - 1)) << (8 * (p % 4));
-            else
+            if constexpr (WIDE)
                 cd[p / 2] |= unsigned(craw[p] & (a.S - 1)) << (8 + 16 * (p % 2));
+            else
+                cd[p / 4] |= unsigned(craw[p] & (a.S - 1)) << (8 * (p % 4));
             sc[p] = ok ? sc[p] : 0.f;
         }
     };
@@ -240,8 +242,13 @@ __global__ __launch_bounds__(WG) void lookup_gather_pair_kernel(PairArgs a) {
                             for (int i = 0; i < GRP; ++i) {
                                 const int p = g0 + i;
                                 if (p < NP) {
-                                    const unsigned half = (p % 2) ? (packed[p / 2] >> 16) : (packed[p / 2] & 0xFFFFu);
-                                    r[i] = *(lds_vec_ptr)(uintptr_t)(half | haddr);
+                                    if constexpr (WIDE) {
+                                        const unsigned half = (p % 2) ? (packed[p / 2] >> 16) : (packed[p / 2] & 0xFFFFu);
+                                        r[i] = *(lds_vec_ptr)(uintptr_t)(half | haddr);
+                                    } else {
+                                        const unsigned row = (packed[p / 4] >> (8 * (p % 4))) & 0xFFu;
+                                        r[i] = *(lds_vec_ptr)(uintptr_t)(haddr + row * (ROW_VECS * 16));
+                                    }
                                 }
                             }
 #pragma unroll
