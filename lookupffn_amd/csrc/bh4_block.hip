@@ -126,6 +126,12 @@ struct BlockArgs {
 // weights is the per-block product P_s^T U_s over all tokens (U_s = the stage's input, which
 // the forward saved), formed by the caller.  Tile load: decay * grad z; result: grad x of
 // this repeat = G_0[:, :H] + residual * grad z[:, :H].
+// Lanes 16-31 and 48-63 get the value of the lane 16 below; the other lanes keep their own.
+__device__ __forceinline__ float from_row_below(float v) {
+    const unsigned u = __float_as_uint(v);
+    return __uint_as_float(__builtin_amdgcn_permlane16_swap(u, u, false, false)[0]);
+}
+
 template <int NB, bool HASH, int NH, bool BWD = false>
 __global__ __launch_bounds__(128 * (4 / NH)) void bh4_block_kernel(BlockArgs a) {
     static_assert(!(HASH && BWD), "one form at a time");
@@ -528,9 +534,11 @@ __global__ __launch_bounds__(128 * (4 / NH)) void bh4_block_kernel(BlockArgs a) 
                         float s_loc = 0.f, p_loc = 1.f;
 #pragma unroll
                         for (int i = 0; i < 4; ++i) { s_loc = s_loc + az[i]; p_loc = p_loc * fz[i]; }
-                        float s_run = lane_xor<16>(s_loc);
-                        float p_run = lane_xor<16>(p_loc);
-                        const int nib_hi = __float_as_int(lane_xor<16>(__int_as_float(nib)));
+                        // odd rows of 16 lanes take over from the lane 16 below (a row swap on the vector
+                        // ALU: with two wavefronts per SIMD an LDS permute here is waited for every time)
+                        float s_run = from_row_below(s_loc);
+                        float p_run = from_row_below(p_loc);
+                        const int nib_hi = __float_as_int(from_row_below(__int_as_float(nib)));
 #pragma unroll
                         for (int i = 0; i < 4; ++i) { s_run = s_run + az[i]; p_run = p_run * fz[i]; }
                         // staged in LDS (the stage buffer is free now), written out row by row below:
