@@ -167,6 +167,19 @@ int lffn_bh4_block_bwd_f32(const float *g_z, const float *w_folded_t, float *g_x
                            int64_t block_size, float decay, float residual, void *stream);
 
 /*
+ * Backward of the layer's LayerNorm (torch.nn.LayerNorm over the last dimension, PL/lookup.py:84,99)
+ * in one kernel; mean and 1/sigma are recomputed from x.
+ *   g = sum_r g_y[r];  g_x = rstd * (g*w - mean(g*w) - x^ * mean(g*w*x^));  g_w = sum_b g*x^;  g_b = sum_b g
+ * x: [B, H]; ln_weight: [H] or null (no affine); g_y: [R, B, H] (R >= 1 gradients that are added up:
+ * the repeats of the projection); g_x: [B, H]; part_weight, part_bias: [num_partials, H], one
+ * partial sum per workgroup, to be added up by the caller, or both null.  H % 4 == 0, H <= 1024.
+ * Replaces what autograd records for the LayerNorm of PL/lookup.py:99.
+ */
+int lffn_layer_norm_bwd_f32(const float *x, const float *ln_weight, float ln_eps, const float *g_y, float *g_x,
+                            float *part_weight, float *part_bias, int64_t B, int64_t H, int64_t R,
+                            int64_t num_partials, void *stream);
+
+/*
  * The whole layer in one launch, for small batches without gradient (PL/lookup.py:99-108):
  *   out[b, :] = sum_t score[b,t] * tables[t, code[b,t], :] + out_bias (+ residual_in[b, :])
  * with (code, score) the 8-bit hash of 0.7 * BH4(LayerNorm(x)) + 0.3 * tile(LayerNorm(x)) +

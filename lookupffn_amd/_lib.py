@@ -45,6 +45,7 @@ SIGNATURES = {
                                ctypes.c_float, ctypes.c_float, _vp],
     "lffn_lookup_ffn_fused_f32": [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
                                   _i64, _i64, _i64, ctypes.c_float, ctypes.c_float, _vp],
+    "lffn_layer_norm_bwd_f32": [_vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "lffn_bh4_block_wgrad_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp],
     "lffn_bh4_fold_f32": [_vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "lffn_bh4_block_f32": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp],

@@ -1,0 +1,132 @@
+// Backward of the layer's LayerNorm (PL/lookup.py:84,99: torch.nn.LayerNorm over the last
+// dimension, biased variance, eps inside the square root), one kernel:
+//
+//   g    = sum_r g_y[r]                       (the projection's R repeats each bring a gradient)
+//   x^   = (x - mean) * rstd                  (recomputed from x: nothing is kept from the forward)
+//   g_x  = rstd * (g*w - mean_H(g*w) - x^ * mean_H(g*w * x^))
+//   g_w  = sum_b g * x^ ,   g_b = sum_b g
+//
+// One wavefront per row, H / 64 values per lane in registers (H <= 1024, H % 4 == 0), two
+// wave reductions per row.  The weight and bias gradients are summed over a workgroup's rows in
+// registers, over its four wavefronts in LDS, and written as one partial per workgroup; the
+// caller adds the partials (a few hundred rows of H values).  This replaces what autograd runs
+// for the reference (two kernels over the rows plus column reductions).
+#include "lffn_common.h"
+
+namespace {
+
+constexpr int NJ_MAX = 4;            // float4 per lane: H <= 1024
+
+struct LnBwdArgs {
+    const float *x;       // [B, H]
+    const float *w;       // [H] or null (no affine: w = 1)
+    const float *gy;      // [R, B, H]
+    float *gx;            // [B, H]
+    float *part_w;        // [num_partials, H] or null
+    float *part_b;        // [num_partials, H] or null
+    int64_t B;
+    int H, R;
+    float eps;
+};
+
+template <int NJ>
+__global__ __launch_bounds__(256) void layer_norm_bwd_kernel(LnBwdArgs a) {
+    __shared__ float red[2][4][NJ * 256];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float inv_h = 1.0f / float(a.H);
+
+    float4 wv[NJ], aw[NJ], ab[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        const int e = 256 * j + 4 * lane;
+        wv[j] = make_float4(1.f, 1.f, 1.f, 1.f);
+        if (a.w && e < a.H) wv[j] = *reinterpret_cast<const float4 *>(a.w + e);
+        aw[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+        ab[j] = aw[j];
+    }
+
+    for (int64_t row = int64_t(blockIdx.x) * 4 + wave; row < a.B; row += int64_t(gridDim.x) * 4) {
+        float4 xv[NJ], g[NJ];
+        float s = 0.f;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const int e = 256 * j + 4 * lane;
+            xv[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+            g[j] = xv[j];
+            if (e < a.H) {
+                xv[j] = *reinterpret_cast<const float4 *>(a.x + row * a.H + e);
+                for (int r = 0; r < a.R; ++r) {
+                    const float4 t = *reinterpret_cast<const float4 *>(a.gy + (int64_t(r) * a.B + row) * a.H + e);
+                    g[j].x += t.x; g[j].y += t.y; g[j].z += t.z; g[j].w += t.w;
+                }
+            }
+            s += (xv[j].x + xv[j].y) + (xv[j].z + xv[j].w);
+        }
+        const float mean = wave_sum(s) * inv_h;
+        float v = 0.f;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const bool on = 256 * j + 4 * lane < a.H;
+            xv[j].x = on ? xv[j].x - mean : 0.f; xv[j].y = on ? xv[j].y - mean : 0.f;
+            xv[j].z = on ? xv[j].z - mean : 0.f; xv[j].w = on ? xv[j].w - mean : 0.f;
+            v += (xv[j].x * xv[j].x + xv[j].y * xv[j].y) + (xv[j].z * xv[j].z + xv[j].w * xv[j].w);
+        }
+        const float rstd = 1.0f / sqrtf(wave_sum(v) * inv_h + a.eps);
+        float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            xv[j].x *= rstd; xv[j].y *= rstd; xv[j].z *= rstd; xv[j].w *= rstd;        // x^
+            aw[j].x += g[j].x * xv[j].x; aw[j].y += g[j].y * xv[j].y; aw[j].z += g[j].z * xv[j].z; aw[j].w += g[j].w * xv[j].w;
+            ab[j].x += g[j].x; ab[j].y += g[j].y; ab[j].z += g[j].z; ab[j].w += g[j].w;
+            g[j].x *= wv[j].x; g[j].y *= wv[j].y; g[j].z *= wv[j].z; g[j].w *= wv[j].w;   // g * w
+            s1 += (g[j].x + g[j].y) + (g[j].z + g[j].w);
+            s2 += (g[j].x * xv[j].x + g[j].y * xv[j].y) + (g[j].z * xv[j].z + g[j].w * xv[j].w);
+        }
+        const float m1 = wave_sum(s1) * inv_h, m2 = wave_sum(s2) * inv_h;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const int e = 256 * j + 4 * lane;
+            if (e < a.H)
+                *reinterpret_cast<float4 *>(a.gx + row * a.H + e) =
+                    make_float4(rstd * (g[j].x - m1 - xv[j].x * m2), rstd * (g[j].y - m1 - xv[j].y * m2),
+                                rstd * (g[j].z - m1 - xv[j].z * m2), rstd * (g[j].w - m1 - xv[j].w * m2));
+        }
+    }
+
+    if (a.part_w) {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            *reinterpret_cast<float4 *>(&red[0][wave][256 * j + 4 * lane]) = aw[j];
+            *reinterpret_cast<float4 *>(&red[1][wave][256 * j + 4 * lane]) = ab[j];
+        }
+        __syncthreads();
+        for (int e = threadIdx.x; e < a.H; e += 256) {
+            a.part_w[(size_t)blockIdx.x * a.H + e] = (red[0][0][e] + red[0][1][e]) + (red[0][2][e] + red[0][3][e]);
+            a.part_b[(size_t)blockIdx.x * a.H + e] = (red[1][0][e] + red[1][1][e]) + (red[1][2][e] + red[1][3][e]);
+        }
+    }
+}
+
+}  // namespace
+
+extern "C" int lffn_layer_norm_bwd_f32(const float *x, const float *ln_weight, float ln_eps, const float *g_y,
+                                       float *g_x, float *part_weight, float *part_bias, int64_t B, int64_t H,
+                                       int64_t R, int64_t num_partials, void *stream) {
+    LFFN_REQUIRE(B >= 0 && H >= 1 && R >= 1 && ln_eps >= 0.f, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(H % 4 == 0 && H <= 256 * NJ_MAX && B <= (int64_t(1) << 31) - 1 && R <= 64, LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(num_partials >= 1 && num_partials <= 65535, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE((part_weight != nullptr) == (part_bias != nullptr), LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE((x && g_y && g_x) || B == 0, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_aligned16(x) && lffn_aligned16(g_y) && lffn_aligned16(g_x) &&
+                     (!ln_weight || lffn_aligned16(ln_weight)), LFFN_ERR_BAD_ARG);
+    LnBwdArgs a{};
+    a.x = x; a.w = ln_weight; a.gy = g_y; a.gx = g_x; a.part_w = part_weight; a.part_b = part_bias;
+    a.B = B; a.H = (int)H; a.R = (int)R; a.eps = ln_eps;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const dim3 grid((unsigned)num_partials);       // every workgroup writes its partial, rows or not
+    if (H <= 256) hipLaunchKernelGGL((layer_norm_bwd_kernel<1>), grid, dim3(256), 0, st, a);
+    else if (H <= 512) hipLaunchKernelGGL((layer_norm_bwd_kernel<2>), grid, dim3(256), 0, st, a);
+    else if (H <= 768) hipLaunchKernelGGL((layer_norm_bwd_kernel<3>), grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((layer_norm_bwd_kernel<4>), grid, dim3(256), 0, st, a);
+    return lffn_launch_status();
+}

@@ -15,6 +15,7 @@ import math
 import numpy as np
 import torch
 import torch.nn as nn
+import torch.nn.functional as F
 
 from . import ops
 from .bh4 import bh4
@@ -242,6 +243,24 @@ class Hashing(nn.Module):
         return code, score
 
 
+class LayerNormFn(torch.autograd.Function):
+    """torch's LayerNorm forward with a one-kernel backward (ops.layer_norm_bwd): mean and 1/sigma are
+    recomputed from the input, the weight and bias gradients come out of the same pass."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, eps):
+        ctx.save_for_backward(x, weight)
+        ctx.eps = float(eps)
+        return F.layer_norm(x, (x.shape[-1],), weight, bias, eps)
+
+    @staticmethod
+    def backward(ctx, g_y):
+        x, weight = ctx.saved_tensors
+        g_x, g_w, g_b = ops.layer_norm_bwd(x, weight, ctx.eps, g_y.contiguous()[None])
+        return (g_x if ctx.needs_input_grad[0] else None, g_w if ctx.needs_input_grad[1] else None,
+                g_b if ctx.needs_input_grad[2] else None, None)
+
+
 class LookupFFN(nn.Module):
     """PL/lookup.py:79-130."""
 
@@ -293,7 +312,12 @@ class LookupFFN(nn.Module):
         elif ln_fusable and self.hash.can_fuse_block(hidden_states):
             code, score = self.hash.forward_block(hidden_states, layer_norm=ln)
         else:
-            hidden_states = ln(hidden_states)
+            if (torch.is_grad_enabled() and hidden_states.is_cuda and hidden_states.dtype == torch.float32
+                    and ln.elementwise_affine and ln.weight is not None and ln.bias is not None
+                    and ln.weight.dtype == torch.float32 and self.hidden_size % 4 == 0 and self.hidden_size <= 1024):
+                hidden_states = LayerNormFn.apply(hidden_states.contiguous(), ln.weight, ln.bias, ln.eps)
+            else:
+                hidden_states = ln(hidden_states)
             code, score = self.hash(hidden_states)
         if self.output_size % 64 == 0 and self.tables.dtype in (torch.float32, torch.bfloat16):
             # table-local codes, offset and bias folded into the gather kernel

@@ -335,6 +335,39 @@ def _(x, ln_w, ln_b, eps, diag, pbias, tables, obias, residual, decay, residual_
     return x.new_empty(x.shape[0], tables.shape[2])
 
 
+LN_BWD_PARTIALS = 512
+
+_L.define("layer_norm_bwd(Tensor x, Tensor? weight, float eps, Tensor g_y) -> (Tensor, Tensor, Tensor)")
+
+
+def _layer_norm_bwd_impl(x, weight, eps, g_y):
+    """Backward of LayerNorm over the last dimension of x [B, H]; g_y is [R, B, H] (the R gradients are
+    added up).  -> (g_x [B, H], g_weight [H], g_bias [H])."""
+    _lib.require_gpu(x, g_y)
+    B, H = x.shape
+    assert g_y.dim() == 3 and tuple(g_y.shape[1:]) == (B, H)
+    for t in (x, weight, g_y):
+        assert t is None or (t.dtype == torch.float32 and t.is_contiguous())
+    R = g_y.shape[0]
+    n = max(1, min(LN_BWD_PARTIALS, (B + 3) // 4))
+    g_x = torch.empty_like(x)
+    part = torch.empty(2, n, H, dtype=torch.float32, device=x.device)
+    with _dev_guard(x):
+        rc = _lib.load().lffn_layer_norm_bwd_f32(_lib.ptr(x), _lib.ptr(weight), eps, _lib.ptr(g_y), _lib.ptr(g_x),
+                                                 _lib.ptr(part[0]), _lib.ptr(part[1]), B, H, R, n, _lib.stream_of(x))
+    _lib.check(rc, f"lffn_layer_norm_bwd_f32(B={B}, H={H}, R={R})")
+    sums = part.sum(1)
+    return g_x, sums[0], sums[1]
+
+
+_L.impl("layer_norm_bwd", _layer_norm_bwd_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::layer_norm_bwd")
+def _(x, weight, eps, g_y):
+    return torch.empty_like(x), x.new_empty(x.shape[1]), x.new_empty(x.shape[1])
+
+
 # ----------------------------------------------------------------------------- mix_code_score
 
 _L.define("mix_code_score(Tensor y, Tensor x, Tensor? bias, int T, int k, int D, float decay, float residual)"
@@ -753,6 +786,7 @@ bh4_block_hash_train = torch.ops.lookupffn.bh4_block_hash_train
 bh4_block_bwd = torch.ops.lookupffn.bh4_block_bwd
 bh4_block_wgrad = torch.ops.lookupffn.bh4_block_wgrad
 lookup_ffn_fused = torch.ops.lookupffn.lookup_ffn_fused
+layer_norm_bwd = torch.ops.lookupffn.layer_norm_bwd
 ln_bh4_block_hash = torch.ops.lookupffn.ln_bh4_block_hash
 project_hash = torch.ops.lookupffn.project_hash
 project_hash_bwd = torch.ops.lookupffn.project_hash_bwd

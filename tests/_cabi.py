@@ -154,6 +154,17 @@ def lookup_ffn_fused(x, ln_w, ln_b, eps, diag, pbias, tables, obias, residual, d
     return host(out)
 
 
+def layer_norm_bwd(x, w, eps, g_y, num_partials=7):
+    xd, gd = dev(x), dev(g_y)
+    wd = None if w is None else dev(w)
+    R, B, H = g_y.shape
+    g_x = torch.full((B, H), float("nan"), dtype=torch.float32, device=DEV)
+    pw = torch.full((num_partials, H), float("nan"), dtype=torch.float32, device=DEV)
+    pb = torch.full((num_partials, H), float("nan"), dtype=torch.float32, device=DEV)
+    _call("lffn_layer_norm_bwd_f32", p(xd), p(wd), float(np.float32(eps)), p(gd), p(g_x), p(pw), p(pb), B, H, R, num_partials)
+    return host(g_x), host(pw).astype(np.float64).sum(0), host(pb).astype(np.float64).sum(0)
+
+
 def mix_code_score(y, x, bias, T, k, D, decay=0.7):
     yd, xd, bd = dev(y), dev(x), dev(bias)
     B, ldy = y.shape

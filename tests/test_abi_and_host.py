@@ -124,6 +124,11 @@ def test_argument_validation_of_the_backward_and_block_entry_points():
     assert lib.lffn_lookup_ffn_fused_f32(P, P, None, 1e-5, P, P, P, P, P, P, 4, 256, 256, 1, 4, 32, 256, 64, 0.7, 0.3, None) == A
     assert lib.lffn_lookup_ffn_fused_f32(P, P, P, 1e-5, P, P, P, P, P, P, 4, 256, 256, 1, 4, 40, 256, 64, 0.7, 0.3, None) == A  # T*8 > R*D
     assert lib.lffn_lookup_ffn_fused_f32(P, P, P, 1e-5, P, P, P, P, P, P, 0, 256, 256, 1, 4, 32, 256, 64, 0.7, 0.3, None) == OK
+    # LayerNorm backward
+    assert lib.lffn_layer_norm_bwd_f32(P, P, 1e-5, P, P, P, P, 4, 1028, 1, 8, None) == U      # H > 1024
+    assert lib.lffn_layer_norm_bwd_f32(P, P, 1e-5, P, P, P, P, 4, 770, 1, 8, None) == U       # H % 4
+    assert lib.lffn_layer_norm_bwd_f32(P, P, 1e-5, P, P, P, None, 4, 768, 1, 8, None) == A    # partials: both or none
+    assert lib.lffn_layer_norm_bwd_f32(P, P, 1e-5, P, P, P, P, 4, 768, 1, 0, None) == A
     # gather with residual
     assert lib.lffn_lookup_gather_residual_f32(P, P, P, None, P + 4, P, 4, 2, 16, 64, None) == A
 

@@ -387,6 +387,29 @@ def test_lookup_ffn_fused_matches_the_two_kernel_form(B, H, D, R, J, T, Do, with
     assert relmax(got, want) <= 1e-5
 
 
+@pytest.mark.parametrize("B,H,R", [(1000, 768, 1), (37, 1024, 4), (5, 4, 1), (300, 260, 2), (0, 64, 1), (64, 512, 1)])
+@pytest.mark.parametrize("affine", [True, False])
+def test_layer_norm_bwd_matches_float64(B, H, R, affine):
+    rng = np.random.RandomState(B + H + R)
+    x = (rng.randn(B, H) * 2 + 0.5).astype(np.float32)
+    w = (1 + 0.2 * rng.randn(H)).astype(np.float32) if affine else None
+    gy = rng.randn(R, B, H).astype(np.float32)
+    eps = 1e-5
+    x64, g = x.astype(np.float64), gy.astype(np.float64).sum(0)
+    mean = x64.mean(1, keepdims=True)
+    rstd = 1.0 / np.sqrt(x64.var(1, keepdims=True) + eps)
+    xh = (x64 - mean) * rstd
+    gw = g * (w.astype(np.float64) if affine else 1.0)
+    want_x = rstd * (gw - gw.mean(1, keepdims=True) - xh * (gw * xh).mean(1, keepdims=True))
+    got_x, got_w, got_b = cabi.layer_norm_bwd(x, w, eps, gy)
+    if B == 0:
+        assert not got_w.any() and not got_b.any()
+        return
+    assert relmax(got_x, want_x) <= 2e-5
+    assert relmax(got_w, (g * xh).sum(0)) <= 2e-5
+    assert relmax(got_b, g.sum(0)) <= 2e-5
+
+
 def test_sign_diagonal_fht_exact():
     # the BASELINE "random +-1 sign diagonal from seed": one round, exact on integers
     rng = np.random.RandomState(8)
