@@ -335,6 +335,26 @@ int lffn_lookup_gather_residual_bf16(const int32_t *code, const float *score, co
                                      int64_t B, int64_t T, int64_t S, int64_t Do, void *stream);
 
 /*
+ * The same gather with a caller-provided workspace, for batches of a few thousand tokens: too
+ * few (token tile, column slice) units to fill the chip at the tile sizes that make staging
+ * tables in LDS pay.  Several workgroups then share a unit, each adding a range of the tables
+ * into its own partial output in the workspace, and a second kernel adds the partials, in table
+ * order, with bias and residual (results are reproducible, and equal to the one-part kernel's
+ * up to the association of the fp32 sums).  lffn_lookup_gather_workspace_bytes sets *bytes to
+ * the workspace that pays for a shape, or to 0 when the plain entry points are as fast
+ * (16384 tokens and more at the RoBERTa-base tables, or very few tokens); with a null or too
+ * small workspace the _ws entry points behave exactly like lffn_lookup_gather_residual_*.
+ * residual may be null.  Same replacement as lffn_lookup_gather_f32 (PL/lookup.py:120-130, 108).
+ */
+int lffn_lookup_gather_workspace_bytes(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t bf16, int64_t *bytes);
+int lffn_lookup_gather_ws_f32(const int32_t *code, const float *score, const float *tables, const float *bias,
+                              const float *residual, float *out, void *workspace, int64_t workspace_bytes,
+                              int64_t B, int64_t T, int64_t S, int64_t Do, void *stream);
+int lffn_lookup_gather_ws_bf16(const int32_t *code, const float *score, const uint16_t *tables, const float *bias,
+                               const float *residual, float *out, void *workspace, int64_t workspace_bytes,
+                               int64_t B, int64_t T, int64_t S, int64_t Do, void *stream);
+
+/*
  * Which kernel lffn_lookup_gather_{f32,bf16} runs for a shape.  Returns the number
  * of tokens whose accumulators one workgroup keeps in registers while it walks the
  * tables through LDS, or 0 when the token-major kernel is used (small batches,

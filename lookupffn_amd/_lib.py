@@ -64,6 +64,9 @@ SIGNATURES = {
                                        ctypes.c_int32, ctypes.c_int32, _vp],
     "lffn_lookup_gather_planned_bf16": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64,
                                         ctypes.c_int32, ctypes.c_int32, _vp],
+    "lffn_lookup_gather_workspace_bytes": [_i64, _i64, _i64, _i64, ctypes.c_int32, ctypes.POINTER(ctypes.c_int64)],
+    "lffn_lookup_gather_ws_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp],
+    "lffn_lookup_gather_ws_bf16": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp],
     "lffn_lookup_gather_plan": [_i64, _i64, _i64, _i64, ctypes.c_int32, ctypes.POINTER(ctypes.c_int32)],
     "lffn_indexed_inner_product_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "lffn_scatter_add_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],

@@ -50,6 +50,10 @@ struct LdsGatherArgs {
     int T, S, Do;
     int ntiles, nslices, per_xcd;
     int row_bytes;         // Do * element size
+    // Table split: a unit is (slice, part, tile); part p adds tables [p * part_tables, (p+1) * part_tables)
+    // and, when nparts > 1, writes its sums without bias and residual to part_out[p][B][Do].
+    int nparts, part_tables;
+    float *part_out;
 };
 
 // Copy this lane's four vectors of a table slice straight from global memory into
@@ -113,9 +117,13 @@ __global__ __launch_bounds__(WG) void lookup_gather_lds_kernel(LdsGatherArgs a) 
 
     const int xcd = blockIdx.x % XCDS;
     const int unit = xcd * a.per_xcd + blockIdx.x / XCDS;
-    if (unit >= a.ntiles * a.nslices) return;     // uniform over the workgroup
-    const int slice = unit / a.ntiles;
+    if (unit >= a.ntiles * a.nslices * a.nparts) return;     // uniform over the workgroup
+    const int slice = unit / (a.ntiles * a.nparts);
+    const int part = (unit / a.ntiles) % a.nparts;
     const int tile = unit % a.ntiles;
+    const int t_begin = part * a.part_tables;                  // a multiple of CHUNK
+    const int t_end = min(a.T, t_begin + a.part_tables);
+    const bool whole = a.nparts == 1;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -129,7 +137,7 @@ __global__ __launch_bounds__(WG) void lookup_gather_lds_kernel(LdsGatherArgs a) 
         float b[EPV];
 #pragma unroll
         for (int e = 0; e < EPV; ++e) b[e] = 0.f;
-        if (a.bias) {
+        if (a.bias && whole) {
             const float *bp = a.bias + (size_t)slice * (SEG_VECS * EPV) + j * EPV;
 #pragma unroll
             for (int e = 0; e < EPV; ++e) b[e] = bp[e];
@@ -146,7 +154,8 @@ __global__ __launch_bounds__(WG) void lookup_gather_lds_kernel(LdsGatherArgs a) 
 
     const CopyLanes cl = copy_lanes(a.row_bytes, tid);
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint4 *)lds;
-    copy_slice_to_lds<FULL>(slice_base, cl, tid, buf_vecs, lds0);
+    copy_slice_to_lds<FULL>(slice_base + (size_t)t_begin * table_bytes, cl, tid, buf_vecs,
+                            lds0 + (uint32_t)((t_begin & 1) * buf_vecs) * 16u);
     __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0): this lane's copies have landed in LDS
     __syncthreads();
 
@@ -157,7 +166,7 @@ __global__ __launch_bounds__(WG) void lookup_gather_lds_kernel(LdsGatherArgs a) 
     // OR of a half-word with the lane's base, a single SDWA or AND-OR instruction.
     constexpr int NQ = BF16 ? (NP + 3) / 4 : (NP + 1) / 2;
     const unsigned lds_base = lds0 + j * 16;
-    for (int t0 = 0; t0 < a.T; t0 += CHUNK) {
+    for (int t0 = t_begin; t0 < t_end; t0 += CHUNK) {
         // Lane j of a token group holds (code, score) of table t0 + j for each of
         // its NP tokens.  Addresses are clamped into range and the loads are
         // unconditional, so that all 2*NP of them are in flight together; what was
@@ -166,7 +175,7 @@ __global__ __launch_bounds__(WG) void lookup_gather_lds_kernel(LdsGatherArgs a) 
         float sc[NP];
         {
             const int tt = t0 + j;
-            const int ttc = min(tt, a.T - 1);
+            const int ttc = min(tt, t_end - 1);
             int craw[NP];
 #pragma unroll
             for (int p = 0; p < NP; ++p) {
@@ -178,7 +187,7 @@ __global__ __launch_bounds__(WG) void lookup_gather_lds_kernel(LdsGatherArgs a) 
             for (int q = 0; q < NQ; ++q) cd[q] = 0u;
 #pragma unroll
             for (int p = 0; p < NP; ++p) {
-                const bool ok = (tok0 + p * 64 < a.B) && (tt < a.T);
+                const bool ok = (tok0 + p * 64 < a.B) && (tt < t_end);
                 if constexpr (BF16)
                     cd[p / 4] |= unsigned(craw[p] & (a.S - 1)) << (8 * (p % 4));
                 else
@@ -194,7 +203,7 @@ __global__ __launch_bounds__(WG) void lookup_gather_lds_kernel(LdsGatherArgs a) 
 #pragma unroll
         for (int p = 0; p < NP; ++p) asm volatile("" : "+v"(sc[p]));
 
-        const int nt = min(CHUNK, a.T - t0);
+        const int nt = min(CHUNK, t_end - t0);
         // The 16 tables of the chunk, unrolled: table t0 + TT takes its codes and scores
         // from lane TT of each 16-lane token group with a DPP row broadcast (a vector-ALU
         // move), so that the only LDS traffic of the pass loop is the row reads.
@@ -205,7 +214,7 @@ __global__ __launch_bounds__(WG) void lookup_gather_lds_kernel(LdsGatherArgs a) 
                 // next table's slice goes straight into the other buffer, which was last
                 // read one table ago, before the previous barrier (the last iteration
                 // re-copies the last table: harmless)
-                copy_slice_to_lds<FULL>(slice_base + (size_t)min(t + 1, a.T - 1) * table_bytes, cl, tid, buf_vecs,
+                copy_slice_to_lds<FULL>(slice_base + (size_t)min(t + 1, t_end - 1) * table_bytes, cl, tid, buf_vecs,
                                         lds0 + (uint32_t)(((t + 1) & 1) * buf_vecs) * 16u);
                 const uint4 *buf = lds + (t & 1) * buf_vecs + j;
                 const unsigned buf_addr = lds_base + (unsigned)((t & 1) * buf_vecs) * 16u;
@@ -277,11 +286,11 @@ __global__ __launch_bounds__(WG) void lookup_gather_lds_kernel(LdsGatherArgs a) 
         const int64_t tok = tok0 + p * 64;
         if (tok < a.B) {
             const size_t off = tok * a.Do + (size_t)slice * (SEG_VECS * EPV) + j * EPV;
-            float *o = a.out + off;
+            float *o = (whole ? a.out : a.part_out + (size_t)part * a.B * a.Do) + off;
 #pragma unroll
             for (int q = 0; q < EPV / 4; ++q) {
                 float4 v = make_float4(acc[p][4 * q], acc[p][4 * q + 1], acc[p][4 * q + 2], acc[p][4 * q + 3]);
-                if (a.residual) {
+                if (a.residual && whole) {
                     const float4 rr = *reinterpret_cast<const float4 *>(a.residual + off + 4 * q);
                     v.x += rr.x; v.y += rr.y; v.z += rr.z; v.w += rr.w;
                 }
@@ -294,7 +303,7 @@ __global__ __launch_bounds__(WG) void lookup_gather_lds_kernel(LdsGatherArgs a) 
 template <bool BF16, int NP, bool FULL>
 int launch_lds_full(LdsGatherArgs a, hipStream_t stream) {
     a.ntiles = (int)((a.B + 64 * NP - 1) / (64 * NP));
-    const int units = a.ntiles * a.nslices;
+    const int units = a.ntiles * a.nslices * a.nparts;
     a.per_xcd = (units + XCDS - 1) / XCDS;
     const size_t lds_bytes = size_t(2) * a.S * SEG_VECS * 16;
     auto kern = lookup_gather_lds_kernel<BF16, NP, FULL>;
@@ -324,11 +333,13 @@ int launch_lds(const LdsGatherArgs &a, hipStream_t stream) {
 // table sets cost BIG times more).  The cheapest predicted time wins.
 struct GatherPlan {
     int kind, np;
+    double us;             // predicted time
 };
 
 template <bool BF16>
 GatherPlan plan_gather(int64_t B, int64_t T, int64_t S, int64_t Do) {
-    GatherPlan best{0, 0};
+    // token-major: every token reads its T rows from L2 / Infinity Cache, measured 9 TB/s
+    GatherPlan best{0, 0, double(B) * double(T) * double(Do) * (BF16 ? 2 : 4) / 9e6 + 5.0};
     if (S > MAX_S || T < 4 || B * T >= (int64_t(1) << 31)) return best;
     struct Option { int kind, np; double us_per_table; };
     static const Option f32_opts[] = {{1, 4, 1.15}, {1, 8, 1.18}, {1, 13, 1.30}, {1, 16, 1.60},
@@ -350,9 +361,66 @@ GatherPlan plan_gather(int64_t B, int64_t T, int64_t S, int64_t Do) {
         const int64_t tiles = (B + tok - 1) / tok;
         const int64_t rounds = (tiles * nslices + 255) / 256;
         const double us = double(rounds) * double(T) * o.us_per_table * (big ? (o.kind == 1 ? 1.3 : 1.15) : 1.0);
-        if (us < best_us) { best_us = us; best = GatherPlan{o.kind, o.np}; }
+        if (us < best_us) { best_us = us; best = GatherPlan{o.kind, o.np, us}; }
     }
     return best;
+}
+
+// Table split (needs a workspace): for a few thousand tokens there are too few (tile, slice) units
+// to fill the chip at the large tiles that make the staging pay, and the token-major kernel reads
+// every row from L2.  nparts workgroups share a unit, each adding a range of part_tables tables
+// (a multiple of the 16-table chunk) into its own partial output; a second kernel adds the
+// partials in a fixed order together with bias and residual.
+struct SplitPlan {
+    int np, nparts, part_tables;
+    double us;
+};
+
+template <bool BF16>
+SplitPlan plan_split(int64_t B, int64_t T, int64_t S, int64_t Do) {
+    SplitPlan best{0, 1, (int)T, 1e300};
+    const int cols = BF16 ? 128 : 64;
+    if (S > MAX_S || T < 32 || Do % cols != 0 || B < 256 || B * T >= (int64_t(1) << 31)) return best;
+    struct Option { int np; double us_per_table; };
+    static const Option f32_opts[] = {{4, 1.15}, {8, 1.18}, {13, 1.30}};
+    static const Option bf16_opts[] = {{4, 1.21}, {8, 1.32}};
+    const Option *opts = BF16 ? bf16_opts : f32_opts;
+    const int nopts = BF16 ? 2 : 3;
+    const int64_t nslices = Do / cols;
+    const bool big = double(T) * double(S) * double(Do) * (BF16 ? 2 : 4) > 200e6;
+    for (int k = 0; k < nopts; ++k) {
+        const int64_t tiles = (B + 64 * opts[k].np - 1) / (64 * opts[k].np);
+        for (int nparts = 2; nparts <= 16; nparts *= 2) {
+            const int64_t part_tables = ((T + nparts - 1) / nparts + CHUNK - 1) / CHUNK * CHUNK;
+            if (part_tables * (nparts - 1) >= T) continue;            // the last part would be empty
+            const int64_t units = tiles * nslices * nparts;
+            if (units > (int64_t(1) << 24)) continue;
+            const int64_t rounds = (units + 255) / 256;
+            // partials written and read once, the result written: about 4 TB/s for buffers of this size
+            const double reduce_us = double(2 * nparts + 1) * double(B) * double(Do) * 4.0 / 4e6 + 6.0;
+            const double us = double(rounds) * double(part_tables) * opts[k].us_per_table * (big ? 1.3 : 1.0) + reduce_us;
+            if (us < best.us) best = SplitPlan{opts[k].np, nparts, (int)part_tables, us};
+        }
+    }
+    return best;
+}
+
+__global__ __launch_bounds__(256) void gather_parts_reduce_kernel(const float *parts, int nparts, const float *bias,
+                                                                  const float *residual, float *out, int64_t B, int Do) {
+    const int64_t n4 = B * Do / 4;
+    const int q = Do / 4;
+    for (int64_t i = int64_t(blockIdx.x) * 256 + threadIdx.x; i < n4; i += int64_t(gridDim.x) * 256) {
+        float4 v = bias ? reinterpret_cast<const float4 *>(bias)[i % q] : make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int p = 0; p < nparts; ++p) {                       // parts in table order, as the one-part kernel adds them
+            const float4 t = reinterpret_cast<const float4 *>(parts)[(int64_t)p * n4 + i];
+            v.x += t.x; v.y += t.y; v.z += t.z; v.w += t.w;
+        }
+        if (residual) {
+            const float4 r = reinterpret_cast<const float4 *>(residual)[i];
+            v.x += r.x; v.y += r.y; v.z += r.z; v.w += r.w;
+        }
+        reinterpret_cast<float4 *>(out)[i] = v;
+    }
 }
 
 // Is (kind, np) a kernel that is built, and does the shape meet its preconditions?
@@ -371,7 +439,7 @@ bool plan_is_valid(const GatherPlan &p, int64_t B, int64_t T, int64_t S, int64_t
 template <bool BF16>
 int lookup_gather_entry(const int32_t *code, const float *score, const void *tables, const float *bias,
                         const float *residual, float *out, int64_t B, int64_t T, int64_t S, int64_t Do, int kind_req, int tokens_req,
-                        void *stream) {
+                        void *stream, void *workspace = nullptr, int64_t workspace_bytes = 0) {
     LFFN_REQUIRE(B >= 0 && T >= 0 && Do >= 1, LFFN_ERR_BAD_ARG);
     LFFN_REQUIRE(lffn_is_pow2(S) && S <= (1 << 24) && T * S <= 0x7fffffff, LFFN_ERR_UNSUPPORTED);
     LFFN_REQUIRE(Do % 64 == 0 && Do <= (1 << 20) && T <= (1 << 24), LFFN_ERR_UNSUPPORTED);
@@ -399,6 +467,32 @@ int lookup_gather_entry(const int32_t *code, const float *score, const void *tab
     GatherPlan plan;
     if (kind_req < 0) {
         plan = plan_gather<BF16>(B, T, S, Do);
+        if (workspace) {
+            const SplitPlan sp = plan_split<BF16>(B, T, S, Do);
+            if (sp.nparts > 1 && sp.us < 0.85 * plan.us && workspace_bytes >= int64_t(sp.nparts) * B * Do * 4) {
+                LFFN_REQUIRE(lffn_aligned16(workspace), LFFN_ERR_BAD_ARG);
+                LdsGatherArgs a{};
+                a.code = code; a.score = score; a.tables = static_cast<const char *>(tables); a.bias = nullptr;
+                a.residual = nullptr; a.out = out;
+                a.B = B; a.T = (int)T; a.S = (int)S; a.Do = (int)Do;
+                a.nslices = (int)(Do / (BF16 ? 128 : 64));
+                a.row_bytes = (int)(Do * (BF16 ? 2 : 4));
+                a.nparts = sp.nparts; a.part_tables = sp.part_tables; a.part_out = static_cast<float *>(workspace);
+                hipStream_t st = static_cast<hipStream_t>(stream);
+                int rc;
+                if constexpr (BF16) {
+                    rc = sp.np == 8 ? launch_lds<true, 8>(a, st) : launch_lds<true, 4>(a, st);
+                } else {
+                    rc = sp.np == 13 ? launch_lds<false, 13>(a, st)
+                                     : (sp.np == 8 ? launch_lds<false, 8>(a, st) : launch_lds<false, 4>(a, st));
+                }
+                if (rc != LFFN_OK) return rc;
+                const int64_t blocks = (B * Do / 4 + 255) / 256;
+                hipLaunchKernelGGL(gather_parts_reduce_kernel, dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256), 0, st,
+                                   a.part_out, sp.nparts, bias, residual, out, B, (int)Do);
+                return lffn_launch_status();
+            }
+        }
     } else {
         plan.kind = kind_req;
         const int per_np = kind_req == 1 ? 64 : 128;
@@ -416,6 +510,7 @@ int lookup_gather_entry(const int32_t *code, const float *score, const void *tab
     a.B = B; a.T = (int)T; a.S = (int)S; a.Do = (int)Do;
     a.nslices = (int)(Do / (BF16 ? 128 : 64));
     a.row_bytes = (int)(Do * (BF16 ? 2 : 4));
+    a.nparts = 1; a.part_tables = (int)T; a.part_out = nullptr;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if constexpr (BF16) {
         return np == 8 ? launch_lds<true, 8>(a, st) : launch_lds<true, 4>(a, st);
@@ -453,6 +548,36 @@ extern "C" int lffn_lookup_gather_residual_bf16(const int32_t *code, const float
                                                 const float *bias, const float *residual, float *out,
                                                 int64_t B, int64_t T, int64_t S, int64_t Do, void *stream) {
     return lookup_gather_entry<true>(code, score, tables, bias, residual, out, B, T, S, Do, -1, 0, stream);
+}
+
+extern "C" int lffn_lookup_gather_workspace_bytes(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t bf16,
+                                                  int64_t *bytes) {
+    LFFN_REQUIRE(bytes, LFFN_ERR_BAD_ARG);
+    *bytes = 0;
+    if (B < 1 || T < 1 || Do < 1 || !lffn_is_pow2(S) || Do % 64 != 0 || B * T >= (int64_t(1) << 31)) return LFFN_OK;
+    if (B >= 2 * 16384) return LFFN_OK;                        // taken in pieces, none of which is split
+    const GatherPlan plan = bf16 ? plan_gather<true>(B, T, S, Do) : plan_gather<false>(B, T, S, Do);
+    const SplitPlan sp = bf16 ? plan_split<true>(B, T, S, Do) : plan_split<false>(B, T, S, Do);
+    if (sp.nparts > 1 && sp.us < 0.85 * plan.us) *bytes = int64_t(sp.nparts) * B * Do * 4;
+    return LFFN_OK;
+}
+
+extern "C" int lffn_lookup_gather_ws_f32(const int32_t *code, const float *score, const float *tables,
+                                         const float *bias, const float *residual, float *out, void *workspace,
+                                         int64_t workspace_bytes, int64_t B, int64_t T, int64_t S, int64_t Do,
+                                         void *stream) {
+    LFFN_REQUIRE(workspace_bytes >= 0 && (workspace || workspace_bytes == 0), LFFN_ERR_BAD_ARG);
+    return lookup_gather_entry<false>(code, score, tables, bias, residual, out, B, T, S, Do, -1, 0, stream, workspace,
+                                      workspace_bytes);
+}
+
+extern "C" int lffn_lookup_gather_ws_bf16(const int32_t *code, const float *score, const uint16_t *tables,
+                                          const float *bias, const float *residual, float *out, void *workspace,
+                                          int64_t workspace_bytes, int64_t B, int64_t T, int64_t S, int64_t Do,
+                                          void *stream) {
+    LFFN_REQUIRE(workspace_bytes >= 0 && (workspace || workspace_bytes == 0), LFFN_ERR_BAD_ARG);
+    return lookup_gather_entry<true>(code, score, tables, bias, residual, out, B, T, S, Do, -1, 0, stream, workspace,
+                                     workspace_bytes);
 }
 
 extern "C" int lffn_lookup_gather_planned_f32(const int32_t *code, const float *score, const float *tables,

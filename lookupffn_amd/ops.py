@@ -628,15 +628,25 @@ def _lookup_gather_impl(code, score, tables, bias, residual=None):
         assert residual.dtype == torch.float32 and residual.is_contiguous() and tuple(residual.shape) == (B, Do)
     out = torch.empty(B, Do, dtype=torch.float32, device=tables.device)
     lib = _lib.load()
-    if tables.dtype == torch.float32:
-        fn, name = lib.lffn_lookup_gather_residual_f32, "lffn_lookup_gather_residual_f32"
-    elif tables.dtype == torch.bfloat16:
-        fn, name = lib.lffn_lookup_gather_residual_bf16, "lffn_lookup_gather_residual_bf16"
-    else:
+    if tables.dtype not in (torch.float32, torch.bfloat16):
         raise NotImplementedError(f"lookup_gather: table dtype {tables.dtype} (float32 and bfloat16 are built)")
+    bf16 = tables.dtype == torch.bfloat16
+    # a few thousand tokens: the table-split form, which wants a workspace for its partial outputs
+    ws_bytes = ctypes.c_int64(0)
+    _lib.check(lib.lffn_lookup_gather_workspace_bytes(B, T, S, Do, int(bf16), ctypes.byref(ws_bytes)),
+               "lffn_lookup_gather_workspace_bytes")
     with _dev_guard(tables):
-        rc = fn(_lib.ptr(code), _lib.ptr(score), _lib.ptr(tables), _lib.ptr(bias), _lib.ptr(residual), _lib.ptr(out),
-                B, T, S, Do, _lib.stream_of(tables))
+        if ws_bytes.value > 0:
+            fn, name = (lib.lffn_lookup_gather_ws_bf16, "lffn_lookup_gather_ws_bf16") if bf16 else \
+                (lib.lffn_lookup_gather_ws_f32, "lffn_lookup_gather_ws_f32")
+            ws = torch.empty(ws_bytes.value, dtype=torch.uint8, device=tables.device)
+            rc = fn(_lib.ptr(code), _lib.ptr(score), _lib.ptr(tables), _lib.ptr(bias), _lib.ptr(residual), _lib.ptr(out),
+                    _lib.ptr(ws), ws_bytes.value, B, T, S, Do, _lib.stream_of(tables))
+        else:
+            fn, name = (lib.lffn_lookup_gather_residual_bf16, "lffn_lookup_gather_residual_bf16") if bf16 else \
+                (lib.lffn_lookup_gather_residual_f32, "lffn_lookup_gather_residual_f32")
+            rc = fn(_lib.ptr(code), _lib.ptr(score), _lib.ptr(tables), _lib.ptr(bias), _lib.ptr(residual), _lib.ptr(out),
+                    B, T, S, Do, _lib.stream_of(tables))
     _lib.check(rc, f"{name}(B={B}, T={T}, S={S}, Do={Do})")
     return out
 

@@ -250,6 +250,27 @@ def lookup_gather(code, score, tables, bias=None, bf16=False, plan=None, residua
     return host(out)
 
 
+def lookup_gather_workspace_bytes(B, T, S, Do, bf16=False):
+    n = ctypes.c_int64(-1)
+    assert _lib.load().lffn_lookup_gather_workspace_bytes(B, T, S, Do, int(bf16), ctypes.byref(n)) == 0
+    return n.value
+
+
+def lookup_gather_ws(code, score, tables, bias=None, bf16=False, residual=None, ws_bytes=None):
+    """The workspace form; ws_bytes None = what lffn_lookup_gather_workspace_bytes asks for."""
+    cd, sd, td, bd = dev(code), dev(score), dev(tables), dev(bias)
+    rd = None if residual is None else dev(residual)
+    B, T = code.shape
+    _, S, Do = tables.shape
+    if ws_bytes is None:
+        ws_bytes = lookup_gather_workspace_bytes(B, T, S, Do, bf16)
+    ws = torch.full((max(ws_bytes, 16) // 4,), float("nan"), dtype=torch.float32, device=DEV)
+    out = torch.full((B, Do), float("nan"), dtype=torch.float32, device=DEV)
+    _call("lffn_lookup_gather_ws_bf16" if bf16 else "lffn_lookup_gather_ws_f32",
+          p(cd), p(sd), p(td), p(bd), p(rd), p(out), p(ws) if ws_bytes else None, ws_bytes, B, T, S, Do)
+    return host(out)
+
+
 def lookup_gather_plan(B, T, S, Do, bf16=False):
     import ctypes
     kind = ctypes.c_int32(-1)

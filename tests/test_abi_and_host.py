@@ -129,6 +129,10 @@ def test_argument_validation_of_the_backward_and_block_entry_points():
     assert lib.lffn_layer_norm_bwd_f32(P, P, 1e-5, P, P, P, P, 4, 770, 1, 8, None) == U       # H % 4
     assert lib.lffn_layer_norm_bwd_f32(P, P, 1e-5, P, P, P, None, 4, 768, 1, 8, None) == A    # partials: both or none
     assert lib.lffn_layer_norm_bwd_f32(P, P, 1e-5, P, P, P, P, 4, 768, 1, 0, None) == A
+    # gather with a workspace
+    assert lib.lffn_lookup_gather_workspace_bytes(2048, 128, 256, 768, 0, None) == A
+    assert lib.lffn_lookup_gather_ws_f32(P, P, P, None, None, P, None, 64, 4, 2, 16, 64, None) == A     # bytes without a workspace
+    assert lib.lffn_lookup_gather_ws_f32(P, P, P, None, None, P + 4, None, 0, 4, 2, 16, 64, None) == A
     # gather with residual
     assert lib.lffn_lookup_gather_residual_f32(P, P, P, None, P + 4, P, 4, 2, 16, 64, None) == A
 

@@ -676,6 +676,46 @@ def test_lookup_gather_takes_many_tokens_in_pieces(bf16):
     assert relmax(got, want + bias + res) <= 1e-5
 
 
+# (B, T, S, Do, bf16): shapes for which the workspace query asks for the table-split form (a few
+# thousand tokens, enough tables to split): 2, 4 and 8 parts, ragged token counts, table counts
+# that leave a short last part (200 = 64 + 64 + 64 + 8, 120 = 32 + 32 + 32 + 24, 200 = 112 + 88)
+SPLIT_SHAPES = [(2048, 128, 256, 768, False), (1024, 128, 256, 768, False), (2500, 96, 256, 768, False),
+                (2049, 200, 256, 768, False), (3000, 120, 64, 1024, False), (1500, 128, 64, 512, False),
+                (5000, 128, 256, 768, True), (5001, 200, 256, 1024, True)]
+
+
+@pytest.mark.parametrize("B,T,S,Do,bf16", SPLIT_SHAPES)
+def test_lookup_gather_table_split_matches_oracle(B, T, S, Do, bf16):
+    rng = np.random.RandomState(B + T + S + Do)
+    tables, code, idx, w = _rand_gather(rng, B, T, S, Do)
+    bias = (0.001 * rng.randn(Do)).astype(np.float32)
+    res = rng.randn(B, Do).astype(np.float32)
+    flat = tables.reshape(T * S, Do)
+    src = oracle.bf16_round(flat) if bf16 else flat
+    nbytes = cabi.lookup_gather_workspace_bytes(B, T, S, Do, bf16)
+    assert nbytes > 0 and nbytes % (B * Do * 4) == 0                     # the split form is asked for
+    got = cabi.lookup_gather_ws(code, w, src.reshape(T, S, Do), bias, bf16=bf16, residual=res)
+    assert not np.isnan(got).any()
+    sub = np.unique(np.concatenate([rng.choice(B, 128, replace=False), np.arange(B - 70, B), np.arange(0, 8)]))
+    w64 = w[sub].astype(np.float64)
+    want = oracle.gather_add_bf16(idx[sub], src, w64) if bf16 else oracle.gather_add(idx[sub], flat.astype(np.float64), w64)
+    assert relmax(got[sub], want + bias + res[sub]) <= 1e-5
+    # every token against the plain entry point (same rows, sums associated differently)
+    plain = cabi.lookup_gather(code, w, src.reshape(T, S, Do), bias, bf16=bf16, residual=res)
+    assert relmax(got, plain) <= 2e-6
+    assert np.array_equal(got, cabi.lookup_gather_ws(code, w, src.reshape(T, S, Do), bias, bf16=bf16, residual=res))
+    # without a workspace the entry point is the plain one
+    assert np.array_equal(cabi.lookup_gather_ws(code, w, src.reshape(T, S, Do), bias, bf16=bf16, residual=res, ws_bytes=0), plain)
+    # no bias, no residual
+    got_nb = cabi.lookup_gather_ws(code, w, src.reshape(T, S, Do), None, bf16=bf16)
+    assert relmax(got_nb[sub], want) <= 1e-5
+
+
+def test_lookup_gather_workspace_query_is_zero_where_the_plain_form_is_as_fast():
+    for shape in ((16384, 128, 256, 768), (65536, 128, 256, 768), (8, 128, 256, 768), (4096, 16, 256, 768), (0, 4, 16, 64)):
+        assert cabi.lookup_gather_workspace_bytes(*shape) == 0, shape
+
+
 @pytest.mark.parametrize("plan", F32_PLANS)
 @pytest.mark.parametrize("B,T,S,Do", LDS_SHAPES)
 def test_lookup_gather_lds_kernels_match_oracle(B, T, S, Do, plan):
