@@ -48,6 +48,11 @@ WORKLOADS = {
     "cfg2b64": dict(B=16384, H=768, T=128, S=256, Do=768, bf16=False, bs=64,
                     desc="config 2 shape with BH4 block size 64 (the reference's training config): 32x512 tokens, "
                          "d=768 padded to 1024, 4 stages of 16 blocks 64x64, 128 tables x 256 x 768 fp32"),
+    # the shape of the reference's own timing script (PL/compare.py:11-22: 64 x 512 tokens, hidden 512,
+    # 128 tables x 256, BH4 block size 64, output 512), which it runs beside a dense FFN 512 -> 2048 -> 512
+    "cmp512": dict(B=32768, H=512, T=128, S=256, Do=512, bf16=False, bs=64,
+                   desc="the reference's compare.py shape: 64x512 tokens, d=512, BH4 block size 64 (2 repeats x 4 stages "
+                        "of 8 blocks), 128 tables x 256 x 512 fp32"),
     # BASELINE.json configs[3]: the 12-layer encoder with every FFN a config-2 LookupFFN
     "cfg4": dict(B=16384, H=768, T=128, S=256, Do=768, bf16=False,
                  desc="config 4: 12-layer pre-norm RoBERTa-base encoder (hidden 768, 12 heads, seq 512, batch 32), "
@@ -536,6 +541,15 @@ def main():
                                     "cold": "1 GiB fill between launches (tables evicted from L2 and Infinity Cache)"},
         "launch": "HIP graph replay" if args.graph else "eager",
     }
+    if args.workload == "cmp512":
+        # the dense block the reference's script times beside the layer (PL/compare.py:40-45), same tokens,
+        # fp32 on the same GPU through PyTorch-ROCm
+        dense = torch.nn.Sequential(torch.nn.LayerNorm(H, eps=1e-5), torch.nn.Linear(H, 4 * H), torch.nn.GELU(),
+                                    torch.nn.Linear(4 * H, Do)).to(dev).eval()
+        with torch.no_grad():
+            res["dense_ffn_same_gpu"] = {"ms": timed(lambda: dense(x), 10), "dtype": "f32",
+                                         "what": f"LayerNorm + Linear({H},{4 * H}) + GELU + Linear({4 * H},{Do}), torch"}
+            res["dense_ffn_same_gpu"]["tokens_per_s"] = B / (res["dense_ffn_same_gpu"]["ms"] * 1e-3)
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(layer, x_cpu, wl)
     else:
