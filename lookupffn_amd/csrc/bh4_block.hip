@@ -41,7 +41,6 @@ namespace {
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int BS = 64;          // block size this file is built for
-constexpr int TOK = 32;         // tokens per workgroup
 constexpr int PAD = 4;          // floats of padding per LDS row
 
 // 64-point unnormalised Hadamard transform down the output index o of every block:
@@ -132,10 +131,15 @@ __device__ __forceinline__ float from_row_below(float v) {
     return __uint_as_float(__builtin_amdgcn_permlane16_swap(u, u, false, false)[0]);
 }
 
-template <int NB, bool HASH, int NH, bool BWD = false>
-__global__ __launch_bounds__(128 * (4 / NH)) void bh4_block_kernel(BlockArgs a) {
+// HV = 16-token halves per workgroup: 2 (32 tokens, one workgroup per CU at D = 1024) or 1 (16
+// tokens, half the LDS, so that two workgroups share a CU and the load, hand-over and hash phases
+// of one run under the products of the other).
+template <int NB, bool HASH, int NH, bool BWD = false, int HV = 2>
+__global__ __launch_bounds__(256 * HV / NH, HV == 1 ? 2 : 1) void bh4_block_kernel(BlockArgs a) {
     static_assert(!(HASH && BWD), "one form at a time");
-    constexpr int NWAVE = 4 * (2 / NH);
+    static_assert(NH <= HV, "a wavefront cannot hold more halves than the tile has");
+    constexpr int TOK = 16 * HV;                  // tokens per workgroup
+    constexpr int NWAVE = 4 * (HV / NH);
     const float *__restrict__ x = a.x;
     const float *__restrict__ wf = a.wf;
     const int64_t B = a.B;
@@ -571,16 +575,17 @@ __global__ __launch_bounds__(128 * (4 / NH)) void bh4_block_kernel(BlockArgs a) 
     }
 }
 
-template <int NB, bool HASH, int NH, bool BWD = false>
+template <int NB, bool HASH, int NH, bool BWD = false, int HV = 2>
 int launch_block(const BlockArgs &a, hipStream_t st) {
+    constexpr int TOK = 16 * HV;
     const size_t lds_bytes = (size_t(TOK) * (BS * NB + PAD) + 2 * TOK + (HASH ? 2 * BS * NB : 0)) * sizeof(float);
-    auto kern = bh4_block_kernel<NB, HASH, NH, BWD>;
+    auto kern = bh4_block_kernel<NB, HASH, NH, BWD, HV>;
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds_bytes) != hipSuccess) {
         (void)hipGetLastError();
         return LFFN_ERR_LAUNCH;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)((a.B + TOK - 1) / TOK)), dim3(128 * (4 / NH)), lds_bytes, st, a);
+    hipLaunchKernelGGL(kern, dim3((unsigned)((a.B + TOK - 1) / TOK)), dim3(256 * HV / NH), lds_bytes, st, a);
     return lffn_launch_status();
 }
 
@@ -603,8 +608,12 @@ int dispatch_block(const BlockArgs &a, int64_t D, hipStream_t st) {
         case 8: return launch_block<8, HASH, 2>(a, st);
         // measured at 16384 x 1024: the plain form 110 us with 4 wavefronts, 118 us with 8 (the
         // second fetch of the weight fragments costs more than the other phases gain); the hash
-        // form 141 us with 4, 133 us with 8 (LayerNorm and the hash are vector-ALU work)
-        default: return HASH ? launch_block<16, HASH, 1>(a, st) : launch_block<16, HASH, 2>(a, st);
+        // form 141 us with 4, 133 us with 8 (LayerNorm and the hash are vector-ALU work), 118 us
+        // (124 before: both with the later epilogue changes) as two 16-token workgroups per CU.
+        // A wavefront that holds one token half fetches 4 KB of weight fragments per 16 products:
+        // eight of them ask the compute unit's 64 bytes per clock of memory pipeline for 58, which
+        // is why desynchronising the phases gains no more than that.
+        default: return HASH ? launch_block<16, HASH, 1, false, 1>(a, st) : launch_block<16, HASH, 2>(a, st);
     }
 }
 
