@@ -8,7 +8,7 @@ registered: calling an op with CPU tensors fails in the dispatcher.  Fake
 """
 from __future__ import annotations
 
-from typing import Optional, Tuple
+from typing import Tuple
 
 import ctypes
 

@@ -272,7 +272,6 @@ def lookup_gather_ws(code, score, tables, bias=None, bf16=False, residual=None, 
 
 
 def lookup_gather_plan(B, T, S, Do, bf16=False):
-    import ctypes
     kind = ctypes.c_int32(-1)
     tokens = _lib.load().lffn_lookup_gather_plan(B, T, S, Do, int(bf16), ctypes.byref(kind))
     return kind.value, tokens

@@ -5,7 +5,6 @@ reference's parameter names, shapes and config attributes (PL/lookup.py:10-130).
 No kernel is launched here.
 """
 import ctypes
-import math
 import os
 import re
 from argparse import Namespace

@@ -3,7 +3,6 @@
 forward against the CPU oracle, gradients against the oracle's backward routines
 and against torch autograd of the reference's slow formulas.
 """
-import math
 from argparse import Namespace
 
 import numpy as np
