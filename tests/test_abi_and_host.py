@@ -143,6 +143,38 @@ def _config(**kw):
     return Namespace(**base)
 
 
+def test_workspace_queries_are_host_side_plans():
+    """The workspace sizes are decided on the host from the shape alone (no GPU needed): which
+    shapes take the table-split gather and the sorted scatter, and how much scratch they want."""
+    lib = _lib.load()
+
+    def gather_ws(B, T, S, Do, bf16=0):
+        n = ctypes.c_int64(-1)
+        assert lib.lffn_lookup_gather_workspace_bytes(B, T, S, Do, bf16, ctypes.byref(n)) == 0
+        return n.value
+
+    def scatter_ws(B, T, S, Do):
+        n = ctypes.c_int64(-1)
+        assert lib.lffn_lookup_scatter_workspace_bytes(B, T, S, Do, ctypes.byref(n)) == 0
+        return n.value
+
+    # RoBERTa-base tables: a few thousand tokens split the tables over 4 or 8 workgroups per unit
+    assert gather_ws(2048, 128, 256, 768) == 4 * 2048 * 768 * 4
+    assert gather_ws(1024, 128, 256, 768) == 8 * 1024 * 768 * 4
+    assert gather_ws(4096, 128, 256, 768) == 4 * 4096 * 768 * 4
+    # enough tokens to fill the chip without a split, too few tokens or tables for it to pay, bad shapes
+    for shape in ((16384, 128, 256, 768), (65536, 128, 256, 768), (256, 32, 256, 256), (4096, 16, 256, 768),
+                  (2048, 128, 512, 768), (2048, 128, 256, 100), (0, 128, 256, 768)):
+        assert gather_ws(*shape) == 0, shape
+    # sorted scatter: pairs + offsets + transposed codes and scores + packed gradient, for at most 16384 tokens
+    one = scatter_ws(16384, 128, 256, 768)
+    assert one >= 16384 * 128 * 8 + 16384 * 768 * 4
+    assert scatter_ws(1 << 20, 128, 256, 768) == one
+    assert scatter_ws(100, 128, 256, 768) < one
+    for shape in ((0, 4, 16, 64), (16, 0, 16, 64), (16, 4, 1024, 64), (16, 4, 16, 48)):
+        assert scatter_ws(*shape) == 0, shape
+
+
 def test_module_surface_matches_reference_names_and_shapes():
     m = lookupffn_amd.LookupFFN(_config(hidden_size=768, ffn_num_table=128, block_size=64), 768)
     sd = m.state_dict()
