@@ -331,9 +331,10 @@ class LookupFFN(nn.Module):
         added to the result inside the gather kernel: the encoder layer's "FFN(x) + x"."""
         shape = hidden_states.shape[:-1]
         dim = hidden_states.shape[-1]
-        hidden_states = hidden_states.reshape(int(np.prod(shape)), dim)
+        tokens = math.prod(shape)
+        hidden_states = hidden_states.reshape(tokens, dim)
         if residual is not None:
-            residual = residual.reshape(int(np.prod(shape)), self.output_size).float()
+            residual = residual.reshape(tokens, self.output_size).float()
         outputs = self._forward(hidden_states, residual)
         return outputs.reshape(*shape, self.output_size)
 
