@@ -341,13 +341,16 @@ def test_checkpoint_round_trip_and_folded_weight_cache(tmp_path):
         assert not torch.equal(b(x), out_a)
 
 
-def test_layer_forward_under_graph_capture():
-    """The eval forward (two kernels, outputs from torch's allocator) can be captured in a HIP
-    graph and replayed: every replay, with eager work and synchronisations in between, gives
-    the eager result for the inputs then in the static buffer."""
+# tokens: 256 takes the one-launch form of the layer, 1536 the projection kernel and the table-split
+# gather with its workspace, 4200 (at 16 tables) the projection kernel and the plain gather
+@pytest.mark.parametrize("tokens,tables,width", [(256, 32, 256), (1536, 128, 768), (4200, 16, 256)])
+def test_layer_forward_under_graph_capture(tokens, tables, width):
+    """The eval forward (outputs and workspaces from torch's allocator, no memset nodes) can be
+    captured in a HIP graph and replayed: every replay, with eager work and synchronisations in
+    between, gives the eager result for the inputs then in the static buffer."""
     torch.manual_seed(31)
-    layer = lookupffn_amd.LookupFFN(_config(hidden_size=256, ffn_num_table=32), 256).eval().to(DEV)
-    static_x = torch.randn(256, 256, device=DEV)
+    layer = lookupffn_amd.LookupFFN(_config(hidden_size=256, ffn_num_table=tables), width).eval().to(DEV)
+    static_x = torch.randn(tokens, 256, device=DEV)
     with torch.no_grad():
         for _ in range(3):                                 # warm-up on a side stream, as torch asks
             s = torch.cuda.Stream()
@@ -359,7 +362,7 @@ def test_layer_forward_under_graph_capture():
         with torch.cuda.graph(g):
             static_out = layer(static_x)
         for i in range(4):
-            x = torch.randn(256, 256, device=DEV)
+            x = torch.randn(tokens, 256, device=DEV)
             static_x.copy_(x)
             g.replay()
             torch.cuda.synchronize()
