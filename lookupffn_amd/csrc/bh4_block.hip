@@ -610,9 +610,9 @@ int dispatch_block(const BlockArgs &a, int64_t D, hipStream_t st) {
         // second fetch of the weight fragments costs more than the other phases gain); the hash
         // form 141 us with 4, 133 us with 8 (LayerNorm and the hash are vector-ALU work), 118 us
         // (124 before: both with the later epilogue changes) as two 16-token workgroups per CU.
-        // A wavefront that holds one token half fetches 4 KB of weight fragments per 16 products:
-        // eight of them ask the compute unit's 64 bytes per clock of memory pipeline for 58, which
-        // is why desynchronising the phases gains no more than that.
+        // Eight wavefronts that hold one token half each fetch 4 KB of weight fragments per 16
+        // products, 31 of the compute unit's 64 bytes per clock of memory pipeline; starting every
+        // other workgroup late so that the two on a compute unit run out of phase gained nothing.
         default: return HASH ? launch_block<16, HASH, 1, false, 1>(a, st) : launch_block<16, HASH, 2>(a, st);
     }
 }
