@@ -398,12 +398,9 @@ def main():
     block = layer.hash.projection.block_size != 1
 
     def hash_front():
-        # as LookupFFN._forward calls it: the kernel also reads the tables through once (cache warming)
-        # when they are small enough for the memory-side cache
-        warm = layer._warm_region()
         if block:        # one kernel: LayerNorm, BH4 on the matrix cores, mix + hash
-            return layer.hash.forward_block(x, layer_norm=layer.LayerNorm, warm=warm)
-        return layer.hash.forward_fused(x, layer_norm=layer.LayerNorm, warm=warm)
+            return layer.hash.forward_block(x, layer_norm=layer.LayerNorm)
+        return layer.hash.forward_fused(x, layer_norm=layer.LayerNorm)
 
     if args.two_kernels:
         type(layer).FUSED_LAYER_MAX_TOKENS = 0
@@ -541,8 +538,7 @@ def main():
         "gather_tokens_per_s": B / (gather_ms * 1e-3),
         "single_launch_median_ms": {"gather_warm": warm_gather, "gather_cold": cold_gather,
                                     "step_warm": warm_step, "step_cold": cold_step,
-                                    "cold": "1 GiB fill between launches (tables evicted from L2 and Infinity Cache)",
-                                    "tables_warmed_by_hash_kernel": (not fused_layer) and layer._warm_region() is not None},
+                                    "cold": "1 GiB fill between launches (tables evicted from L2 and Infinity Cache)"},
         "launch": "HIP graph replay" if args.graph else "eager",
     }
     if args.workload == "cmp512":

@@ -39,7 +39,7 @@ extern "C" {
 #define LFFN_ERR_UNSUPPORTED -2   /* a shape outside what the kernels are built for */
 #define LFFN_ERR_LAUNCH      -3   /* hipGetLastError() after the launch was not hipSuccess */
 
-#define LFFN_ABI_VERSION 3
+#define LFFN_ABI_VERSION 2
 
 /* ABI version of the loaded library (LFFN_ABI_VERSION at build time). */
 int lffn_version(void);
@@ -260,37 +260,6 @@ int lffn_ln_project_hash_f32(const float *x, const float *ln_weight, const float
                              float *z_out, int32_t *codes, float *scores,
                              int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
                              float decay, float residual, void *stream);
-
-/*
- * The two one-kernel hashing front ends with cache warming.  While it computes, the kernel also
- * reads [warm, warm + warm_bytes) once and discards it (global -> LDS copies into an area nobody
- * reads), which leaves that region in the memory-side cache for the kernel that follows.  The
- * layer passes its tables: the hashing kernels leave the memory system almost idle, and the
- * gather behind them then takes its table slices from the cache instead of from HBM even when
- * other layers ran since this one's last call.  Results are those of the entry points without
- * warming, bit for bit.  warm: 16-byte aligned or NULL; a wavefront reads at most 32 KiB, so a
- * small batch warms only part of a large region; a tail shorter than 1 KiB is not read.
- *
- * lffn_project_hash_warm_f32: lffn_project_hash_f32 (ln_weight == NULL) or
- * lffn_ln_project_hash_f32 (ln_weight, ln_bias given) with the two arguments added.
- * lffn_bh4_block_hash_warm_f32: lffn_ln_bh4_block_hash_f32 (z == stage_inputs == NULL;
- * ln_weight optional) or lffn_bh4_block_hash_train_f32 (z and, for J > 1, stage_inputs given,
- * ln_weight == NULL); T >= 1.
- * The reference has no counterpart of the warming itself (its gather, PL/gather/kernel.py:11-25,
- * reads table rows from wherever they are); the entry points replace what the ones they extend
- * replace.
- */
-int lffn_project_hash_warm_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
-                               const float *diag, const float *proj_bias,
-                               float *z_out, int32_t *codes, float *scores,
-                               int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
-                               float decay, float residual, const void *warm, int64_t warm_bytes,
-                               void *stream);
-int lffn_bh4_block_hash_warm_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
-                                 const float *w_folded, const float *proj_bias, int32_t *codes, float *scores,
-                                 float *z, float *stage_inputs, int64_t B, int64_t H, int64_t D, int64_t R,
-                                 int64_t J, int64_t T, int64_t block_size, float decay, float residual,
-                                 const void *warm, int64_t warm_bytes, void *stream);
 
 /* ---------------------------------------------------------------- code + score */
 

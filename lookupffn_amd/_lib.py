@@ -15,7 +15,7 @@ _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 # LOOKUPFFN_HIP_LIB points at another build of the same ABI (e.g. a tuning build)
 LIB_PATH = os.environ.get("LOOKUPFFN_HIP_LIB") or os.path.join(_PKG_DIR, "liblookupffn_hip.so")
 
-ABI_VERSION = 3
+ABI_VERSION = 2
 
 LFFN_OK = 0
 LFFN_ERR_BAD_ARG = -1
@@ -52,10 +52,6 @@ SIGNATURES = {
     "lffn_project_hash_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _vp],
     "lffn_ln_project_hash_f32": [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _vp,
                                  _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _vp],
-    "lffn_project_hash_warm_f32": [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _vp,
-                                   _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _vp, _i64, _vp],
-    "lffn_bh4_block_hash_warm_f32": [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _vp, _vp,
-                                     _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _vp, _i64, _vp],
     "lffn_code_score_f32": [_vp, _vp, _vp, _i64, _i64, _vp],
     "lffn_code_score_bwd_f32": [_vp, _vp, _vp, _i64, _i64, _vp],
     "lffn_gather_add_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],

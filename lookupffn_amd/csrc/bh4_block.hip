@@ -108,8 +108,6 @@ struct BlockArgs {
     int64_t B;
     int H, R, J, T;
     float decay, residual;
-    const char *warm;      // hash form: a region read once and discarded while the kernel computes, or null
-    int64_t warm_bytes;
 };
 
 // NH = token halves per wavefront.  NH == 2: 4 wavefronts, each both 16-token halves (a weight
@@ -555,13 +553,6 @@ __global__ __launch_bounds__(256 * HV / NH, HV == 1 ? 2 : 1) void bh4_block_kern
                         }
                     }
                 }
-                // Cache warming goes behind the last load of the kernel (loads return in order, so a
-                // load issued after these copies would wait for them): what follows is LDS and stores.
-                if (a.warm && r == R - 1) {                    // uniform
-                    __shared__ uint4 sink[64];
-                    const int64_t w = int64_t(blockIdx.x) * NWAVE + __builtin_amdgcn_readfirstlane(wave);
-                    cache_warm(a.warm, a.warm_bytes, w, int64_t(gridDim.x) * NWAVE, sink, lane);
-                }
                 __syncthreads();
                 // every wavefront writes the D/8 codes and scores of TOK/NWAVE tokens
 #pragma unroll 1
@@ -582,7 +573,6 @@ __global__ __launch_bounds__(256 * HV / NH, HV == 1 ? 2 : 1) void bh4_block_kern
             }
         }
     }
-    if constexpr (HASH) cache_warm_drain();
 }
 
 template <int NB, bool HASH, int NH, bool BWD = false, int HV = 2>
@@ -710,34 +700,6 @@ extern "C" int lffn_bh4_block_hash_train_f32(const float *x, const float *w_fold
     a.x = x; a.wf = w_folded; a.pbias = proj_bias; a.codes = codes; a.scores = scores; a.z_out = z;
     a.stage_save = stage_inputs; a.B = B; a.H = (int)H; a.R = (int)R; a.J = (int)J; a.T = (int)T;
     a.decay = decay; a.residual = residual;
-    return dispatch_block<true>(a, D, static_cast<hipStream_t>(stream));
-}
-
-extern "C" int lffn_bh4_block_hash_warm_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
-                                            const float *w_folded, const float *proj_bias, int32_t *codes,
-                                            float *scores, float *z, float *stage_inputs, int64_t B, int64_t H,
-                                            int64_t D, int64_t R, int64_t J, int64_t T, int64_t block_size,
-                                            float decay, float residual, const void *warm, int64_t warm_bytes,
-                                            void *stream) {
-    LFFN_REQUIRE(B >= 0 && R >= 1 && J >= 1 && D >= 1 && H >= 1 && H <= D && T >= 1, LFFN_ERR_BAD_ARG);
-    LFFN_REQUIRE(H % 4 == 0 && J <= 64, LFFN_ERR_UNSUPPORTED);
-    LFFN_REQUIRE(block_size == BS && lffn_is_pow2(D) && D >= BS && D <= 1024, LFFN_ERR_UNSUPPORTED);
-    LFFN_REQUIRE(R <= 4096 && B <= (int64_t(1) << 31) - 1 && T <= (1 << 24), LFFN_ERR_UNSUPPORTED);
-    LFFN_REQUIRE(T * 8 <= R * D, LFFN_ERR_BAD_ARG);
-    LFFN_REQUIRE(!ln_weight || (ln_bias && ln_eps >= 0.f), LFFN_ERR_BAD_ARG);
-    LFFN_REQUIRE(warm_bytes >= 0 && (warm || warm_bytes == 0) && lffn_aligned16(warm), LFFN_ERR_BAD_ARG);
-    if (B == 0) return LFFN_OK;
-    LFFN_REQUIRE(x && w_folded && codes && scores, LFFN_ERR_BAD_ARG);
-    LFFN_REQUIRE(lffn_aligned16(x) && lffn_aligned16(w_folded) && (!proj_bias || lffn_aligned16(proj_bias)) &&
-                     (!ln_weight || (lffn_aligned16(ln_weight) && lffn_aligned16(ln_bias))) &&
-                     (!z || lffn_aligned16(z)) && (!stage_inputs || lffn_aligned16(stage_inputs)),
-                 LFFN_ERR_BAD_ARG);
-    BlockArgs a{};
-    a.x = x; a.ln_w = ln_weight; a.ln_b = ln_bias; a.ln_eps = ln_eps; a.wf = w_folded; a.pbias = proj_bias;
-    a.codes = codes; a.scores = scores; a.z_out = z; a.stage_save = stage_inputs;
-    a.B = B; a.H = (int)H; a.R = (int)R; a.J = (int)J; a.T = (int)T;
-    a.decay = decay; a.residual = residual;
-    if (warm_bytes) { a.warm = static_cast<const char *>(warm); a.warm_bytes = warm_bytes; }
     return dispatch_block<true>(a, D, static_cast<hipStream_t>(stream));
 }
 

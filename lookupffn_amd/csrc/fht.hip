@@ -158,9 +158,6 @@ struct ProjectArgs {
     const float *gres;    // [B, Do] or null: added to the result
     float *gout;          // [B, Do]
     int S, Do;
-    // hash form only: a region read once and discarded while the kernel computes, or null
-    const char *warm;
-    int64_t warm_bytes;
 };
 
 constexpr int FUSED_MAX_T = 512;   // (code, score) pairs a wavefront keeps in LDS for its token
@@ -255,29 +252,6 @@ __global__ __launch_bounds__(256) void project_kernel(ProjectArgs a) {
             fht_rows<LOGD>(v, lr);
         }
 
-        // the bias of this repeat's columns
-        float4 bb[NJ];
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-            const int col = r * D + 256 * j + 4 * lr;
-            bb[j] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (a.mix && a.pbias && col < a.out_cols) bb[j] = *reinterpret_cast<const float4 *>(a.pbias + col);
-        }
-        if constexpr (HASH && !GATHER) {
-            // Cache warming goes here, behind the wavefront's last load: loads return in order
-            // and the compiler's waits count only its own loads, so any load still in flight
-            // or issued later would end up waiting for these copies; the epilogue below is
-            // arithmetic and stores.
-            if (a.warm && r == a.R - 1) {                           // uniform
-#pragma unroll
-                for (int j = 0; j < NJ; ++j)
-                    asm volatile("" : "+v"(bb[j].x), "+v"(bb[j].y), "+v"(bb[j].z), "+v"(bb[j].w));   // the bias has landed
-                __shared__ uint4 sink[64];
-                const int64_t w = int64_t(blockIdx.x) * 4 + __builtin_amdgcn_readfirstlane(wave);
-                cache_warm(a.warm, a.warm_bytes, w, int64_t(gridDim.x) * 4, sink, lane);
-            }
-        }
-
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
             const int e0 = 256 * j + 4 * lr;
@@ -294,7 +268,8 @@ __global__ __launch_bounds__(256) void project_kernel(ProjectArgs a) {
                     z[c] = m0 + m1;
                 }
                 if (a.pbias && in_cols) {
-                    z[0] = z[0] + bb[j].x; z[1] = z[1] + bb[j].y; z[2] = z[2] + bb[j].z; z[3] = z[3] + bb[j].w;
+                    const float4 bb = *reinterpret_cast<const float4 *>(a.pbias + col);
+                    z[0] = z[0] + bb.x; z[1] = z[1] + bb.y; z[2] = z[2] + bb.z; z[3] = z[3] + bb.w;
                 }
             }
             if (a.out && live && in_cols)
@@ -390,7 +365,6 @@ __global__ __launch_bounds__(256) void project_kernel(ProjectArgs a) {
             }
         }
     }
-    if constexpr (HASH && !GATHER) cache_warm_drain();
 }
 
 template <bool HASH>
@@ -714,7 +688,7 @@ static int project_hash_impl(const float *x, const float *ln_w, const float *ln_
                              const float *diag, const float *proj_bias,
                              float *z_out, int32_t *codes, float *scores,
                              int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
-                             float decay, float residual, const void *warm, int64_t warm_bytes, void *stream);
+                             float decay, float residual, void *stream);
 
 extern "C" int lffn_ln_project_hash_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
                                         const float *diag, const float *proj_bias,
@@ -723,7 +697,7 @@ extern "C" int lffn_ln_project_hash_f32(const float *x, const float *ln_weight, 
                                         float decay, float residual, void *stream) {
     LFFN_REQUIRE(ln_weight && ln_bias && ln_eps >= 0.f, LFFN_ERR_BAD_ARG);
     return project_hash_impl(x, ln_weight, ln_bias, ln_eps, diag, proj_bias, z_out, codes, scores,
-                             B, H, D, R, J, T, decay, residual, nullptr, 0, stream);
+                             B, H, D, R, J, T, decay, residual, stream);
 }
 
 extern "C" int lffn_project_hash_f32(const float *x, const float *diag, const float *proj_bias,
@@ -731,26 +705,14 @@ extern "C" int lffn_project_hash_f32(const float *x, const float *diag, const fl
                                      int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
                                      float decay, float residual, void *stream) {
     return project_hash_impl(x, nullptr, nullptr, 0.f, diag, proj_bias, z_out, codes, scores,
-                             B, H, D, R, J, T, decay, residual, nullptr, 0, stream);
-}
-
-extern "C" int lffn_project_hash_warm_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
-                                          const float *diag, const float *proj_bias,
-                                          float *z_out, int32_t *codes, float *scores,
-                                          int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
-                                          float decay, float residual, const void *warm, int64_t warm_bytes,
-                                          void *stream) {
-    LFFN_REQUIRE((ln_weight != nullptr) == (ln_bias != nullptr) && ln_eps >= 0.f, LFFN_ERR_BAD_ARG);
-    LFFN_REQUIRE(warm_bytes >= 0 && (warm || warm_bytes == 0) && lffn_aligned16(warm), LFFN_ERR_BAD_ARG);
-    return project_hash_impl(x, ln_weight, ln_bias, ln_eps, diag, proj_bias, z_out, codes, scores,
-                             B, H, D, R, J, T, decay, residual, warm_bytes ? warm : nullptr, warm_bytes, stream);
+                             B, H, D, R, J, T, decay, residual, stream);
 }
 
 static int project_hash_impl(const float *x, const float *ln_w, const float *ln_b, float ln_eps,
                              const float *diag, const float *proj_bias,
                              float *z_out, int32_t *codes, float *scores,
                              int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
-                             float decay, float residual, const void *warm, int64_t warm_bytes, void *stream) {
+                             float decay, float residual, void *stream) {
     LFFN_REQUIRE(x && diag && codes && scores, LFFN_ERR_BAD_ARG);
     int rc = check_dims(B, H, D, R, J);
     if (rc != LFFN_OK) return rc;
@@ -766,7 +728,6 @@ static int project_hash_impl(const float *x, const float *ln_w, const float *ln_
     a.out_stride = (int)(T * 8); a.out_cols = (int)(T * 8); a.T = (int)T;
     a.decay = decay; a.residual = residual; a.mix = 1;
     a.vec_in = (lffn_aligned16(x) && H % 4 == 0) ? 1 : 0;
-    a.warm = static_cast<const char *>(warm); a.warm_bytes = warm_bytes;
     return launch_project<true>(a, lffn_log2(D), static_cast<hipStream_t>(stream));
 }
 

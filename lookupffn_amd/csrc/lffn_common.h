@@ -146,30 +146,5 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
-// Cache warming.  A kernel that leaves the memory system idle can pull a region another kernel
-// will want (the layer's tables) through L2 into the memory-side cache while it computes: this
-// wavefront reads KiB number first_kib, first_kib + stride_kib, ... of [base, base + bytes), at
-// most WARM_MAX_KIB of them, with global -> LDS copies (16 bytes per lane) into `sink`, 1 KiB of
-// LDS nobody reads.  No register is written, so nothing has to stay live while the copies fly;
-// loads return in order, so the wavefront's next ordinary load waits for them too.  The caller
-// must run cache_warm_drain() before the workgroup ends: a copy still in flight would land
-// in LDS that may by then belong to another workgroup.  A tail shorter than 1 KiB is not read.
-constexpr int WARM_MAX_KIB = 32;
-__device__ __forceinline__ void cache_warm(const char *base, int64_t bytes, int64_t first_kib, int64_t stride_kib,
-                                           void *sink, int lane) {
-    const uint32_t sink_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)sink;
-    const uint32_t off = (uint32_t)lane * 16u;
-    const int64_t n_kib = bytes >> 10;
-    int64_t kib = first_kib;
-    for (int i = 0; i < WARM_MAX_KIB && kib < n_kib; ++i, kib += stride_kib) {
-        const char *p = base + (kib << 10);
-        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                     :
-                     : "v"(off), "s"(p), "s"(sink_addr)
-                     : "memory");
-    }
-}
-__device__ __forceinline__ void cache_warm_drain() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0)
-
 __device__ __forceinline__ float bf16_lo(uint32_t packed) { return __uint_as_float(packed << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t packed) { return __uint_as_float(packed & 0xFFFF0000u); }

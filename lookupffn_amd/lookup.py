@@ -72,11 +72,11 @@ class ProjectHash(torch.autograd.Function):
     (PL/lookup.py:29-39, PL/compute_code_score/kernel.py:47-53); the code has no gradient."""
 
     @staticmethod
-    def forward(ctx, x, weight, bias, T, decay, warm=None):
+    def forward(ctx, x, weight, bias, T, decay):
         R, J = weight.shape[0], weight.shape[1]
         diag = weight.reshape(R, J, -1).contiguous()
         x = x.contiguous()
-        code, score, z = ops.project_hash(x, diag, bias, T, float(decay), float(1 - decay), True, warm)
+        code, score, z = ops.project_hash(x, diag, bias, T, float(decay), float(1 - decay), True)
         ctx.save_for_backward(x, diag, z)
         ctx.weight_shape = weight.shape
         ctx.has_bias = bias is not None
@@ -90,7 +90,7 @@ class ProjectHash(torch.autograd.Function):
         g_x, g_diag, g_bias = ops.project_hash_bwd(x, diag, z, g_score.contiguous(), ctx.decay, 1 - ctx.decay)
         return (g_x if ctx.needs_input_grad[0] else None,
                 g_diag.reshape(ctx.weight_shape) if ctx.needs_input_grad[1] else None,
-                g_bias if (ctx.has_bias and ctx.needs_input_grad[2]) else None, None, None, None)
+                g_bias if (ctx.has_bias and ctx.needs_input_grad[2]) else None, None, None)
 
 
 class BlockProjectHash(torch.autograd.Function):
@@ -103,11 +103,11 @@ class BlockProjectHash(torch.autograd.Function):
     autograd (PL/bh4/kernel.py:23-36, PL/lookup.py:29-39)."""
 
     @staticmethod
-    def forward(ctx, x, weight, bias, T, decay, warm=None):
+    def forward(ctx, x, weight, bias, T, decay):
         x = x.contiguous()
         w = weight.contiguous()
         folded = ops.bh4_fold_mode(w, 0)
-        code, score, z, stage_in = ops.bh4_block_hash_train(x, folded, bias, T, float(decay), float(1 - decay), warm)
+        code, score, z, stage_in = ops.bh4_block_hash_train(x, folded, bias, T, float(decay), float(1 - decay))
         ctx.save_for_backward(x, w, z, stage_in)
         ctx.has_bias = bias is not None
         ctx.decay = float(decay)
@@ -129,7 +129,7 @@ class BlockProjectHash(torch.autograd.Function):
             g_w = ops.bh4_fold_mode(g_folded, 2)
         g_x = g_x[0] if R == 1 else g_x.sum(0)
         g_bias = g_z.sum(0) if (ctx.has_bias and ctx.needs_input_grad[2]) else None
-        return (g_x if ctx.needs_input_grad[0] else None, g_w, g_bias, None, None, None)
+        return (g_x if ctx.needs_input_grad[0] else None, g_w, g_bias, None, None)
 
 
 class Hashing(nn.Module):
@@ -158,19 +158,18 @@ class Hashing(nn.Module):
                 and p.padded_in_dim <= 1024 and p.padded_in_dim >= 8
                 and x.dtype == torch.float32 and x.is_cuda and not needs_grad)
 
-    def forward_fused(self, x, layer_norm=None, warm=None):
-        """One kernel: (LayerNorm ->) diagonal BH4 -> mix -> bias -> code + score.  ``warm``: a tensor
-        the kernel reads through once while it computes (the tables the gather is about to use)."""
+    def forward_fused(self, x, layer_norm=None):
+        """One kernel: (LayerNorm ->) diagonal BH4 -> mix -> bias -> code + score."""
         p = self.projection
         diag = p.weight.reshape(p.num_repeat, p.weight.shape[1], p.padded_in_dim).contiguous()
         if layer_norm is not None:
             code, score, _ = ops.ln_project_hash(
                 x.contiguous(), layer_norm.weight, layer_norm.bias, float(layer_norm.eps), diag, p.bias,
-                self.num_table, float(p.decay_coeff), float(1 - p.decay_coeff), False, warm)
+                self.num_table, float(p.decay_coeff), float(1 - p.decay_coeff), False)
         else:
             code, score, _ = ops.project_hash(
                 x.contiguous(), diag, p.bias, self.num_table,
-                float(p.decay_coeff), float(1 - p.decay_coeff), False, warm)
+                float(p.decay_coeff), float(1 - p.decay_coeff), False)
         return code, score
 
     def can_fuse_block(self, x):
@@ -194,7 +193,7 @@ class Hashing(nn.Module):
             self._folded = cached
         return cached[1]
 
-    def forward_block(self, x, layer_norm=None, warm=None):
+    def forward_block(self, x, layer_norm=None):
         """8-bit codes: one kernel, (LayerNorm ->) BH4 on the matrix cores -> mix -> bias ->
         code + score.  Other code lengths: the BH4 kernel, then mix + hash in a second one."""
         p = self.projection
@@ -204,7 +203,7 @@ class Hashing(nn.Module):
             lb = None if layer_norm is None else layer_norm.bias
             eps = 0.0 if layer_norm is None else float(layer_norm.eps)
             return ops.ln_bh4_block_hash(x, lw, lb, eps, self.folded_weight(), p.bias, self.num_table,
-                                         float(p.decay_coeff), float(1 - p.decay_coeff), warm)
+                                         float(p.decay_coeff), float(1 - p.decay_coeff))
         if layer_norm is not None:
             x = layer_norm(x)
         y = ops.bh4_block(x, self.folded_weight())
@@ -226,20 +225,18 @@ class Hashing(nn.Module):
                 and 64 <= p.padded_in_dim <= 1024 and p.in_dim % 4 == 0
                 and x.dtype == torch.float32 and x.is_cuda and p.weight.dtype == torch.float32)
 
-    def forward(self, x, warm=None):
-        """PL/lookup.py:57-62.  ``warm`` (not in the reference): see forward_fused; the forms that
-        are not one kernel ignore it."""
+    def forward(self, x):
         B, D = x.shape
         if self.can_fuse(x):                      # no gradient needed: the inference kernels
-            return self.forward_fused(x, warm=warm)
+            return self.forward_fused(x)
         if self.can_fuse_block(x):
-            return self.forward_block(x, warm=warm)
+            return self.forward_block(x)
         if self.can_fuse_training(x):
             p = self.projection
-            return ProjectHash.apply(x, p.weight, p.bias, self.num_table, p.decay_coeff, warm)
+            return ProjectHash.apply(x, p.weight, p.bias, self.num_table, p.decay_coeff)
         if self.can_fuse_block_training(x):
             p = self.projection
-            return BlockProjectHash.apply(x, p.weight, p.bias, self.num_table, p.decay_coeff, warm)
+            return BlockProjectHash.apply(x, p.weight, p.bias, self.num_table, p.decay_coeff)
         z = self.projection(x)
         z = z.reshape(B, self.num_table, self.code_length)
         code, score = compute_code_score(z, training=self.training)
@@ -297,19 +294,6 @@ class LookupFFN(nn.Module):
                 and self.output_size % 4 == 0 and self.tables.dtype == torch.float32
                 and self.bias.dtype == torch.float32)
 
-    # Tables up to this size are read through once by the hashing kernel, which leaves the memory
-    # system idle, so that the gather behind it finds them in the 256 MB memory-side cache even
-    # when other layers ran in between (measured at 16384 tokens, 128 x 256 x 768 fp32 tables,
-    # caches flushed before the layer: 353 -> 264 us; tables already cached: +2 us).
-    WARM_TABLES_MAX_BYTES = 192 << 20
-
-    def _warm_region(self):
-        t = self.tables
-        if (t.is_cuda and t.is_contiguous() and t.dtype in (torch.float32, torch.bfloat16)
-                and self.output_size % 64 == 0 and 0 < t.numel() * t.element_size() <= self.WARM_TABLES_MAX_BYTES):
-            return t.detach()
-        return None
-
     def _forward(self, hidden_states, residual=None):
         ln = self.LayerNorm
         ln_fusable = (ln.elementwise_affine and ln.weight is not None and ln.bias is not None
@@ -324,9 +308,9 @@ class LookupFFN(nn.Module):
                                         float(p.decay_coeff), float(1 - p.decay_coeff))
         if ln_fusable and self.hash.can_fuse(hidden_states):
             # inference: LayerNorm runs inside the projection kernel
-            code, score = self.hash.forward_fused(hidden_states, layer_norm=ln, warm=self._warm_region())
+            code, score = self.hash.forward_fused(hidden_states, layer_norm=ln)
         elif ln_fusable and self.hash.can_fuse_block(hidden_states):
-            code, score = self.hash.forward_block(hidden_states, layer_norm=ln, warm=self._warm_region())
+            code, score = self.hash.forward_block(hidden_states, layer_norm=ln)
         else:
             if (torch.is_grad_enabled() and hidden_states.is_cuda and hidden_states.dtype == torch.float32
                     and ln.elementwise_affine and ln.weight is not None and ln.bias is not None
@@ -334,7 +318,7 @@ class LookupFFN(nn.Module):
                 hidden_states = LayerNormFn.apply(hidden_states.contiguous(), ln.weight, ln.bias, ln.eps)
             else:
                 hidden_states = ln(hidden_states)
-            code, score = self.hash(hidden_states, warm=self._warm_region())
+            code, score = self.hash(hidden_states)
         if self.output_size % 64 == 0 and self.tables.dtype in (torch.float32, torch.bfloat16):
             # table-local codes, offset and bias folded into the gather kernel
             return lookup_gather(code, score.float(), self.tables, self.bias.float(), residual)

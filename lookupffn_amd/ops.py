@@ -138,20 +138,11 @@ def _(x, w_folded):
 
 # ----------------------------------------------------------------------------- ln_bh4_block_hash
 
-def _warm_args(warm, like):
-    """(pointer, bytes) of the region a hashing kernel reads once while it computes, so that the
-    kernel after it (the gather over the tables) finds it in the memory-side cache."""
-    if warm is None or warm.numel() == 0:
-        return None, 0
-    assert warm.is_cuda and warm.device == like.device and warm.is_contiguous()
-    return warm.data_ptr(), warm.numel() * warm.element_size()
-
-
 _L.define("ln_bh4_block_hash(Tensor x, Tensor? ln_weight, Tensor? ln_bias, float ln_eps, Tensor w_folded, "
-          "Tensor? bias, int T, float decay, float residual, Tensor? warm=None) -> (Tensor, Tensor)")
+          "Tensor? bias, int T, float decay, float residual) -> (Tensor, Tensor)")
 
 
-def _ln_bh4_block_hash_impl(x, ln_weight, ln_bias, ln_eps, w_folded, bias, T, decay, residual, warm=None):
+def _ln_bh4_block_hash_impl(x, ln_weight, ln_bias, ln_eps, w_folded, bias, T, decay, residual):
     _lib.require_gpu(x, ln_weight, ln_bias, w_folded, bias)
     assert x.dim() == 2 and w_folded.dim() == 5
     assert x.dtype == torch.float32 and w_folded.dtype == torch.float32
@@ -168,15 +159,11 @@ def _ln_bh4_block_hash_impl(x, ln_weight, ln_bias, ln_eps, w_folded, bias, T, de
         assert bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == T * 8
     codes = torch.empty(B, T, dtype=torch.int32, device=x.device)
     scores = torch.empty(B, T, dtype=torch.float32, device=x.device)
-    if B == 0 or T == 0:
-        return codes, scores
-    wp, wb = _warm_args(warm, x)
     with _dev_guard(x):
-        rc = _lib.load().lffn_bh4_block_hash_warm_f32(
+        rc = _lib.load().lffn_ln_bh4_block_hash_f32(
             _lib.ptr(x), _lib.ptr(ln_weight), _lib.ptr(ln_bias), ln_eps, _lib.ptr(w_folded), _lib.ptr(bias),
-            _lib.ptr(codes), _lib.ptr(scores), None, None, B, H, D, R, J, T, bs, decay, residual, wp, wb,
-            _lib.stream_of(x))
-    _lib.check(rc, f"lffn_bh4_block_hash_warm_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T}, block_size={bs})")
+            _lib.ptr(codes), _lib.ptr(scores), B, H, D, R, J, T, bs, decay, residual, _lib.stream_of(x))
+    _lib.check(rc, f"lffn_ln_bh4_block_hash_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T}, block_size={bs})")
     return codes, scores
 
 
@@ -184,7 +171,7 @@ _L.impl("ln_bh4_block_hash", _ln_bh4_block_hash_impl, "CUDA")
 
 
 @torch.library.register_fake("lookupffn::ln_bh4_block_hash")
-def _(x, ln_weight, ln_bias, ln_eps, w_folded, bias, T, decay, residual, warm=None):
+def _(x, ln_weight, ln_bias, ln_eps, w_folded, bias, T, decay, residual):
     return (torch.empty(x.shape[0], T, dtype=torch.int32, device=x.device),
             torch.empty(x.shape[0], T, dtype=torch.float32, device=x.device))
 
@@ -216,11 +203,11 @@ def _(w, mode):
     return torch.empty_like(w)
 
 
-_L.define("bh4_block_hash_train(Tensor x, Tensor w_folded, Tensor? bias, int T, float decay, float residual, "
-          "Tensor? warm=None) -> (Tensor, Tensor, Tensor, Tensor)")
+_L.define("bh4_block_hash_train(Tensor x, Tensor w_folded, Tensor? bias, int T, float decay, float residual)"
+          " -> (Tensor, Tensor, Tensor, Tensor)")
 
 
-def _bh4_block_hash_train_impl(x, w_folded, bias, T, decay, residual, warm=None):
+def _bh4_block_hash_train_impl(x, w_folded, bias, T, decay, residual):
     """-> (codes [B,T], scores [B,T], z [B,T*8], stage_inputs [R,J-1,B,D])."""
     _lib.require_gpu(x, w_folded, bias)
     assert x.dim() == 2 and w_folded.dim() == 5
@@ -236,13 +223,11 @@ def _bh4_block_hash_train_impl(x, w_folded, bias, T, decay, residual, warm=None)
     scores = torch.empty(B, T, dtype=torch.float32, device=x.device)
     z = torch.empty(B, T * 8, dtype=torch.float32, device=x.device)
     stage_in = torch.empty(R, max(J - 1, 0), B, D, dtype=torch.float32, device=x.device)
-    wp, wb = _warm_args(warm, x)
     with _dev_guard(x):
-        rc = _lib.load().lffn_bh4_block_hash_warm_f32(
-            _lib.ptr(x), None, None, 0.0, _lib.ptr(w_folded), _lib.ptr(bias), _lib.ptr(codes), _lib.ptr(scores),
-            _lib.ptr(z), _lib.ptr(stage_in) if J > 1 else None, B, H, D, R, J, T, bs, decay, residual, wp, wb,
-            _lib.stream_of(x))
-    _lib.check(rc, f"lffn_bh4_block_hash_warm_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T}, training form)")
+        rc = _lib.load().lffn_bh4_block_hash_train_f32(
+            _lib.ptr(x), _lib.ptr(w_folded), _lib.ptr(bias), _lib.ptr(codes), _lib.ptr(scores), _lib.ptr(z),
+            _lib.ptr(stage_in) if J > 1 else None, B, H, D, R, J, T, bs, decay, residual, _lib.stream_of(x))
+    _lib.check(rc, f"lffn_bh4_block_hash_train_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T})")
     return codes, scores, z, stage_in
 
 
@@ -250,7 +235,7 @@ _L.impl("bh4_block_hash_train", _bh4_block_hash_train_impl, "CUDA")
 
 
 @torch.library.register_fake("lookupffn::bh4_block_hash_train")
-def _(x, w_folded, bias, T, decay, residual, warm=None):
+def _(x, w_folded, bias, T, decay, residual):
     B = x.shape[0]
     R, J, NB, bs, _ = w_folded.shape
     return (torch.empty(B, T, dtype=torch.int32, device=x.device), x.new_empty(B, T), x.new_empty(B, T * 8),
@@ -420,11 +405,11 @@ def _(y, x, bias, T, k, D, decay, residual):
 
 # ----------------------------------------------------------------------------- project_hash
 
-_L.define("project_hash(Tensor x, Tensor diag, Tensor? bias, int T, float decay, float residual, bool keep_z, "
-          "Tensor? warm=None) -> (Tensor, Tensor, Tensor)")
+_L.define("project_hash(Tensor x, Tensor diag, Tensor? bias, int T, float decay, float residual, bool keep_z)"
+          " -> (Tensor, Tensor, Tensor)")
 
 
-def _project_hash_impl(x, diag, bias, T, decay, residual, keep_z, warm=None):
+def _project_hash_impl(x, diag, bias, T, decay, residual, keep_z):
     _lib.require_gpu(x, diag, bias)
     assert x.dim() == 2 and diag.dim() == 3
     assert x.dtype == torch.float32 and diag.dtype == torch.float32
@@ -437,12 +422,11 @@ def _project_hash_impl(x, diag, bias, T, decay, residual, keep_z, warm=None):
     codes = torch.empty(B, T, dtype=torch.int32, device=x.device)
     scores = torch.empty(B, T, dtype=torch.float32, device=x.device)
     z = torch.empty((B, T * 8) if keep_z else (0,), dtype=torch.float32, device=x.device)
-    wp, wb = _warm_args(warm, x)
     with _dev_guard(x):
-        rc = _lib.load().lffn_project_hash_warm_f32(
-            _lib.ptr(x), None, None, 0.0, _lib.ptr(diag), _lib.ptr(bias), _lib.ptr(z) if keep_z else None,
-            _lib.ptr(codes), _lib.ptr(scores), B, H, D, R, J, T, decay, residual, wp, wb, _lib.stream_of(x))
-    _lib.check(rc, f"lffn_project_hash_warm_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T})")
+        rc = _lib.load().lffn_project_hash_f32(
+            _lib.ptr(x), _lib.ptr(diag), _lib.ptr(bias), _lib.ptr(z) if keep_z else None,
+            _lib.ptr(codes), _lib.ptr(scores), B, H, D, R, J, T, decay, residual, _lib.stream_of(x))
+    _lib.check(rc, f"lffn_project_hash_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T})")
     return codes, scores, z
 
 
@@ -450,7 +434,7 @@ _L.impl("project_hash", _project_hash_impl, "CUDA")
 
 
 @torch.library.register_fake("lookupffn::project_hash")
-def _(x, diag, bias, T, decay, residual, keep_z, warm=None):
+def _(x, diag, bias, T, decay, residual, keep_z):
     B = x.shape[0]
     return (x.new_empty(B, T, dtype=torch.int32), x.new_empty(B, T),
             x.new_empty((B, T * 8) if keep_z else (0,)))
@@ -495,10 +479,10 @@ def _(x, diag, z, g_score, decay, residual):
 
 
 _L.define("ln_project_hash(Tensor x, Tensor ln_weight, Tensor ln_bias, float eps, Tensor diag, Tensor? bias, "
-          "int T, float decay, float residual, bool keep_z, Tensor? warm=None) -> (Tensor, Tensor, Tensor)")
+          "int T, float decay, float residual, bool keep_z) -> (Tensor, Tensor, Tensor)")
 
 
-def _ln_project_hash_impl(x, ln_weight, ln_bias, eps, diag, bias, T, decay, residual, keep_z, warm=None):
+def _ln_project_hash_impl(x, ln_weight, ln_bias, eps, diag, bias, T, decay, residual, keep_z):
     _lib.require_gpu(x, ln_weight, ln_bias, diag, bias)
     assert x.dim() == 2 and diag.dim() == 3
     assert x.dtype == torch.float32 and diag.dtype == torch.float32
@@ -512,13 +496,12 @@ def _ln_project_hash_impl(x, ln_weight, ln_bias, eps, diag, bias, T, decay, resi
     codes = torch.empty(B, T, dtype=torch.int32, device=x.device)
     scores = torch.empty(B, T, dtype=torch.float32, device=x.device)
     z = torch.empty((B, T * 8) if keep_z else (0,), dtype=torch.float32, device=x.device)
-    wp, wb = _warm_args(warm, x)
     with _dev_guard(x):
-        rc = _lib.load().lffn_project_hash_warm_f32(
+        rc = _lib.load().lffn_ln_project_hash_f32(
             _lib.ptr(x), _lib.ptr(ln_weight), _lib.ptr(ln_bias), eps, _lib.ptr(diag), _lib.ptr(bias),
             _lib.ptr(z) if keep_z else None, _lib.ptr(codes), _lib.ptr(scores),
-            B, H, D, R, J, T, decay, residual, wp, wb, _lib.stream_of(x))
-    _lib.check(rc, f"lffn_project_hash_warm_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T}, with LayerNorm)")
+            B, H, D, R, J, T, decay, residual, _lib.stream_of(x))
+    _lib.check(rc, f"lffn_ln_project_hash_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T})")
     return codes, scores, z
 
 
@@ -526,7 +509,7 @@ _L.impl("ln_project_hash", _ln_project_hash_impl, "CUDA")
 
 
 @torch.library.register_fake("lookupffn::ln_project_hash")
-def _(x, ln_weight, ln_bias, eps, diag, bias, T, decay, residual, keep_z, warm=None):
+def _(x, ln_weight, ln_bias, eps, diag, bias, T, decay, residual, keep_z):
     B = x.shape[0]
     return (x.new_empty(B, T, dtype=torch.int32), x.new_empty(B, T),
             x.new_empty((B, T * 8) if keep_z else (0,)))

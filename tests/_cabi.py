@@ -336,37 +336,3 @@ def lookup_inner(code, g, tables):
     out = torch.full((B, T), float("nan"), dtype=torch.float32, device=DEV)   # must be fully overwritten
     _call("lffn_lookup_inner_f32", p(cd), p(gd), p(td), p(out), B, T, S, Do)
     return host(out)
-
-
-def project_hash_warm(x, ln_w, ln_b, eps, diag, bias, T, warm, warm_bytes=None, decay=0.7):
-    """ln_w None: no LayerNorm.  warm: numpy array read through by the kernel (or None)."""
-    xd, wd, bd2, dd, bd, wm = dev(x), dev(ln_w), dev(ln_b), dev(diag), dev(bias), dev(warm)
-    B, H = x.shape
-    R, J, D = diag.shape
-    codes = torch.full((B, T), -1, dtype=torch.int32, device=DEV)
-    scores = torch.full((B, T), float("nan"), dtype=torch.float32, device=DEV)
-    z = torch.full((B, T * 8), float("nan"), dtype=torch.float32, device=DEV)
-    nbytes = (0 if warm is None else warm.nbytes) if warm_bytes is None else warm_bytes
-    _call("lffn_project_hash_warm_f32", p(xd), p(wd), p(bd2), float(np.float32(eps)), p(dd), p(bd), p(z), p(codes),
-          p(scores), B, H, D, R, J, T, float(np.float32(decay)), float(np.float32(1 - decay)), p(wm), nbytes)
-    return host(codes), host(scores), host(z)
-
-
-def bh4_block_hash_warm(x, ln_w, ln_b, eps, w, bias, T, warm, warm_bytes=None, train=False, decay=0.7):
-    """-> codes, scores (+ z, stage_inputs when train); w: [R, J, NB, 64, 64]."""
-    xd, lw, lb, wd, bd, wm = dev(x), dev(ln_w), dev(ln_b), dev(w), dev(bias), dev(warm)
-    B, H = x.shape
-    R, J, NB, bs, _ = w.shape
-    D = NB * bs
-    wf = torch.empty_like(wd)
-    _call("lffn_bh4_fold_f32", p(wd), p(wf), R, J, NB, bs)
-    codes = torch.full((B, T), -1, dtype=torch.int32, device=DEV)
-    scores = torch.full((B, T), float("nan"), dtype=torch.float32, device=DEV)
-    z = torch.full((B, T * 8), float("nan"), dtype=torch.float32, device=DEV) if train else None
-    st = torch.full((R, max(J - 1, 1), B, D), float("nan"), dtype=torch.float32, device=DEV) if train else None
-    nbytes = (0 if warm is None else warm.nbytes) if warm_bytes is None else warm_bytes
-    _call("lffn_bh4_block_hash_warm_f32", p(xd), p(lw), p(lb), float(np.float32(eps)), p(wf), p(bd), p(codes), p(scores),
-          p(z), p(st), B, H, D, R, J, T, bs, float(np.float32(decay)), float(np.float32(1 - decay)), p(wm), nbytes)
-    if train:
-        return host(codes), host(scores), host(z), host(st)[:, :J - 1]
-    return host(codes), host(scores)

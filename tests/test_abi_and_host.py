@@ -88,20 +88,6 @@ def test_argument_validation_of_the_backward_and_block_entry_points():
                                           0.7, 0.3, None) == A                      # LayerNorm weight without bias
     assert lib.lffn_ln_bh4_block_hash_f32(P, None, None, 0.0, P, None, P, P, 0, 768, 1024, 1, 4, 128, 64,
                                           0.7, 0.3, None) == OK
-    # the hashing front ends with cache warming: the region is checked before anything is launched
-    ph = lib.lffn_project_hash_warm_f32
-    assert ph(P, P, P, 1e-5, P, None, None, P, P, 4, 768, 1024, 1, 4, 128, 0.7, 0.3, None, 64, None) == A    # bytes, no region
-    assert ph(P, P, P, 1e-5, P, None, None, P, P, 4, 768, 1024, 1, 4, 128, 0.7, 0.3, P, -1, None) == A
-    assert ph(P, P, P, 1e-5, P, None, None, P, P, 4, 768, 1024, 1, 4, 128, 0.7, 0.3, P + 4, 64, None) == A   # misaligned
-    assert ph(P, P, None, 1e-5, P, None, None, P, P, 4, 768, 1024, 1, 4, 128, 0.7, 0.3, P, 64, None) == A    # weight, no bias
-    assert ph(P, None, None, 0.0, P, None, None, P, P, 4, 768, 1024, 1, 4, 200, 0.7, 0.3, P, 64, None) == A  # T*8 > R*D
-    assert ph(P, None, None, 0.0, P, None, None, P, P, 0, 768, 1024, 1, 4, 128, 0.7, 0.3, P, 64, None) == OK
-    bw = lib.lffn_bh4_block_hash_warm_f32
-    assert bw(P, None, None, 0.0, P, None, P, P, None, None, 4, 768, 1024, 1, 4, 128, 64, 0.7, 0.3, None, 64, None) == A
-    assert bw(P, None, None, 0.0, P, None, P, P, None, None, 4, 768, 1024, 1, 4, 128, 64, 0.7, 0.3, P + 8, 64, None) == A
-    assert bw(P, None, None, 0.0, P, None, P, P, None, None, 4, 768, 1024, 1, 4, 128, 32, 0.7, 0.3, P, 64, None) == U
-    assert bw(P, None, None, 0.0, P, None, P, P, P + 4, None, 4, 768, 1024, 1, 4, 128, 64, 0.7, 0.3, P, 64, None) == A  # z
-    assert bw(P, None, None, 0.0, P, None, P, P, None, None, 0, 768, 1024, 1, 4, 128, 64, 0.7, 0.3, P, 64, None) == OK
     # mix + hash
     assert lib.lffn_mix_code_score_f32(P, P, None, P, P, 4, 8, 25, 64, 64, 256, 0.7, 0.3, None) == U   # k > 24
     assert lib.lffn_mix_code_score_f32(P, P, None, P, P, 4, 40, 8, 64, 64, 256, 0.7, 0.3, None) == A   # T*k > ldy

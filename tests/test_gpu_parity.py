@@ -477,59 +477,6 @@ def test_ln_project_hash_matches_oracle(H, D, R, T):
     assert np.abs(z - z2).max() <= 1e-5 * scale
 
 
-@pytest.mark.parametrize("B,H,D,R,T,with_ln", [(300, 768, 1024, 1, 128, True), (41, 256, 256, 2, 64, False),
-                                                (5, 100, 128, 2, 30, True), (2048, 768, 1024, 1, 128, True)])
-@pytest.mark.parametrize("warm_bytes", [0, 16, 1008, 1024, 5 * 1024 + 16, 3 << 20])
-def test_project_hash_with_cache_warming_is_bit_identical(B, H, D, R, T, with_ln, warm_bytes):
-    """The kernel reads the region through while it computes and discards it: codes, scores and z
-    are those of the entry points without warming, bit for bit, whatever the region's size (empty,
-    shorter than the 1 KiB unit, not a multiple of it, more than the wavefronts' 32 KiB shares
-    cover at a small batch)."""
-    rng = np.random.RandomState(B + H + T + warm_bytes % 1000)
-    J = 4
-    x = (rng.randn(B, H) * 1.5 + 0.3).astype(np.float32)
-    ln_w = (1 + 0.1 * rng.randn(H)).astype(np.float32) if with_ln else None
-    ln_b = (0.1 * rng.randn(H)).astype(np.float32) if with_ln else None
-    diag = (rng.randn(R, J, D) / math.sqrt(D)).astype(np.float32)
-    bias = (0.05 * rng.randn(T * 8)).astype(np.float32)
-    region = rng.randn(max(warm_bytes // 4, 4)).astype(np.float32)
-    if with_ln:
-        want = cabi.ln_project_hash(x, ln_w, ln_b, 1e-5, diag, bias, T)
-    else:
-        want = cabi.project_hash(x, diag, bias, T)
-    got = cabi.project_hash_warm(x, ln_w, ln_b, 1e-5 if with_ln else 0.0, diag, bias, T,
-                                 region if warm_bytes else None, warm_bytes)
-    for g, w in zip(got, want):
-        assert np.array_equal(g, w)
-
-
-@pytest.mark.parametrize("B,H,D,R,T,with_ln,train", [(100, 768, 1024, 1, 128, True, False),
-                                                      (33, 256, 256, 2, 64, False, True),
-                                                      (17, 64, 64, 1, 8, True, False),
-                                                      (70, 768, 1024, 1, 128, False, True)])
-@pytest.mark.parametrize("warm_bytes", [0, 1008, 7 * 1024 + 32, 3 << 20])
-def test_bh4_block_hash_with_cache_warming_is_bit_identical(B, H, D, R, T, with_ln, train, warm_bytes):
-    """64 x 64 blocks: the warming entry point covers the inference form (LayerNorm optional) and
-    the training form (z and the stage inputs kept) and returns what those return, bit for bit."""
-    rng = np.random.RandomState(B + H + T + warm_bytes % 1000)
-    J, NB = 4, D // 64
-    x = (rng.randn(B, H) * 1.5 + 0.3).astype(np.float32)
-    ln_w = (1 + 0.1 * rng.randn(H)).astype(np.float32) if with_ln else None
-    ln_b = (0.1 * rng.randn(H)).astype(np.float32) if with_ln else None
-    w = (rng.randn(R, J, NB, 64, 64) / math.sqrt(64 * D)).astype(np.float32)
-    bias = (0.05 * rng.randn(T * 8)).astype(np.float32)
-    region = rng.randn(max(warm_bytes // 4, 4)).astype(np.float32)
-    if train:
-        want = cabi.bh4_block_train(x, w, bias, T)
-    else:
-        want = cabi.ln_bh4_block_hash(x, ln_w, ln_b, 1e-5, w, bias, T)
-    got = cabi.bh4_block_hash_warm(x, ln_w, ln_b, 1e-5 if with_ln else 0.0, w, bias, T,
-                                   region if warm_bytes else None, warm_bytes, train=train)
-    assert len(got) == len(want)
-    for g, wv in zip(got, want):
-        assert np.array_equal(g, wv)
-
-
 def test_project_hash_near_zero_flip_count():
     # end to end against the float64 truth: flips may only happen where |z| is tiny
     rng = np.random.RandomState(9)
