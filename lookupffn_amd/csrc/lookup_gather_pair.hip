@@ -48,6 +48,7 @@ struct PairArgs {
     int T, S, Do;
     int ntiles, nslices, per_xcd;
     int row_bytes;         // Do * element size
+    int touch_ahead;       // the team touch runs this many table pairs ahead of the pair being read; 0: no touch
 };
 
 // global_load_lds_dwordx4: lane i of the wavefront writes its 16 bytes at the LDS
@@ -91,7 +92,9 @@ __device__ __forceinline__ int half_row_broadcast(int v) {
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) const u32x4 *lds_vec_ptr;
 
-template <bool BF16, int NP, bool FULL>
+// TOUCH: with the team touch (a template parameter: a run-time branch in the pair loop, even a uniform
+// one, makes the compiler spill hundreds of registers here).
+template <bool BF16, int NP, bool FULL, bool TOUCH>
 __global__ __launch_bounds__(WG) void lookup_gather_pair_kernel(PairArgs a) {
     constexpr int EPV = BF16 ? 8 : 4;
     // bf16: four 8-bit codes per register.  fp32: two per register, each at bits 8..15 of its
@@ -139,6 +142,15 @@ __global__ __launch_bounds__(WG) void lookup_gather_pair_kernel(PairArgs a) {
     const size_t table_bytes = (size_t)a.S * a.row_bytes;
     const int npairs = (a.T + 1) / 2;
     const int last_t = a.T - 1;
+    // Team touch (see lookup_gather.hip): the workgroups that share this slice each pull a share of
+    // the 2*S lines of the pair after next (one line per table row) into the XCD's L2.
+    // (Only whole pairs are touched: with an odd number of tables the last one comes untouched.)
+    const int touch_line = team_touch_line(a.S * 2, a.ntiles, tile, tid);
+    const bool touch_second = touch_line >= a.S;                      // a row of the pair's second table
+    const uint32_t touch_off = (touch_second ? (uint32_t)table_bytes : 0u) +
+                               (uint32_t)(touch_line - (touch_second ? a.S : 0)) * (uint32_t)a.row_bytes;
+    const int last_whole_pair = max(a.T / 2 - 1, 0);
+    const uint32_t touch_dst = lds0 + (uint32_t)(2 * buf_vecs) * 16u;
 
     // (code, score) of tables c*8 + j for this lane's NP tokens; tokens and tables
     // past the end read a valid address and get score 0
@@ -197,6 +209,8 @@ __global__ __launch_bounds__(WG) void lookup_gather_pair_kernel(PairArgs a) {
                     copy_pair_to_lds<FULL>(slice_base, table_bytes, 2 * kn, min(2 * kn + 1, last_t), a.row_bytes,
                                            tid, buf_vecs, lds + ((k + 1) & 1) * buf_vecs);
                 }
+                if constexpr (TOUCH)
+                    l2_touch(slice_base + (size_t)(2 * min(k + a.touch_ahead, last_whole_pair)) * table_bytes, touch_off, touch_dst);
                 const uint4 *buf = lds + (k & 1) * buf_vecs + j;
                 static_for<2>([&](auto half_c) {
                     constexpr int HALF = decltype(half_c)::value;
@@ -266,11 +280,13 @@ __global__ __launch_bounds__(WG) void lookup_gather_pair_kernel(PairArgs a) {
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 });
-                __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the copy issued above has landed
+                // the copy issued above has landed; the touch, issued after it, may still be out
+                __builtin_amdgcn_s_waitcnt(TOUCH ? WAIT_VMCNT_1 : WAIT_VMCNT_0);
                 __syncthreads();
             }
         });
     }
+    __builtin_amdgcn_s_waitcnt(0x0F70);         // nothing may still be writing this workgroup's LDS when it ends
 
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
@@ -291,13 +307,13 @@ __global__ __launch_bounds__(WG) void lookup_gather_pair_kernel(PairArgs a) {
     }
 }
 
-template <bool BF16, int NP, bool FULL>
+template <bool BF16, int NP, bool FULL, bool TOUCH>
 int launch_pair_full(PairArgs a, hipStream_t stream) {
     a.ntiles = (int)((a.B + 128 * NP - 1) / (128 * NP));
     const int units = a.ntiles * a.nslices;
     a.per_xcd = (units + XCDS - 1) / XCDS;
-    const size_t lds_bytes = size_t(2) * a.S * ROW_VECS * 16;
-    auto kern = lookup_gather_pair_kernel<BF16, NP, FULL>;
+    const size_t lds_bytes = size_t(2) * a.S * ROW_VECS * 16 + TOUCH_SINK_BYTES;     // two buffers + the touches' scratch
+    auto kern = lookup_gather_pair_kernel<BF16, NP, FULL, TOUCH>;
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds_bytes) != hipSuccess) {
         (void)hipGetLastError();
@@ -309,7 +325,10 @@ int launch_pair_full(PairArgs a, hipStream_t stream) {
 
 template <bool BF16, int NP>
 int launch_pair(const PairArgs &a, hipStream_t stream) {
-    return a.S == MAX_S ? launch_pair_full<BF16, NP, true>(a, stream) : launch_pair_full<BF16, NP, false>(a, stream);
+    // the touch: 256-row tables only (as in lookup_gather.hip) and only while the table set fits the cache
+    if (a.S != MAX_S) return launch_pair_full<BF16, NP, false, false>(a, stream);
+    return a.touch_ahead > 0 ? launch_pair_full<BF16, NP, true, true>(a, stream)
+                             : launch_pair_full<BF16, NP, true, false>(a, stream);
 }
 
 }  // namespace
@@ -325,7 +344,7 @@ int lffn_internal_lookup_gather_pair(const int32_t *code, const float *score, co
     a.code = code; a.score = score; a.tables = static_cast<const char *>(tables); a.bias = bias; a.residual = residual; a.out = out;
     a.B = B; a.T = (int)T; a.S = (int)S; a.Do = (int)Do;
     a.nslices = (int)(Do / (bf16 ? 64 : 32));
-    a.row_bytes = (int)(Do * (bf16 ? 2 : 4));
+    a.row_bytes = (int)(Do * (bf16 ? 2 : 4)); a.touch_ahead = lffn_touch_ahead(T * S * Do * (bf16 ? 2 : 4)) == 2 ? 2 : 0;   // measured 2-4% slower when the table set does not fit the cache
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (bf16) return np == 8 ? launch_pair<true, 8>(a, st) : launch_pair<true, 4>(a, st);
     switch (np) {

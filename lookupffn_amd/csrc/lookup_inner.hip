@@ -45,6 +45,7 @@ struct InnerArgs {
     int T, S, Do;
     int ntiles, nslices, per_xcd;
     int row_bytes;
+    int touch_ahead;       // the team touch runs this many tables ahead of the table being read (1 or 2)
 };
 
 // global_load_lds_dwordx4: lane i of the wavefront writes its 16 bytes at the LDS
@@ -114,6 +115,12 @@ __global__ __launch_bounds__(WG) void lookup_inner_lds_kernel(InnerArgs a) {
     const char *slice_base = a.tables + (size_t)slice * (SEG_VECS * 16);
     const size_t table_bytes = (size_t)a.S * a.row_bytes;
 
+    // Team touch (see lookup_gather.hip): the workgroups that share this slice each pull a share of
+    // the lines of the table after next into the XCD's L2.
+    const int touch_line = team_touch_line(a.S * 2, a.ntiles, tile, tid);
+    const uint32_t touch_off = (uint32_t)(touch_line >> 1) * (uint32_t)a.row_bytes + (touch_line & 1) * 128;
+    const uint32_t touch_dst = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint4 *)(lds + 2 * buf_vecs);
+
     copy_slice_to_lds<FULL>(slice_base, a.row_bytes, tid, buf_vecs, lds);
     __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0)
     __syncthreads();
@@ -154,6 +161,8 @@ __global__ __launch_bounds__(WG) void lookup_inner_lds_kernel(InnerArgs a) {
                 const int t = t0 + TT;
                 copy_slice_to_lds<FULL>(slice_base + (size_t)min(t + 1, a.T - 1) * table_bytes, a.row_bytes, tid,
                                         buf_vecs, lds + ((t + 1) & 1) * buf_vecs);
+                if constexpr (FULL)
+                    l2_touch(slice_base + (size_t)min(t + a.touch_ahead, a.T - 1) * table_bytes, touch_off, touch_dst);
                 const uint4 *buf = lds + (t & 1) * buf_vecs + j;
                 constexpr int GRP = 4;
 #pragma unroll
@@ -190,7 +199,8 @@ __global__ __launch_bounds__(WG) void lookup_inner_lds_kernel(InnerArgs a) {
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0): the copy issued above has landed
+                __builtin_amdgcn_s_waitcnt(FULL ? WAIT_VMCNT_1 : WAIT_VMCNT_0);     // vmcnt(1): the copy issued above has landed; the touch,
+                                                        // issued after it, may still be out
                 __syncthreads();
             }
         });
@@ -204,6 +214,7 @@ __global__ __launch_bounds__(WG) void lookup_inner_lds_kernel(InnerArgs a) {
             }
         }
     }
+    __builtin_amdgcn_s_waitcnt(0x0F70);         // nothing may still be writing this workgroup's LDS when it ends
 }
 
 __global__ __launch_bounds__(256) void fill_zero_f32_kernel(float *p, int64_t n) {
@@ -215,7 +226,7 @@ int launch_inner_full(InnerArgs a, hipStream_t stream) {
     a.ntiles = (int)((a.B + 64 * NP - 1) / (64 * NP));
     const int units = a.ntiles * a.nslices;
     a.per_xcd = (units + XCDS - 1) / XCDS;
-    const size_t lds_bytes = size_t(2) * a.S * SEG_VECS * 16;
+    const size_t lds_bytes = size_t(2) * a.S * SEG_VECS * 16 + TOUCH_SINK_BYTES;     // two buffers + the touches' scratch
     auto kern = lookup_inner_lds_kernel<NP, FULL>;
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds_bytes) != hipSuccess) {
@@ -260,7 +271,7 @@ extern "C" int lffn_lookup_inner_f32(const int32_t *code, const float *g, const 
     a.code = code; a.g = g; a.tables = reinterpret_cast<const char *>(tables); a.out = grad_score;
     a.B = B; a.T = (int)T; a.S = (int)S; a.Do = (int)Do;
     a.nslices = (int)nslices;
-    a.row_bytes = (int)(Do * 4);
+    a.row_bytes = (int)(Do * 4); a.touch_ahead = lffn_touch_ahead(T * S * Do * 4);
     // tile: fewest rounds of 256 workgroups, then the larger tile (fewer table copies)
     const int nps[] = {13, 8, 4};
     int best = 4;
