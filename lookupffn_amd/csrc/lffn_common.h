@@ -172,12 +172,9 @@ __device__ __forceinline__ int team_touch_line(int nlines, int nteam, int member
     return min(line, nlines - 1);
 }
 
-// How far ahead the team touches: the table (or table pair) after next while the table set fits the
-// 256 MB memory-side cache; beyond that the kernels are bound by HBM traffic, the (code, score)
-// stream pushes lines touched that early out of L2 before their copy comes (measured at 537 MB of
-// tables: 4% more traffic, 2% slower), and the touch falls back on the table the copy has just asked
-// for, which costs nothing.
-static inline int lffn_touch_ahead(int64_t table_set_bytes) { return table_set_bytes <= (int64_t(256) << 20) ? 2 : 1; }
+// How far ahead of the table being read the team touches: the copy of table t+1 is issued with the
+// reads of table t, the touch of table t+2 with it (3 or 4 ahead measured no better).
+constexpr int TOUCH_AHEAD = 2;
 
 __device__ __forceinline__ float bf16_lo(uint32_t packed) { return __uint_as_float(packed << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t packed) { return __uint_as_float(packed & 0xFFFF0000u); }

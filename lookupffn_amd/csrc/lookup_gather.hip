@@ -54,7 +54,6 @@ struct LdsGatherArgs {
     // and, when nparts > 1, writes its sums without bias and residual to part_out[p][B][Do].
     int nparts, part_tables;
     float *part_out;
-    int touch_ahead;       // the team touch runs this many tables ahead of the table being read (1 or 2)
 };
 
 // Copy this lane's four vectors of a table slice straight from global memory into
@@ -227,7 +226,7 @@ __global__ __launch_bounds__(WG) void lookup_gather_lds_kernel(LdsGatherArgs a) 
                 copy_slice_to_lds<FULL>(slice_base + (size_t)min(t + 1, t_end - 1) * table_bytes, cl, tid, buf_vecs,
                                         lds0 + (uint32_t)(((t + 1) & 1) * buf_vecs) * 16u);
                 if constexpr (FULL)
-                    l2_touch(slice_base + (size_t)min(t + a.touch_ahead, t_end - 1) * table_bytes, touch_off, touch_dst);
+                    l2_touch(slice_base + (size_t)min(t + TOUCH_AHEAD, t_end - 1) * table_bytes, touch_off, touch_dst);
                 const uint4 *buf = lds + (t & 1) * buf_vecs + j;
                 const unsigned buf_addr = lds_base + (unsigned)((t & 1) * buf_vecs) * 16u;
                 unsigned packed[NQ];
@@ -490,7 +489,7 @@ int lookup_gather_entry(const int32_t *code, const float *score, const void *tab
                 a.residual = nullptr; a.out = out;
                 a.B = B; a.T = (int)T; a.S = (int)S; a.Do = (int)Do;
                 a.nslices = (int)(Do / (BF16 ? 128 : 64));
-                a.row_bytes = (int)(Do * (BF16 ? 2 : 4)); a.touch_ahead = lffn_touch_ahead(T * S * Do * (BF16 ? 2 : 4));
+                a.row_bytes = (int)(Do * (BF16 ? 2 : 4));
                 a.nparts = sp.nparts; a.part_tables = sp.part_tables; a.part_out = static_cast<float *>(workspace);
                 hipStream_t st = static_cast<hipStream_t>(stream);
                 int rc;
@@ -523,7 +522,7 @@ int lookup_gather_entry(const int32_t *code, const float *score, const void *tab
     a.code = code; a.score = score; a.tables = static_cast<const char *>(tables); a.bias = bias; a.residual = residual; a.out = out;
     a.B = B; a.T = (int)T; a.S = (int)S; a.Do = (int)Do;
     a.nslices = (int)(Do / (BF16 ? 128 : 64));
-    a.row_bytes = (int)(Do * (BF16 ? 2 : 4)); a.touch_ahead = lffn_touch_ahead(T * S * Do * (BF16 ? 2 : 4));
+    a.row_bytes = (int)(Do * (BF16 ? 2 : 4));
     a.nparts = 1; a.part_tables = (int)T; a.part_out = nullptr;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if constexpr (BF16) {

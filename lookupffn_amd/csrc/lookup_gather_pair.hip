@@ -48,7 +48,7 @@ struct PairArgs {
     int T, S, Do;
     int ntiles, nslices, per_xcd;
     int row_bytes;         // Do * element size
-    int touch_ahead;       // the team touch runs this many table pairs ahead of the pair being read; 0: no touch
+    int touch;             // 1: with the team touch (decided by the host, see launch_pair)
 };
 
 // global_load_lds_dwordx4: lane i of the wavefront writes its 16 bytes at the LDS
@@ -210,7 +210,7 @@ __global__ __launch_bounds__(WG) void lookup_gather_pair_kernel(PairArgs a) {
                                            tid, buf_vecs, lds + ((k + 1) & 1) * buf_vecs);
                 }
                 if constexpr (TOUCH)
-                    l2_touch(slice_base + (size_t)(2 * min(k + a.touch_ahead, last_whole_pair)) * table_bytes, touch_off, touch_dst);
+                    l2_touch(slice_base + (size_t)(2 * min(k + TOUCH_AHEAD, last_whole_pair)) * table_bytes, touch_off, touch_dst);
                 const uint4 *buf = lds + (k & 1) * buf_vecs + j;
                 static_for<2>([&](auto half_c) {
                     constexpr int HALF = decltype(half_c)::value;
@@ -325,9 +325,11 @@ int launch_pair_full(PairArgs a, hipStream_t stream) {
 
 template <bool BF16, int NP>
 int launch_pair(const PairArgs &a, hipStream_t stream) {
-    // the touch: 256-row tables only (as in lookup_gather.hip) and only while the table set fits the cache
+    // The touch: 256-row tables only (as in lookup_gather.hip) and only while the table set fits the
+    // 256 MB memory-side cache: beyond that this kernel is bound by HBM traffic and was measured 2-4%
+    // slower with it (537 MB of tables).
     if (a.S != MAX_S) return launch_pair_full<BF16, NP, false, false>(a, stream);
-    return a.touch_ahead > 0 ? launch_pair_full<BF16, NP, true, true>(a, stream)
+    return a.touch ? launch_pair_full<BF16, NP, true, true>(a, stream)
                              : launch_pair_full<BF16, NP, true, false>(a, stream);
 }
 
@@ -344,7 +346,7 @@ int lffn_internal_lookup_gather_pair(const int32_t *code, const float *score, co
     a.code = code; a.score = score; a.tables = static_cast<const char *>(tables); a.bias = bias; a.residual = residual; a.out = out;
     a.B = B; a.T = (int)T; a.S = (int)S; a.Do = (int)Do;
     a.nslices = (int)(Do / (bf16 ? 64 : 32));
-    a.row_bytes = (int)(Do * (bf16 ? 2 : 4)); a.touch_ahead = lffn_touch_ahead(T * S * Do * (bf16 ? 2 : 4)) == 2 ? 2 : 0;   // measured 2-4% slower when the table set does not fit the cache
+    a.row_bytes = (int)(Do * (bf16 ? 2 : 4)); a.touch = T * S * Do * (bf16 ? 2 : 4) <= (int64_t(256) << 20) ? 1 : 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (bf16) return np == 8 ? launch_pair<true, 8>(a, st) : launch_pair<true, 4>(a, st);
     switch (np) {

@@ -45,7 +45,6 @@ struct InnerArgs {
     int T, S, Do;
     int ntiles, nslices, per_xcd;
     int row_bytes;
-    int touch_ahead;       // the team touch runs this many tables ahead of the table being read (1 or 2)
 };
 
 // global_load_lds_dwordx4: lane i of the wavefront writes its 16 bytes at the LDS
@@ -162,7 +161,7 @@ __global__ __launch_bounds__(WG) void lookup_inner_lds_kernel(InnerArgs a) {
                 copy_slice_to_lds<FULL>(slice_base + (size_t)min(t + 1, a.T - 1) * table_bytes, a.row_bytes, tid,
                                         buf_vecs, lds + ((t + 1) & 1) * buf_vecs);
                 if constexpr (FULL)
-                    l2_touch(slice_base + (size_t)min(t + a.touch_ahead, a.T - 1) * table_bytes, touch_off, touch_dst);
+                    l2_touch(slice_base + (size_t)min(t + TOUCH_AHEAD, a.T - 1) * table_bytes, touch_off, touch_dst);
                 const uint4 *buf = lds + (t & 1) * buf_vecs + j;
                 constexpr int GRP = 4;
 #pragma unroll
@@ -271,7 +270,7 @@ extern "C" int lffn_lookup_inner_f32(const int32_t *code, const float *g, const 
     a.code = code; a.g = g; a.tables = reinterpret_cast<const char *>(tables); a.out = grad_score;
     a.B = B; a.T = (int)T; a.S = (int)S; a.Do = (int)Do;
     a.nslices = (int)nslices;
-    a.row_bytes = (int)(Do * 4); a.touch_ahead = lffn_touch_ahead(T * S * Do * 4);
+    a.row_bytes = (int)(Do * 4);
     // tile: fewest rounds of 256 workgroups, then the larger tile (fewer table copies)
     const int nps[] = {13, 8, 4};
     int best = 4;
