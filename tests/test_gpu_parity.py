@@ -80,7 +80,7 @@ def test_fht_integer_inputs_exact_and_involution():
 
 
 def test_fht_full_size_properties():
-    # BASELINE config 2 shape: 16384 x 1024; linearity + Parseval + involution
+    # BASELINE.json config 2 shape: 16384 x 1024; linearity + Parseval + involution
     rng = np.random.RandomState(6)
     B, D = 16384, 1024
     x = rng.randn(B, D).astype(np.float32)
@@ -411,7 +411,7 @@ def test_layer_norm_bwd_matches_float64(B, H, R, affine):
 
 
 def test_sign_diagonal_fht_exact():
-    # the BASELINE "random +-1 sign diagonal from seed": one round, exact on integers
+    # the BASELINE.json "random +-1 sign diagonal from seed": one round, exact on integers
     rng = np.random.RandomState(8)
     B, D = 33, 1024
     x = rng.randint(-8, 9, size=(B, D)).astype(np.float32)
@@ -730,7 +730,7 @@ def test_lookup_gather_lds_kernels_bf16_match_oracle(B, T, S, Do, plan):
 
 def test_lookup_gather_plan_and_planned_entry():
     from lookupffn_amd import _lib
-    # what the heuristic picks at the BASELINE shapes
+    # what the heuristic picks at the BASELINE.json shapes
     assert cabi.lookup_gather_plan(16384, 128, 256, 768) == (1, 832)            # config 2
     assert cabi.lookup_gather_plan(16384, 512, 256, 1024) == (2, 2048)          # config 3 fp32
     assert cabi.lookup_gather_plan(16384, 512, 256, 1024, bf16=True) == (2, 1024)
@@ -771,7 +771,7 @@ def test_gather_special_cases():
 
 
 def test_gather_full_size_properties():
-    # BASELINE config 2: 16384 tokens, 128 tables x 256 x 768 fp32
+    # BASELINE.json config 2: 16384 tokens, 128 tables x 256 x 768 fp32
     rng = np.random.RandomState(31)
     B, T, S, Do = 16384, 128, 256, 768
     tables, code, idx, w = _rand_gather(rng, B, T, S, Do)
@@ -890,7 +890,7 @@ def test_lookup_scatter_sorted_workspace_query():
 
 
 def test_lookup_scatter_sorted_full_size_zipf():
-    # BASELINE config 5: config-2 shape, codes Zipf(1.1) over 256 entries (the hottest code takes ~18 % of the tokens)
+    # BASELINE.json config 5: config-2 shape, codes Zipf(1.1) over 256 entries (the hottest code takes ~18 % of the tokens)
     rng = np.random.RandomState(41)
     B, T, S, Do = 16384, 128, 256, 768
     p = 1.0 / np.arange(1, S + 1) ** 1.1
@@ -908,7 +908,7 @@ def test_lookup_scatter_sorted_full_size_zipf():
 
 
 def test_lookup_scatter_full_size_zipf_properties():
-    # BASELINE config 5: config-2 shape, codes Zipf(1.1) over 256 entries
+    # BASELINE.json config 5: config-2 shape, codes Zipf(1.1) over 256 entries
     rng = np.random.RandomState(41)
     B, T, S, Do = 16384, 128, 256, 768
     p = 1.0 / np.arange(1, S + 1) ** 1.1
@@ -962,7 +962,7 @@ def test_lookup_inner_matches_oracle(B, T, S, Do):
 
 
 def test_lookup_inner_full_size_duality():
-    # BASELINE config 2 shape: <G(w), g> = sum_bt w[b,t] * grad_score[b,t], and linearity in g
+    # BASELINE.json config 2 shape: <G(w), g> = sum_bt w[b,t] * grad_score[b,t], and linearity in g
     rng = np.random.RandomState(43)
     B, T, S, Do = 16384, 128, 256, 768
     tables, code, idx, w = _rand_gather(rng, B, T, S, Do)
@@ -980,7 +980,7 @@ def test_lookup_inner_full_size_duality():
 
 
 def test_scatter_duplicates_zipf():
-    # heavy duplication of rows (BASELINE config 5 draws codes Zipf(1.1))
+    # heavy duplication of rows (BASELINE.json config 5 draws codes Zipf(1.1))
     rng = np.random.RandomState(40)
     B, T, S, Do = 2048, 16, 256, 256
     p = 1.0 / np.arange(1, S + 1) ** 1.1
