@@ -129,7 +129,14 @@ def ptr(t):
     return None if t is None else t.data_ptr()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_of(t: torch.Tensor) -> int:
+    """The HIP stream torch currently launches on for t's device, as an integer handle."""
+    if _raw_stream is not None:          # a tenth of the cost of building a torch.cuda.Stream object
+        idx = t.device.index
+        return _raw_stream(torch.cuda.current_device() if idx is None else idx)
     return torch.cuda.current_stream(t.device).cuda_stream
 
 

@@ -161,6 +161,7 @@ struct ProjectArgs {
 };
 
 constexpr int FUSED_MAX_T = 512;   // (code, score) pairs a wavefront keeps in LDS for its token
+constexpr int FUSED_MAX_NC = 4;    // column passes of 256 the one-launch layer's gather keeps in flight together
 
 // Part of the score recurrence over the four values of one float4:
 // s <- s + a_c, p <- p * f_c with a_c = |z_c| and f_c = 1 + exp(-2|z_c|), c ascending.
@@ -170,6 +171,74 @@ __device__ __forceinline__ void score_chain(const float (&a)[4], const float (&f
         s = s + a[c];
         p = p * f[c];
     }
+}
+
+// The gather-add of one token inside the one-launch layer (PL/lookup.py:120-130, 108): this
+// wavefront adds the rows of tables [t_lo, t_hi) that the (code, score) pairs in `mine` select,
+// eight tables at a time and all NC column passes of 256 columns of those eight rows in flight
+// together (the token's chain of dependent memory round trips is what a small batch waits for:
+// 8 * NC row loads per round trip instead of 8); the four wavefronts' partial sums meet in LDS and
+// wavefront 0 adds bias and residual and writes the row.  Loads are unconditional at clamped
+// columns, so that none of them waits for another; what a clamped lane loaded is never stored.
+template <int NC>
+__device__ __forceinline__ void fused_gather(const ProjectArgs &a, const uint2 *mine, float4 (*part)[FUSED_MAX_NC][64],
+                                             int64_t row, int col0, int t_lo, int t_hi, int wave, int lane) {
+    int gc[NC];
+    bool on[NC];
+    float4 acc[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        on[c] = col0 + 256 * c + 4 * lane < a.Do;
+        gc[c] = on[c] ? col0 + 256 * c + 4 * lane : 0;
+        acc[c] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    for (int t0 = t_lo; t0 < t_hi; t0 += 8) {
+        float4 rv[8][NC];
+        float sv[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int tt = min(t0 + u, t_hi - 1);
+            const uint2 pr = mine[tt];
+            sv[u] = t0 + u < t_hi ? __uint_as_float(pr.y) : 0.f;
+            const float *rowp = a.tables + ((size_t)tt * a.S + pr.x) * a.Do;
+#pragma unroll
+            for (int c = 0; c < NC; ++c) rv[u][c] = *reinterpret_cast<const float4 *>(rowp + gc[c]);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                acc[c].x = fmaf(sv[u], rv[u][c].x, acc[c].x);
+                acc[c].y = fmaf(sv[u], rv[u][c].y, acc[c].y);
+                acc[c].z = fmaf(sv[u], rv[u][c].z, acc[c].z);
+                acc[c].w = fmaf(sv[u], rv[u][c].w, acc[c].w);
+            }
+    }
+#pragma unroll
+    for (int c = 0; c < NC; ++c) part[wave][c][lane] = acc[c];
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            if (!on[c]) continue;
+            float4 o = part[0][c][lane];
+#pragma unroll
+            for (int w = 1; w < 4; ++w) {
+                const float4 q = part[w][c][lane];
+                o.x += q.x; o.y += q.y; o.z += q.z; o.w += q.w;
+            }
+            if (a.obias) {
+                const float4 bb = *reinterpret_cast<const float4 *>(a.obias + gc[c]);
+                o.x += bb.x; o.y += bb.y; o.z += bb.z; o.w += bb.w;
+            }
+            if (a.gres) {
+                const float4 rr = *reinterpret_cast<const float4 *>(a.gres + row * a.Do + gc[c]);
+                o.x += rr.x; o.y += rr.y; o.z += rr.z; o.w += rr.w;
+            }
+            *reinterpret_cast<float4 *>(a.gout + row * a.Do + gc[c]) = o;
+        }
+    }
+    __syncthreads();                                         // `part` is free again
 }
 
 template <int LOGD, bool HASH, bool GATHER = false>
@@ -304,58 +373,20 @@ __global__ __launch_bounds__(256) void project_kernel(ProjectArgs a) {
                         pairs[wave][t] = make_uint2((unsigned)((nib_hi << 4) | nib), __float_as_uint(s_run / p_run));
                     if (r == a.R - 1 && j == NJ - 1) {
                         // Small batches: the gather-add of the token's T rows follows in the same
-                        // workgroup (PL/lookup.py:120-130, 108): wavefront w takes tables
-                        // [w*T/4, (w+1)*T/4), 256 columns per pass, eight row loads in flight; the
-                        // four partial sums meet in LDS.  No codes or scores go to memory and
-                        // nothing else is launched.
-                        __shared__ float4 part[4][64];
+                        // workgroup: wavefront w takes tables [w*T/4, (w+1)*T/4) (fused_gather).
+                        // No codes or scores go to memory and nothing else is launched.
+                        __shared__ float4 part[4][FUSED_MAX_NC][64];
                         __syncthreads();                         // the odd lanes' pairs are visible to the whole wavefront
-                        const uint2 *mine = pairs[wave];         // this wavefront's own copy
                         const int tq = (a.T + 3) / 4;
                         const int t_lo = min(wave * tq, a.T), t_hi = min(t_lo + tq, a.T);
-                        for (int c0 = 0; c0 < a.Do; c0 += 256) {
-                            const int gc = c0 + 4 * lane;
-                            const bool on = gc < a.Do;
-                            float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-                            for (int t0 = t_lo; t0 < t_hi; t0 += 8) {
-                                float4 rv[8];
-                                float sv[8];
-#pragma unroll
-                                for (int u = 0; u < 8; ++u) {
-                                    const int tt = min(t0 + u, t_hi - 1);
-                                    const uint2 pr = mine[tt];
-                                    sv[u] = t0 + u < t_hi ? __uint_as_float(pr.y) : 0.f;
-                                    const float *rowp = a.tables + ((size_t)tt * a.S + pr.x) * a.Do;
-                                    rv[u] = on ? *reinterpret_cast<const float4 *>(rowp + gc) : make_float4(0.f, 0.f, 0.f, 0.f);
-                                }
-#pragma unroll
-                                for (int u = 0; u < 8; ++u) {
-                                    acc.x = fmaf(sv[u], rv[u].x, acc.x);
-                                    acc.y = fmaf(sv[u], rv[u].y, acc.y);
-                                    acc.z = fmaf(sv[u], rv[u].z, acc.z);
-                                    acc.w = fmaf(sv[u], rv[u].w, acc.w);
-                                }
+                        // up to four column passes of 256 in flight together; wider rows in rounds of 1024
+                        for (int col0 = 0; col0 < a.Do; col0 += 256 * FUSED_MAX_NC) {
+                            switch (min(FUSED_MAX_NC, (a.Do - col0 + 255) / 256)) {
+                                case 1: fused_gather<1>(a, pairs[wave], part, row, col0, t_lo, t_hi, wave, lane); break;
+                                case 2: fused_gather<2>(a, pairs[wave], part, row, col0, t_lo, t_hi, wave, lane); break;
+                                case 3: fused_gather<3>(a, pairs[wave], part, row, col0, t_lo, t_hi, wave, lane); break;
+                                default: fused_gather<4>(a, pairs[wave], part, row, col0, t_lo, t_hi, wave, lane); break;
                             }
-                            part[wave][lane] = acc;
-                            __syncthreads();
-                            if (wave == 0 && on) {
-                                float4 o = part[0][lane];
-#pragma unroll
-                                for (int w = 1; w < 4; ++w) {
-                                    const float4 q = part[w][lane];
-                                    o.x += q.x; o.y += q.y; o.z += q.z; o.w += q.w;
-                                }
-                                if (a.obias) {
-                                    const float4 bb = *reinterpret_cast<const float4 *>(a.obias + gc);
-                                    o.x += bb.x; o.y += bb.y; o.z += bb.z; o.w += bb.w;
-                                }
-                                if (a.gres) {
-                                    const float4 rr = *reinterpret_cast<const float4 *>(a.gres + row * a.Do + gc);
-                                    o.x += rr.x; o.y += rr.y; o.z += rr.z; o.w += rr.w;
-                                }
-                                *reinterpret_cast<float4 *>(a.gout + row * a.Do + gc) = o;
-                            }
-                            __syncthreads();
                         }
                     }
                 } else if (live && (lr & 1) && t < a.T) {

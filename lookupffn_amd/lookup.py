@@ -287,25 +287,51 @@ class LookupFFN(nn.Module):
     FUSED_LAYER_MAX_TOKENS = 512
 
     def can_fuse_layer(self, x):
+        """The one-launch form applies: few tokens, fp32 on the GPU, no gradient wanted, and parameters
+        of the kind it is built for (diagonal BH4, 8-bit codes, 256-entry tables: _fused_params)."""
+        return (x.shape[0] <= self.FUSED_LAYER_MAX_TOKENS and x.is_cuda and x.dtype == torch.float32
+                and not (torch.is_grad_enabled()
+                         and (x.requires_grad or any(q.requires_grad for q in self.parameters())))
+                and self._fused_params() is not None)
+
+    def _fused_params(self):
+        """What the one-launch layer takes from the parameters, or None when their kind rules it out;
+        worked out once and kept until a parameter is replaced, moved or cast (in-place updates keep
+        the storage, so the cached view of the BH4 weight stays good).  The launch is a few
+        microseconds: re-deriving this per call cost more than the kernel."""
         p = self.hash.projection
-        no_grad = not (torch.is_grad_enabled() and (self.tables.requires_grad or self.bias.requires_grad))
-        return (x.shape[0] <= self.FUSED_LAYER_MAX_TOKENS and self.hash.can_fuse(x) and no_grad
-                and p.padded_in_dim >= 256 and self.num_table <= 512 and self.table_size == 256
-                and self.output_size % 4 == 0 and self.tables.dtype == torch.float32
-                and self.bias.dtype == torch.float32)
+        ln = self.LayerNorm
+        params = (ln.weight, ln.bias, getattr(p, "weight", None), getattr(p, "bias", None), self.tables, self.bias)
+        key = tuple((id(q), q.data_ptr(), q.dtype) if q is not None else None for q in params)
+        cached = getattr(self, "_fused_cache", None)
+        if cached is not None and cached[0] == key:
+            return cached[1]
+        ok = (isinstance(p, BH4) and p.block_size == 1 and self.hash.code_length == 8
+              and 256 <= p.padded_in_dim <= 1024 and self.num_table <= 512 and self.table_size == 256
+              and self.output_size % 4 == 0 and ln.elementwise_affine and ln.weight is not None
+              and ln.bias is not None
+              and all(q is None or (q.dtype == torch.float32 and q.is_cuda and q.is_contiguous()
+                                    and q.device == self.tables.device) for q in params))
+        state = None
+        if ok:
+            diag = p.weight.detach().reshape(p.num_repeat, p.weight.shape[1], p.padded_in_dim)
+            state = (ln.weight.detach(), ln.bias.detach(), float(ln.eps), diag,
+                     None if p.bias is None else p.bias.detach(), self.tables.detach(), self.bias.detach(),
+                     float(p.decay_coeff), float(1 - p.decay_coeff))
+        self._fused_cache = (key, state)
+        return state
 
     def _forward(self, hidden_states, residual=None):
+        if self.can_fuse_layer(hidden_states):
+            # small batches without gradient: the whole layer in one launch
+            lw, lb, eps, diag, pbias, tables, obias, decay, res_coef = self._fused_params()
+            return ops.lookup_ffn_fused_direct(hidden_states.contiguous(), lw, lb, eps, diag, pbias, tables,
+                                               obias, None if residual is None else residual.contiguous(),
+                                               decay, res_coef)
         ln = self.LayerNorm
         ln_fusable = (ln.elementwise_affine and ln.weight is not None and ln.bias is not None
                       and ln.weight.dtype == torch.float32
                       and not (torch.is_grad_enabled() and (ln.weight.requires_grad or ln.bias.requires_grad)))
-        if ln_fusable and self.can_fuse_layer(hidden_states):
-            # small batches without gradient: the whole layer in one launch
-            p = self.hash.projection
-            diag = p.weight.reshape(p.num_repeat, p.weight.shape[1], p.padded_in_dim).contiguous()
-            return ops.lookup_ffn_fused(hidden_states.contiguous(), ln.weight, ln.bias, float(ln.eps), diag, p.bias,
-                                        self.tables, self.bias, None if residual is None else residual.contiguous(),
-                                        float(p.decay_coeff), float(1 - p.decay_coeff))
         if ln_fusable and self.hash.can_fuse(hidden_states):
             # inference: LayerNorm runs inside the projection kernel
             code, score = self.hash.forward_fused(hidden_states, layer_norm=ln)

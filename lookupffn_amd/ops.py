@@ -23,7 +23,22 @@ def _is_pow2(v: int) -> bool:
     return v > 0 and (v & (v - 1)) == 0
 
 
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
 def _dev_guard(t: torch.Tensor):
+    """Make t's device current for the launch; free when it already is (the usual case)."""
+    idx = t.device.index
+    if idx is None or idx == torch.cuda.current_device():
+        return _NO_GUARD
     return torch.cuda.device(t.device)
 
 
@@ -328,6 +343,31 @@ def _lookup_ffn_fused_impl(x, ln_w, ln_b, eps, diag, pbias, tables, obias, resid
 
 
 _L.impl("lookup_ffn_fused", _lookup_ffn_fused_impl, "CUDA")
+
+
+def lookup_ffn_fused_direct(x, ln_w, ln_b, eps, diag, pbias, tables, obias, residual, decay, residual_coef):
+    """lookup_ffn_fused for a caller that has already checked the parameters (LookupFFN caches that):
+    no dispatcher, no per-call checks beyond x itself.  The layer's launch is a few microseconds, so
+    at small batches the host side of a call is most of its time."""
+    if torch.compiler.is_compiling():
+        return torch.ops.lookupffn.lookup_ffn_fused(x, ln_w, ln_b, eps, diag, pbias, tables, obias, residual,
+                                                    decay, residual_coef)
+    assert x.dtype == torch.float32 and x.is_cuda and x.is_contiguous() and x.device == tables.device
+    B, H = x.shape
+    R, J, D = diag.shape
+    T, S, Do = tables.shape
+    assert H == ln_w.numel() and (residual is None or (residual.dtype == torch.float32 and residual.is_contiguous()
+                                                        and tuple(residual.shape) == (B, Do)))
+    out = torch.empty((B, Do), dtype=torch.float32, device=x.device)
+    with _dev_guard(x):
+        rc = _lib.load().lffn_lookup_ffn_fused_f32(
+            x.data_ptr(), ln_w.data_ptr(), ln_b.data_ptr(), eps, diag.data_ptr(),
+            None if pbias is None else pbias.data_ptr(), tables.data_ptr(),
+            None if obias is None else obias.data_ptr(), None if residual is None else residual.data_ptr(),
+            out.data_ptr(), B, H, D, R, J, T, S, Do, decay, residual_coef, _lib.stream_of(x))
+    if rc != 0:
+        _lib.check(rc, f"lffn_lookup_ffn_fused_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T}, S={S}, Do={Do})")
+    return out
 
 
 @torch.library.register_fake("lookupffn::lookup_ffn_fused")

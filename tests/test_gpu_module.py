@@ -341,6 +341,54 @@ def test_checkpoint_round_trip_and_folded_weight_cache(tmp_path):
         assert not torch.equal(b(x), out_a)
 
 
+def test_one_launch_layer_follows_its_parameters():
+    """Small batches take the one-launch form, which keeps views of the parameters between calls:
+    they must follow in-place updates, a loaded state dict, a replaced parameter and a cast, and
+    the result must stay that of the two-kernel form (same kernels' arithmetic, same codes)."""
+    torch.manual_seed(33)
+    cfg = _config(hidden_size=256, ffn_num_table=32, block_size=1)
+    layer = lookupffn_amd.LookupFFN(cfg, 256).eval().to(DEV)
+    other = lookupffn_amd.LookupFFN(cfg, 256).eval().to(DEV)
+    x = torch.randn(40, 256, device=DEV)
+    res = torch.randn(40, 256, device=DEV)
+
+    def two_kernels(m, *a):
+        keep = type(m).FUSED_LAYER_MAX_TOKENS
+        type(m).FUSED_LAYER_MAX_TOKENS = 0
+        try:
+            return m(*a)
+        finally:
+            type(m).FUSED_LAYER_MAX_TOKENS = keep
+
+    def check():
+        assert layer.can_fuse_layer(x)
+        got, want = layer(x), two_kernels(layer, x)
+        assert relmax(npf(got), npf(want)) <= 1e-5
+        assert relmax(npf(layer(x, res)), npf(want + res)) <= 1e-5
+        return got
+
+    with torch.no_grad():
+        out0 = check()
+        layer.tables.mul_(2.0)                                  # in place: an optimizer step
+        layer.hash.projection.weight.mul_(-1.0)
+        out1 = check()
+        assert not torch.equal(out0, out1)
+        layer.load_state_dict(other.state_dict())               # copies into the same storage
+        assert torch.equal(check(), other(x))
+        layer.hash.projection.weight = torch.nn.Parameter(layer.hash.projection.weight.detach().clone() * 0.5)
+        layer.tables.data = layer.tables.data.clone() * 3.0     # new storage behind the same Parameter
+        out2 = check()
+        assert not torch.equal(out2, other(x))
+        layer.double()
+        assert not layer.can_fuse_layer(x)                      # fp64 parameters: not this form
+        layer.float()
+        assert relmax(npf(check()), npf(out2)) <= 1e-6
+    xg = x.clone().requires_grad_(True)
+    assert not layer.can_fuse_layer(xg)                         # a gradient is wanted: the differentiable path
+    layer(xg).sum().backward()
+    assert xg.grad is not None and layer.tables.grad is not None
+
+
 # tokens: 256 takes the one-launch form of the layer, 1536 the projection kernel and the table-split
 # gather with its workspace, 4200 (at 16 tables) the projection kernel and the plain gather
 @pytest.mark.parametrize("tokens,tables,width", [(256, 32, 256), (1536, 128, 768), (4200, 16, 256)])
