@@ -286,48 +286,84 @@ class LookupFFN(nn.Module):
     # table-major gather, which stages every table slice in LDS and needs many tokens to pay for it.
     FUSED_LAYER_MAX_TOKENS = 512
 
+    def _no_gradient_wanted(self, x):
+        return not (torch.is_grad_enabled()
+                    and (x.requires_grad or any(q.requires_grad for q in self.parameters())))
+
     def can_fuse_layer(self, x):
         """The one-launch form applies: few tokens, fp32 on the GPU, no gradient wanted, and parameters
-        of the kind it is built for (diagonal BH4, 8-bit codes, 256-entry tables: _fused_params)."""
-        return (x.shape[0] <= self.FUSED_LAYER_MAX_TOKENS and x.is_cuda and x.dtype == torch.float32
-                and not (torch.is_grad_enabled()
-                         and (x.requires_grad or any(q.requires_grad for q in self.parameters())))
-                and self._fused_params() is not None)
+        of the kind it is built for (diagonal BH4, 8-bit codes, 256-entry fp32 tables)."""
+        if not (x.shape[0] <= self.FUSED_LAYER_MAX_TOKENS and x.is_cuda and x.dtype == torch.float32
+                and self._no_gradient_wanted(x)):
+            return False
+        st = self._inference_state()
+        return st is not None and st["one_launch"]
 
-    def _fused_params(self):
-        """What the one-launch layer takes from the parameters, or None when their kind rules it out;
-        worked out once and kept until a parameter is replaced, moved or cast (in-place updates keep
-        the storage, so the cached view of the BH4 weight stays good).  The launch is a few
-        microseconds: re-deriving this per call cost more than the kernel."""
+    def _inference_state(self):
+        """What the inference kernels take from the parameters, or None when the parameters are not of
+        a kind those kernels are built for; worked out once and kept until a parameter is replaced,
+        moved or cast (in-place updates keep the storage, so the cached views stay good).  A launch
+        is a few microseconds: re-deriving this on every call cost more than the kernels at small
+        batches.  Keys: form ("diag": one kernel for LayerNorm + diagonal BH4 + hash; "block": the
+        matrix-core kernel for 64 x 64 blocks), one_launch (the whole layer in one kernel is possible),
+        and the detached parameter views."""
         p = self.hash.projection
         ln = self.LayerNorm
         params = (ln.weight, ln.bias, getattr(p, "weight", None), getattr(p, "bias", None), self.tables, self.bias)
         key = tuple((id(q), q.data_ptr(), q.dtype) if q is not None else None for q in params)
-        cached = getattr(self, "_fused_cache", None)
+        cached = getattr(self, "_inference_cache", None)
         if cached is not None and cached[0] == key:
             return cached[1]
-        ok = (isinstance(p, BH4) and p.block_size == 1 and self.hash.code_length == 8
-              and 256 <= p.padded_in_dim <= 1024 and self.num_table <= 512 and self.table_size == 256
-              and self.output_size % 4 == 0 and ln.elementwise_affine and ln.weight is not None
-              and ln.bias is not None
+        small = (ln.weight, ln.bias, getattr(p, "weight", None), getattr(p, "bias", None), self.bias)
+        ok = (isinstance(p, BH4) and self.hash.code_length == 8 and ln.elementwise_affine
+              and ln.weight is not None and ln.bias is not None and p.in_dim == self.hidden_size
               and all(q is None or (q.dtype == torch.float32 and q.is_cuda and q.is_contiguous()
-                                    and q.device == self.tables.device) for q in params))
+                                    and q.device == self.tables.device) for q in small)
+              and self.tables.is_cuda and self.tables.is_contiguous()
+              and self.tables.dtype in (torch.float32, torch.bfloat16) and self.output_size % 64 == 0)
+        form = None
+        if ok and p.block_size == 1 and 8 <= p.padded_in_dim <= 1024:
+            form = "diag"
+        elif ok and p.block_size == 64 and 64 <= p.padded_in_dim <= 1024 and p.in_dim % 4 == 0:
+            form = "block"
         state = None
-        if ok:
-            diag = p.weight.detach().reshape(p.num_repeat, p.weight.shape[1], p.padded_in_dim)
-            state = (ln.weight.detach(), ln.bias.detach(), float(ln.eps), diag,
-                     None if p.bias is None else p.bias.detach(), self.tables.detach(), self.bias.detach(),
-                     float(p.decay_coeff), float(1 - p.decay_coeff))
-        self._fused_cache = (key, state)
+        if form is not None:
+            state = dict(
+                form=form,
+                one_launch=(form == "diag" and p.padded_in_dim >= 256 and self.num_table <= 512
+                            and self.table_size == 256 and self.tables.dtype == torch.float32),
+                ln_w=ln.weight.detach(), ln_b=ln.bias.detach(), eps=float(ln.eps),
+                diag=(p.weight.detach().reshape(p.num_repeat, p.weight.shape[1], p.padded_in_dim)
+                      if form == "diag" else None),
+                pbias=None if p.bias is None else p.bias.detach(), tables=self.tables.detach(),
+                obias=self.bias.detach(), decay=float(p.decay_coeff), res_coef=float(1 - p.decay_coeff))
+        self._inference_cache = (key, state)
         return state
 
+    def _forward_inference(self, x, residual, st):
+        """No gradient wanted and parameters the inference kernels are built for: the entry points
+        are called without the operator dispatcher or autograd (same kernels, same results)."""
+        x = x.contiguous()
+        if residual is not None:
+            residual = residual.contiguous()
+        if st["one_launch"] and x.shape[0] <= self.FUSED_LAYER_MAX_TOKENS:
+            # small batches: the whole layer in one launch
+            return ops.lookup_ffn_fused_direct(x, st["ln_w"], st["ln_b"], st["eps"], st["diag"], st["pbias"],
+                                               st["tables"], st["obias"], residual, st["decay"], st["res_coef"])
+        if st["form"] == "diag":
+            code, score, _ = ops.ln_project_hash_direct(x, st["ln_w"], st["ln_b"], st["eps"], st["diag"], st["pbias"],
+                                                        self.num_table, st["decay"], st["res_coef"], False)
+        else:
+            code, score = ops.ln_bh4_block_hash_direct(x, st["ln_w"], st["ln_b"], st["eps"], self.hash.folded_weight(),
+                                                       st["pbias"], self.num_table, st["decay"], st["res_coef"])
+        return ops.lookup_gather_direct(code, score, st["tables"], st["obias"], residual)
+
     def _forward(self, hidden_states, residual=None):
-        if self.can_fuse_layer(hidden_states):
-            # small batches without gradient: the whole layer in one launch
-            lw, lb, eps, diag, pbias, tables, obias, decay, res_coef = self._fused_params()
-            return ops.lookup_ffn_fused_direct(hidden_states.contiguous(), lw, lb, eps, diag, pbias, tables,
-                                               obias, None if residual is None else residual.contiguous(),
-                                               decay, res_coef)
+        if (hidden_states.is_cuda and hidden_states.dtype == torch.float32 and not torch.compiler.is_compiling()
+                and self._no_gradient_wanted(hidden_states)):
+            st = self._inference_state()
+            if st is not None:
+                return self._forward_inference(hidden_states, residual, st)
         ln = self.LayerNorm
         ln_fusable = (ln.elementwise_affine and ln.weight is not None and ln.bias is not None
                       and ln.weight.dtype == torch.float32

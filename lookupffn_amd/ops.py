@@ -345,6 +345,21 @@ def _lookup_ffn_fused_impl(x, ln_w, ln_b, eps, diag, pbias, tables, obias, resid
 _L.impl("lookup_ffn_fused", _lookup_ffn_fused_impl, "CUDA")
 
 
+# The inference path of the layer calls the implementations below directly: outside torch.compile
+# the dispatcher adds nothing but a few microseconds per call, which is the larger part of a step
+# at small batches.
+def ln_project_hash_direct(*args):
+    return _ln_project_hash_impl(*args)
+
+
+def ln_bh4_block_hash_direct(*args):
+    return _ln_bh4_block_hash_impl(*args)
+
+
+def lookup_gather_direct(*args):
+    return _lookup_gather_impl(*args)
+
+
 def lookup_ffn_fused_direct(x, ln_w, ln_b, eps, diag, pbias, tables, obias, residual, decay, residual_coef):
     """lookup_ffn_fused for a caller that has already checked the parameters (LookupFFN caches that):
     no dispatcher, no per-call checks beyond x itself.  The layer's launch is a few microseconds, so
