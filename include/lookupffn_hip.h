@@ -167,6 +167,22 @@ int lffn_bh4_block_bwd_f32(const float *g_z, const float *w_folded_t, float *g_x
                            int64_t block_size, float decay, float residual, void *stream);
 
 /*
+ * Column sums of the per-workgroup partial sums that lffn_layer_norm_bwd_f32 and
+ * lffn_project_hash_bwd_f32 leave to the caller, two arrays in one launch:
+ *   out_a[c] = sum_p parts_a[p][c]  (c < n_a),   out_b[c] = sum_p parts_b[p][c]  (c < n_b),
+ * p < num_partials, in a fixed order (reproducible).  n_a, n_b multiples of 4 (n_b == 0: one array).
+ * chunks > 1 splits the rows into that many consecutive chunks of ceil(num_partials / chunks) rows and
+ * writes one row of sums per chunk (out_a: [chunks, n_a], out_b: [chunks, n_b]; no chunk may be
+ * empty): a first pass over a long array (the bias gradient g.sum(0) over all tokens), whose
+ * result a second call with chunks == 1 finishes.
+ * Replaces the column reductions autograd runs for the weight and bias gradients of
+ * torch.nn.LayerNorm (PL/lookup.py:99), of BH4's diagonal weights and bias (PL/lookup.py:29-39) and
+ * of the layer's output bias (PL/lookup.py:108).
+ */
+int lffn_sum_partials_f32(const float *parts_a, float *out_a, int64_t n_a, const float *parts_b, float *out_b,
+                          int64_t n_b, int64_t num_partials, int64_t chunks, void *stream);
+
+/*
  * Backward of the layer's LayerNorm (torch.nn.LayerNorm over the last dimension, PL/lookup.py:84,99)
  * in one kernel; mean and 1/sigma are recomputed from x.
  *   g = sum_r g_y[r];  g_x = rstd * (g*w - mean(g*w) - x^ * mean(g*w*x^));  g_w = sum_b g*x^;  g_b = sum_b g

@@ -107,7 +107,86 @@ __global__ __launch_bounds__(256) void layer_norm_bwd_kernel(LnBwdArgs a) {
     }
 }
 
+// Column sums of up to two arrays of per-workgroup partial sums, parts[p][n] over p, in one launch
+// and in a fixed order (p ascending within a lane, then the 16 lanes of a column group ascending):
+// what the backward kernels' callers need for the weight and bias gradients.  A workgroup owns 64
+// columns; 16 lanes side by side read 256 contiguous bytes of a row, the 16 lane groups take rows
+// 16 apart, eight loads in flight each.
+struct SumPartialsArgs {
+    const float *pa;
+    float *oa;
+    int64_t na;
+    const float *pb;
+    float *ob;
+    int64_t nb;
+    int P;
+    int blocks_a;
+    int rows_per_chunk;    // blockIdx.y = chunk: rows [y * rows_per_chunk, ...) summed into row y of the outputs
+};
+
+__global__ __launch_bounds__(256) void sum_partials_kernel(SumPartialsArgs a) {
+    __shared__ float4 red[16][16];
+    const bool second = (int)blockIdx.x >= a.blocks_a;
+    const float *parts = second ? a.pb : a.pa;
+    float *out = second ? a.ob : a.oa;
+    const int64_t n = second ? a.nb : a.na;
+    const int blk = second ? blockIdx.x - a.blocks_a : blockIdx.x;
+    const int c4 = threadIdx.x & 15, rq = threadIdx.x >> 4;
+    const int64_t col = int64_t(blk) * 64 + c4 * 4;
+    const bool on = col < n;                                  // n % 4 == 0: all four columns or none
+    const int64_t colc = on ? col : 0;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    const int p_begin = blockIdx.y * a.rows_per_chunk, p_end = min(a.P, p_begin + a.rows_per_chunk);
+    for (int p0 = p_begin + rq; p0 < p_end; p0 += 16 * 8) {
+        float4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {                         // unconditional loads at clamped rows
+            const int p = min(p0 + 16 * u, p_end - 1);
+            v[u] = *reinterpret_cast<const float4 *>(parts + int64_t(p) * n + colc);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            if (p0 + 16 * u < p_end) { acc.x += v[u].x; acc.y += v[u].y; acc.z += v[u].z; acc.w += v[u].w; }
+        }
+    }
+    red[rq][c4] = acc;
+    __syncthreads();
+    if (rq == 0 && on) {
+        float4 s = red[0][c4];
+#pragma unroll
+        for (int r = 1; r < 16; ++r) {
+            const float4 q = red[r][c4];
+            s.x += q.x; s.y += q.y; s.z += q.z; s.w += q.w;
+        }
+        *reinterpret_cast<float4 *>(out + int64_t(blockIdx.y) * n + col) = s;
+    }
+}
+
 }  // namespace
+
+extern "C" int lffn_sum_partials_f32(const float *parts_a, float *out_a, int64_t n_a, const float *parts_b,
+                                     float *out_b, int64_t n_b, int64_t num_partials, int64_t chunks,
+                                     void *stream) {
+    LFFN_REQUIRE(n_a >= 0 && n_b >= 0 && num_partials >= 1 && num_partials <= (int64_t(1) << 30), LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(chunks >= 1 && chunks <= 65535 && chunks <= num_partials, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(n_a % 4 == 0 && n_b % 4 == 0 && n_a <= (int64_t(1) << 30) && n_b <= (int64_t(1) << 30),
+                 LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE((n_a == 0 || (parts_a && out_a)) && (n_b == 0 || (parts_b && out_b)), LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_aligned16(parts_a) && lffn_aligned16(out_a) && lffn_aligned16(parts_b) && lffn_aligned16(out_b),
+                 LFFN_ERR_BAD_ARG);
+    if (n_a + n_b == 0) return LFFN_OK;
+    SumPartialsArgs a{};
+    a.pa = parts_a; a.oa = out_a; a.na = n_a; a.pb = parts_b; a.ob = out_b; a.nb = n_b; a.P = (int)num_partials;
+    a.blocks_a = (int)((n_a + 63) / 64);
+    a.rows_per_chunk = (int)((num_partials + chunks - 1) / chunks);
+    const int blocks = a.blocks_a + (int)((n_b + 63) / 64);
+    // every chunk has rows: chunks <= num_partials and rows_per_chunk = ceil, so the last chunk may be
+    // short but (chunks - 1) * rows_per_chunk < num_partials must hold for it not to be empty
+    LFFN_REQUIRE((chunks - 1) * (int64_t)a.rows_per_chunk < num_partials, LFFN_ERR_BAD_ARG);
+    hipLaunchKernelGGL(sum_partials_kernel, dim3((unsigned)blocks, (unsigned)chunks), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), a);
+    return lffn_launch_status();
+}
 
 extern "C" int lffn_layer_norm_bwd_f32(const float *x, const float *ln_weight, float ln_eps, const float *g_y,
                                        float *g_x, float *part_weight, float *part_bias, int64_t B, int64_t H,

@@ -152,7 +152,7 @@ class LookupGather(Function):
         T, S, Do = tables.shape
         grad_score = ops.lookup_inner(code, grad_outputs, tables) if ctx.needs_input_grad[1] else None
         grad_tables = ops.lookup_scatter(code, score, grad_outputs, S) if ctx.needs_input_grad[2] else None
-        grad_bias = grad_outputs.sum(dim=0) if (ctx.has_bias and ctx.needs_input_grad[3]) else None
+        grad_bias = ops.column_sums(grad_outputs) if (ctx.has_bias and ctx.needs_input_grad[3]) else None
         grad_residual = grad_outputs if (ctx.has_residual and ctx.needs_input_grad[4]) else None
         return None, grad_score, grad_tables, grad_bias, grad_residual
 

@@ -128,7 +128,7 @@ class BlockProjectHash(torch.autograd.Function):
             g_folded = ops.bh4_block_wgrad(stage_g.reshape(R * J, B, NB * bs), x, stage_in, R, J).view_as(w)
             g_w = ops.bh4_fold_mode(g_folded, 2)
         g_x = g_x[0] if R == 1 else g_x.sum(0)
-        g_bias = g_z.sum(0) if (ctx.has_bias and ctx.needs_input_grad[2]) else None
+        g_bias = ops.column_sums(g_z) if (ctx.has_bias and ctx.needs_input_grad[2]) else None
         return (g_x if ctx.needs_input_grad[0] else None, g_w, g_bias, None, None)
 
 

@@ -42,6 +42,45 @@ def _dev_guard(t: torch.Tensor):
     return torch.cuda.device(t.device)
 
 
+def _sum_partials(parts_a: torch.Tensor, parts_b: torch.Tensor = None):
+    """Column sums of one or two [P, n] arrays of per-workgroup partial sums in one launch, fixed
+    order of additions (the backward kernels' weight and bias gradients)."""
+    P, na = parts_a.shape
+    nb = 0 if parts_b is None else parts_b.shape[1]
+    assert parts_a.is_contiguous() and (parts_b is None or (parts_b.is_contiguous() and parts_b.shape[0] == P))
+    if P > COLUMN_SUM_CHUNK_ROWS * 4:
+        # many rows (a gradient over all tokens): a first pass over chunks of rows on many workgroups
+        chunks = (P + COLUMN_SUM_CHUNK_ROWS - 1) // COLUMN_SUM_CHUNK_ROWS
+        chunks = (P + ((P + chunks - 1) // chunks) - 1) // ((P + chunks - 1) // chunks)     # no empty chunk
+        mid_a = torch.empty(chunks, na, dtype=torch.float32, device=parts_a.device)
+        mid_b = None if parts_b is None else torch.empty(chunks, nb, dtype=torch.float32, device=parts_a.device)
+        with _dev_guard(parts_a):
+            rc = _lib.load().lffn_sum_partials_f32(_lib.ptr(parts_a), _lib.ptr(mid_a), na, _lib.ptr(parts_b),
+                                                   _lib.ptr(mid_b), nb, P, chunks, _lib.stream_of(parts_a))
+        _lib.check(rc, f"lffn_sum_partials_f32(P={P}, n_a={na}, n_b={nb}, chunks={chunks})")
+        parts_a, parts_b, P = mid_a, mid_b, chunks
+    out_a = torch.empty(na, dtype=torch.float32, device=parts_a.device)
+    out_b = None if parts_b is None else torch.empty(nb, dtype=torch.float32, device=parts_a.device)
+    with _dev_guard(parts_a):
+        rc = _lib.load().lffn_sum_partials_f32(_lib.ptr(parts_a), _lib.ptr(out_a), na, _lib.ptr(parts_b),
+                                               _lib.ptr(out_b), nb, P, 1, _lib.stream_of(parts_a))
+    _lib.check(rc, f"lffn_sum_partials_f32(P={P}, n_a={na}, n_b={nb})")
+    return out_a, out_b
+
+
+COLUMN_SUM_CHUNK_ROWS = 256
+
+
+def column_sums(g: torch.Tensor) -> torch.Tensor:
+    """g.sum(0) of a contiguous fp32 [B, n] array on the GPU with n % 4 == 0 (a bias gradient over all
+    tokens), reproducible; other inputs go to torch."""
+    if (g.is_cuda and g.dim() == 2 and g.dtype == torch.float32 and g.is_contiguous() and g.shape[1] % 4 == 0
+            and 1 <= g.shape[0] <= 65535 * COLUMN_SUM_CHUNK_ROWS and g.data_ptr() % 16 == 0
+            and not torch.compiler.is_compiling()):
+        return _sum_partials(g)[0]
+    return g.sum(dim=0)
+
+
 # ----------------------------------------------------------------------------- fht
 
 _L.define("fht(Tensor x) -> Tensor")
@@ -411,8 +450,8 @@ def _layer_norm_bwd_impl(x, weight, eps, g_y):
         rc = _lib.load().lffn_layer_norm_bwd_f32(_lib.ptr(x), _lib.ptr(weight), eps, _lib.ptr(g_y), _lib.ptr(g_x),
                                                  _lib.ptr(part[0]), _lib.ptr(part[1]), B, H, R, n, _lib.stream_of(x))
     _lib.check(rc, f"lffn_layer_norm_bwd_f32(B={B}, H={H}, R={R})")
-    sums = part.sum(1)
-    return g_x, sums[0], sums[1]
+    g_w, g_b = _sum_partials(part[0], part[1])
+    return g_x, g_w, g_b
 
 
 _L.impl("layer_norm_bwd", _layer_norm_bwd_impl, "CUDA")
@@ -522,7 +561,8 @@ def _project_hash_bwd_impl(x, diag, z, g_score, decay, residual):
         _lib.check(rc, f"lffn_project_hash_bwd_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T})")
     else:
         part_d.zero_(); part_b.zero_()
-    return (g_x[0] if R == 1 else g_x.sum(0)), part_d.sum(0), part_b.sum(0)[:T * 8]
+    g_d, g_b = _sum_partials(part_d.view(nparts, R * J * D), part_b)
+    return (g_x[0] if R == 1 else g_x.sum(0)), g_d.view(R, J, D), g_b[:T * 8]
 
 
 _L.impl("project_hash_bwd", _project_hash_bwd_impl, "CUDA")

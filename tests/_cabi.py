@@ -336,3 +336,16 @@ def lookup_inner(code, g, tables):
     out = torch.full((B, T), float("nan"), dtype=torch.float32, device=DEV)   # must be fully overwritten
     _call("lffn_lookup_inner_f32", p(cd), p(gd), p(td), p(out), B, T, S, Do)
     return host(out)
+
+
+def sum_partials(parts_a, parts_b=None, chunks=1):
+    """-> column sums of one or two [P, n] arrays, one row of sums per chunk of rows."""
+    ad, bd = dev(parts_a), dev(parts_b)
+    P, na = parts_a.shape
+    nb = 0 if parts_b is None else parts_b.shape[1]
+    oa = torch.full((chunks, na), float("nan"), dtype=torch.float32, device=DEV)
+    ob = None if parts_b is None else torch.full((chunks, nb), float("nan"), dtype=torch.float32, device=DEV)
+    _call("lffn_sum_partials_f32", p(ad), p(oa), na, p(bd), p(ob), nb, P, chunks)
+    if chunks == 1:
+        return host(oa)[0], (None if ob is None else host(ob)[0])
+    return host(oa), (None if ob is None else host(ob))

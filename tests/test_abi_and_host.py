@@ -88,6 +88,14 @@ def test_argument_validation_of_the_backward_and_block_entry_points():
                                           0.7, 0.3, None) == A                      # LayerNorm weight without bias
     assert lib.lffn_ln_bh4_block_hash_f32(P, None, None, 0.0, P, None, P, P, 0, 768, 1024, 1, 4, 128, 64,
                                           0.7, 0.3, None) == OK
+    # column sums of partial sums
+    assert lib.lffn_sum_partials_f32(P, P, 6, None, None, 0, 16, 1, None) == U          # n % 4
+    assert lib.lffn_sum_partials_f32(P, P, 8, None, None, 4, 16, 1, None) == A          # second array missing
+    assert lib.lffn_sum_partials_f32(P, P + 4, 8, None, None, 0, 16, 1, None) == A      # misaligned
+    assert lib.lffn_sum_partials_f32(P, P, 8, None, None, 0, 0, 1, None) == A           # no partials
+    assert lib.lffn_sum_partials_f32(P, P, 8, None, None, 0, 16, 17, None) == A         # more chunks than rows
+    assert lib.lffn_sum_partials_f32(P, P, 8, None, None, 0, 10, 8, None) == A          # ceil(10/8) = 2 rows: chunk 5.. empty
+    assert lib.lffn_sum_partials_f32(None, None, 0, None, None, 0, 16, 1, None) == OK   # nothing to add
     # mix + hash
     assert lib.lffn_mix_code_score_f32(P, P, None, P, P, 4, 8, 25, 64, 64, 256, 0.7, 0.3, None) == U   # k > 24
     assert lib.lffn_mix_code_score_f32(P, P, None, P, P, 4, 40, 8, 64, 64, 256, 0.7, 0.3, None) == A   # T*k > ldy

@@ -477,6 +477,48 @@ def test_ln_project_hash_matches_oracle(H, D, R, T):
     assert np.abs(z - z2).max() <= 1e-5 * scale
 
 
+@pytest.mark.parametrize("P,na,nb", [(1, 4, 0), (7, 64, 100), (512, 768, 768), (512, 4096, 1024), (1000, 260, 4),
+                                      (129, 0, 72), (16, 8, 0)])
+def test_sum_partials_matches_float64(P, na, nb):
+    """The column sums of the backward kernels' partial sums: against float64, and bit-identical
+    from call to call (fixed order of additions)."""
+    rng = np.random.RandomState(P + na + nb)
+    a = rng.randn(P, na).astype(np.float32)
+    b = rng.randn(P, nb).astype(np.float32) if nb else None
+    if na == 0:                                   # the first array may be the empty one
+        got_b, _ = cabi.sum_partials(b)
+        got_a = np.zeros(0, dtype=np.float32)
+    else:
+        got_a, got_b = cabi.sum_partials(a, b)
+    assert got_a.shape == (na,)
+    if na:
+        want = a.astype(np.float64).sum(0)
+        assert np.abs(got_a - want).max() <= 1e-6 * max(1.0, np.abs(a).sum(0).max())
+        again, _ = cabi.sum_partials(a, b)
+        assert np.array_equal(again, got_a)
+    if nb:
+        want = b.astype(np.float64).sum(0)
+        assert np.abs(got_b - want).max() <= 1e-6 * max(1.0, np.abs(b).sum(0).max())
+
+
+@pytest.mark.parametrize("P,n,chunks", [(1000, 68, 4), (16384, 768, 64), (257, 8, 257), (5000, 128, 7)])
+def test_sum_partials_in_chunks_and_column_sums(P, n, chunks):
+    """chunks > 1: one row of sums per chunk of ceil(P / chunks) consecutive rows (the first pass over
+    a gradient with many rows); the package's column_sums strings two passes together."""
+    rng = np.random.RandomState(P + n)
+    a = rng.randn(P, n).astype(np.float32)
+    rows = -(-P // chunks)
+    if (chunks - 1) * rows >= P:
+        pytest.skip("an empty chunk: rejected by the entry point")
+    got, _ = cabi.sum_partials(a, chunks=chunks)
+    want = np.stack([a[c * rows:(c + 1) * rows].astype(np.float64).sum(0) for c in range(chunks)])
+    assert got.shape == (chunks, n)
+    assert np.abs(got - want).max() <= 1e-6 * np.abs(a).sum(0).max()
+    from lookupffn_amd import ops
+    s = ops.column_sums(torch.tensor(a, device="cuda:0")).cpu().numpy()
+    assert np.abs(s - a.astype(np.float64).sum(0)).max() <= 1e-6 * np.abs(a).sum(0).max()
+
+
 def test_project_hash_near_zero_flip_count():
     # end to end against the float64 truth: flips may only happen where |z| is tiny
     rng = np.random.RandomState(9)
