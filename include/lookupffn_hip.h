@@ -99,6 +99,20 @@ int lffn_project_hash_bwd_f32(const float *x, const float *diag, const float *z,
                               float decay, float residual, void *stream);
 
 /*
+ * lffn_ln_project_hash_bwd_f32: the same for the forward with LayerNorm inside
+ * (lffn_ln_project_hash_f32 with z kept): h = LayerNorm(x; ln_weight, ln_bias, ln_eps) is formed on
+ * load as in that forward, and g_h [R, B, H] is the gradient w.r.t. h, which
+ * lffn_layer_norm_bwd_f32 takes on to x and the LayerNorm parameters (it adds the R slabs itself).
+ * Replaces what autograd records for self.LayerNorm's output feeding BH4._forward +
+ * compute_code_score_torch (PL/lookup.py:99,29-39): the normalised activations are never stored.
+ */
+int lffn_ln_project_hash_bwd_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
+                                 const float *diag, const float *z, const float *g_score, float *g_h,
+                                 float *part_diag, float *part_bias, int64_t B, int64_t H, int64_t D, int64_t R,
+                                 int64_t J, int64_t T, int64_t num_partials, float decay, float residual,
+                                 void *stream);
+
+/*
  * BH4 mixing with 64 x 64 blocks, all stages of a repeat in one kernel:
  *   for r < R:  y = pad(x);  for j < J:  y = FHT(blockdiag(w[r,j]) y);  out[b, r*D:(r+1)*D] = y
  * x: [B, H], H <= D, H % 4 == 0 (zero-padded on load, PL/lookup.py:32-34);

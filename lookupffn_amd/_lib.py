@@ -52,6 +52,8 @@ SIGNATURES = {
     "lffn_project_hash_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _vp],
     "lffn_ln_project_hash_f32": [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _vp,
                                  _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _vp],
+    "lffn_ln_project_hash_bwd_f32": [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _vp, _vp,
+                                     _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _vp],
     "lffn_sum_partials_f32": [_vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _vp],
     "lffn_code_score_f32": [_vp, _vp, _vp, _i64, _i64, _vp],
     "lffn_code_score_bwd_f32": [_vp, _vp, _vp, _i64, _i64, _vp],

@@ -152,6 +152,7 @@ struct ProjectArgs {
     float decay, residual;
     int mix;              // 1: out = decay*y + residual*x (+ bias); 0: out = y
     int vec_in;           // x rows are 16-byte aligned and H % 4 == 0
+    int vec_ln;           // and so are ln_w and ln_b: the LayerNorm parameters load as float4
     // GATHER only: the table rows the codes select are added up in the same kernel
     const float *tables;  // [T, S, Do]
     const float *obias;   // [Do] or null
@@ -290,13 +291,28 @@ __global__ __launch_bounds__(256) void project_kernel(ProjectArgs a) {
                 s2 += dlt * dlt;
             }
         const float rstd = 1.0f / sqrtf(lane_group_sum<LPR>(s2) / float(a.H) + a.ln_eps);
+        if (a.vec_ln) {                                       // H % 4 == 0: a float4 of weights and biases per lane
 #pragma unroll
-        for (int j = 0; j < NJ; ++j)
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const int e = 256 * j + 4 * lr + c;
-                if (e < a.H) orig[j][c] = (orig[j][c] - mean) * rstd * a.ln_w[e] + a.ln_b[e];
+            for (int j = 0; j < NJ; ++j) {
+                const int e0 = 256 * j + 4 * lr;
+                if (e0 < a.H) {
+                    const float4 lw = *reinterpret_cast<const float4 *>(a.ln_w + e0);
+                    const float4 lb = *reinterpret_cast<const float4 *>(a.ln_b + e0);
+                    orig[j][0] = (orig[j][0] - mean) * rstd * lw.x + lb.x;
+                    orig[j][1] = (orig[j][1] - mean) * rstd * lw.y + lb.y;
+                    orig[j][2] = (orig[j][2] - mean) * rstd * lw.z + lb.z;
+                    orig[j][3] = (orig[j][3] - mean) * rstd * lw.w + lb.w;
+                }
             }
+        } else {
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const int e = 256 * j + 4 * lr + c;
+                    if (e < a.H) orig[j][c] = (orig[j][c] - mean) * rstd * a.ln_w[e] + a.ln_b[e];
+                }
+        }
     }
 
     for (int r = 0; r < a.R; ++r) {
@@ -453,6 +469,9 @@ struct ProjectBwdArgs {
     int64_t B;
     int H, R, J, T;
     float decay, residual;
+    const float *ln_w;     // [H] or null: the projection's input is LayerNorm(x; ln_w, ln_b, ln_eps), formed on
+    const float *ln_b;     // load as in the forward; g_x is then the gradient w.r.t. that LayerNorm output
+    float ln_eps;
 };
 
 template <int LOGD>
@@ -490,6 +509,37 @@ __global__ __launch_bounds__(256) void project_hash_bwd_kernel(ProjectBwdArgs a)
             float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
             if (e0 < a.H) v = *reinterpret_cast<const float4 *>(a.x + row * a.H + e0);
             t[j][0] = v.x; t[j][1] = v.y; t[j][2] = v.z; t[j][3] = v.w;
+        }
+        if (a.ln_w) {                                         // uniform
+            // LayerNorm over the H valid columns exactly as project_kernel forms it (biased variance,
+            // two passes, eps inside the square root; padding columns stay zero)
+            float s1 = 0.f;
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) s1 += t[j][c];
+            const float mean = lane_group_sum<64>(s1) / float(a.H);
+            float s2 = 0.f;
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const float dlt = (256 * j + 4 * lr + c < a.H) ? t[j][c] - mean : 0.f;
+                    s2 += dlt * dlt;
+                }
+            const float rstd = 1.0f / sqrtf(lane_group_sum<64>(s2) / float(a.H) + a.ln_eps);
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                const int e0 = 256 * j + 4 * lr;
+                if (e0 < a.H) {                               // H % 4 == 0: all four columns or none
+                    const float4 lw = *reinterpret_cast<const float4 *>(a.ln_w + e0);
+                    const float4 lb = *reinterpret_cast<const float4 *>(a.ln_b + e0);
+                    t[j][0] = (t[j][0] - mean) * rstd * lw.x + lb.x;
+                    t[j][1] = (t[j][1] - mean) * rstd * lw.y + lb.y;
+                    t[j][2] = (t[j][2] - mean) * rstd * lw.z + lb.z;
+                    t[j][3] = (t[j][3] - mean) * rstd * lw.w + lb.w;
+                }
+            }
         }
 #pragma unroll
         for (int s = 0; s < MAXJ; ++s) {
@@ -759,6 +809,7 @@ static int project_hash_impl(const float *x, const float *ln_w, const float *ln_
     a.out_stride = (int)(T * 8); a.out_cols = (int)(T * 8); a.T = (int)T;
     a.decay = decay; a.residual = residual; a.mix = 1;
     a.vec_in = (lffn_aligned16(x) && H % 4 == 0) ? 1 : 0;
+    a.vec_ln = (H % 4 == 0 && ln_w && lffn_aligned16(ln_w) && lffn_aligned16(ln_b)) ? 1 : 0;
     return launch_project<true>(a, lffn_log2(D), static_cast<hipStream_t>(stream));
 }
 
@@ -785,6 +836,7 @@ extern "C" int lffn_lookup_ffn_fused_f32(const float *x, const float *ln_weight,
     a.out_stride = (int)(T * 8); a.out_cols = (int)(T * 8); a.T = (int)T;
     a.decay = decay; a.residual = residual; a.mix = 1;
     a.vec_in = (lffn_aligned16(x) && H % 4 == 0) ? 1 : 0;
+    a.vec_ln = (H % 4 == 0 && ln_weight && lffn_aligned16(ln_weight) && lffn_aligned16(ln_bias)) ? 1 : 0;
     a.tables = tables; a.obias = out_bias; a.gres = residual_in; a.gout = out; a.S = (int)S; a.Do = (int)Do;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const dim3 grid((unsigned)B);                       // one token per workgroup
@@ -804,10 +856,36 @@ extern "C" int lffn_fht_bf16(const uint16_t *in, uint16_t *out, int64_t B, int64
     return fht16_entry<true>(in, out, B, D, stream);
 }
 
+static int project_hash_bwd_impl(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
+                                 const float *diag, const float *z, const float *g_score,
+                                 float *g_x, float *part_diag, float *part_bias, int64_t B, int64_t H,
+                                 int64_t D, int64_t R, int64_t J, int64_t T, int64_t num_partials,
+                                 float decay, float residual, void *stream);
+
 extern "C" int lffn_project_hash_bwd_f32(const float *x, const float *diag, const float *z, const float *g_score,
                                          float *g_x, float *part_diag, float *part_bias, int64_t B, int64_t H,
                                          int64_t D, int64_t R, int64_t J, int64_t T, int64_t num_partials,
                                          float decay, float residual, void *stream) {
+    return project_hash_bwd_impl(x, nullptr, nullptr, 0.f, diag, z, g_score, g_x, part_diag, part_bias, B, H, D, R,
+                                 J, T, num_partials, decay, residual, stream);
+}
+
+extern "C" int lffn_ln_project_hash_bwd_f32(const float *x, const float *ln_weight, const float *ln_bias,
+                                            float ln_eps, const float *diag, const float *z,
+                                            const float *g_score, float *g_h, float *part_diag, float *part_bias,
+                                            int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
+                                            int64_t num_partials, float decay, float residual, void *stream) {
+    LFFN_REQUIRE(ln_weight && ln_bias && ln_eps >= 0.f, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_aligned16(ln_weight) && lffn_aligned16(ln_bias), LFFN_ERR_BAD_ARG);
+    return project_hash_bwd_impl(x, ln_weight, ln_bias, ln_eps, diag, z, g_score, g_h, part_diag, part_bias, B, H, D,
+                                 R, J, T, num_partials, decay, residual, stream);
+}
+
+static int project_hash_bwd_impl(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
+                                 const float *diag, const float *z, const float *g_score,
+                                 float *g_x, float *part_diag, float *part_bias, int64_t B, int64_t H,
+                                 int64_t D, int64_t R, int64_t J, int64_t T, int64_t num_partials,
+                                 float decay, float residual, void *stream) {
     int rc = check_dims(B, H, D, R, J);
     if (rc != LFFN_OK) return rc;
     LFFN_REQUIRE(D >= 256 && J >= 1 && J <= 4 && H % 4 == 0 && R <= 65535, LFFN_ERR_UNSUPPORTED);
@@ -818,6 +896,7 @@ extern "C" int lffn_project_hash_bwd_f32(const float *x, const float *diag, cons
     ProjectBwdArgs a{};
     a.x = x; a.diag = diag; a.z = z; a.g_score = g_score; a.g_x = g_x; a.part_d = part_diag; a.part_b = part_bias;
     a.B = B; a.H = (int)H; a.R = (int)R; a.J = (int)J; a.T = (int)T; a.decay = decay; a.residual = residual;
+    a.ln_w = ln_weight; a.ln_b = ln_bias; a.ln_eps = ln_eps;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const dim3 grid((unsigned)num_partials, (unsigned)R);
     switch (lffn_log2(D)) {

@@ -261,6 +261,41 @@ class LayerNormFn(torch.autograd.Function):
                 g_b if ctx.needs_input_grad[2] else None, None)
 
 
+class LnProjectHash(torch.autograd.Function):
+    """LayerNorm -> diagonal BH4 -> mix -> bias -> 8-bit code + score as one differentiable operator
+    (PL/lookup.py:99, 29-39, PL/compute_code_score/kernel.py:47-53).  Forward: the inference kernel
+    with z kept.  Backward: the projection's backward with LayerNorm recomputed on load, then the
+    LayerNorm backward kernel; the normalised activations are never stored."""
+
+    @staticmethod
+    def forward(ctx, x, ln_weight, ln_bias, eps, weight, bias, T, decay):
+        R, J = weight.shape[0], weight.shape[1]
+        diag = weight.reshape(R, J, -1).contiguous()
+        x = x.contiguous()
+        code, score, z = ops.ln_project_hash(x, ln_weight, ln_bias, float(eps), diag, bias, T, float(decay),
+                                             float(1 - decay), True)
+        ctx.save_for_backward(x, ln_weight, ln_bias, diag, z)
+        ctx.eps = float(eps)
+        ctx.weight_shape = weight.shape
+        ctx.has_bias = bias is not None
+        ctx.decay = float(decay)
+        ctx.mark_non_differentiable(code)
+        return code, score
+
+    @staticmethod
+    def backward(ctx, _g_code, g_score):
+        x, ln_weight, ln_bias, diag, z = ctx.saved_tensors
+        g_h, g_diag, g_bias = ops.project_hash_bwd(x, diag, z, g_score.contiguous(), ctx.decay, 1 - ctx.decay,
+                                                   ln_weight, ln_bias, ctx.eps)
+        need = ctx.needs_input_grad
+        g_x = g_lw = g_lb = None
+        if need[0] or need[1] or need[2]:
+            g_x, g_lw, g_lb = ops.layer_norm_bwd(x, ln_weight, ctx.eps, g_h)
+        return (g_x if need[0] else None, g_lw if need[1] else None, g_lb if need[2] else None, None,
+                g_diag.reshape(ctx.weight_shape) if need[4] else None,
+                g_bias if (ctx.has_bias and need[5]) else None, None, None)
+
+
 class LookupFFN(nn.Module):
     """PL/lookup.py:79-130."""
 
@@ -374,13 +409,21 @@ class LookupFFN(nn.Module):
         elif ln_fusable and self.hash.can_fuse_block(hidden_states):
             code, score = self.hash.forward_block(hidden_states, layer_norm=ln)
         else:
-            if (torch.is_grad_enabled() and hidden_states.is_cuda and hidden_states.dtype == torch.float32
-                    and ln.elementwise_affine and ln.weight is not None and ln.bias is not None
-                    and ln.weight.dtype == torch.float32 and self.hidden_size % 4 == 0 and self.hidden_size <= 1024):
+            ln_kernel_ok = (torch.is_grad_enabled() and hidden_states.is_cuda and hidden_states.dtype == torch.float32
+                            and ln.elementwise_affine and ln.weight is not None and ln.bias is not None
+                            and ln.weight.dtype == torch.float32 and self.hidden_size % 4 == 0
+                            and self.hidden_size <= 1024)
+            if ln_kernel_ok and self.hash.can_fuse_training(hidden_states):
+                # training, diagonal BH4: LayerNorm inside the projection kernel forward and backward
+                p = self.hash.projection
+                code, score = LnProjectHash.apply(hidden_states, ln.weight, ln.bias, ln.eps, p.weight, p.bias,
+                                                  self.num_table, p.decay_coeff)
+            elif ln_kernel_ok:
                 hidden_states = LayerNormFn.apply(hidden_states.contiguous(), ln.weight, ln.bias, ln.eps)
+                code, score = self.hash(hidden_states)
             else:
                 hidden_states = ln(hidden_states)
-            code, score = self.hash(hidden_states)
+                code, score = self.hash(hidden_states)
         if self.output_size % 64 == 0 and self.tables.dtype in (torch.float32, torch.bfloat16):
             # table-local codes, offset and bias folded into the gather kernel
             return lookup_gather(code, score.float(), self.tables, self.bias.float(), residual)

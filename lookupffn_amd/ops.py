@@ -534,17 +534,20 @@ def _(x, diag, bias, T, decay, residual, keep_z):
             x.new_empty((B, T * 8) if keep_z else (0,)))
 
 
-_L.define("project_hash_bwd(Tensor x, Tensor diag, Tensor z, Tensor g_score, float decay, float residual)"
-          " -> (Tensor, Tensor, Tensor)")
+_L.define("project_hash_bwd(Tensor x, Tensor diag, Tensor z, Tensor g_score, float decay, float residual, "
+          "Tensor? ln_weight=None, Tensor? ln_bias=None, float ln_eps=0.0) -> (Tensor, Tensor, Tensor)")
 
 PROJECT_BWD_PARTIALS = 512      # workgroups per repeat: two per compute unit
 
 
-def _project_hash_bwd_impl(x, diag, z, g_score, decay, residual):
-    """-> (grad x [B,H], grad diag [R,J,D], grad bias [T*8])."""
-    _lib.require_gpu(x, diag, z, g_score)
-    for t in (x, diag, z, g_score):
-        assert t.dtype == torch.float32 and t.is_contiguous()
+def _project_hash_bwd_impl(x, diag, z, g_score, decay, residual, ln_weight=None, ln_bias=None, ln_eps=0.0):
+    """-> (grad x [B,H], grad diag [R,J,D], grad bias [T*8]).  With ln_weight / ln_bias the projection's
+    input is LayerNorm(x), formed on load, and the first result is [R,B,H]: the gradient w.r.t. that
+    LayerNorm output, one slab per repeat (layer_norm_bwd adds them)."""
+    _lib.require_gpu(x, diag, z, g_score, ln_weight, ln_bias)
+    for t in (x, diag, z, g_score, ln_weight, ln_bias):
+        assert t is None or (t.dtype == torch.float32 and t.is_contiguous())
+    assert (ln_weight is None) == (ln_bias is None)
     B, H = x.shape
     R, J, D = diag.shape
     T = g_score.shape[1]
@@ -553,7 +556,15 @@ def _project_hash_bwd_impl(x, diag, z, g_score, decay, residual):
     g_x = torch.empty(R, B, H, dtype=torch.float32, device=x.device)
     part_d = torch.empty(nparts, R, J, D, dtype=torch.float32, device=x.device)
     part_b = torch.empty(nparts, R * D, dtype=torch.float32, device=x.device)
-    if B > 0:
+    if B > 0 and ln_weight is not None:
+        assert ln_weight.numel() == H and ln_bias.numel() == H
+        with _dev_guard(x):
+            rc = _lib.load().lffn_ln_project_hash_bwd_f32(
+                _lib.ptr(x), _lib.ptr(ln_weight), _lib.ptr(ln_bias), ln_eps, _lib.ptr(diag), _lib.ptr(z),
+                _lib.ptr(g_score), _lib.ptr(g_x), _lib.ptr(part_d), _lib.ptr(part_b), B, H, D, R, J, T, nparts,
+                decay, residual, _lib.stream_of(x))
+        _lib.check(rc, f"lffn_ln_project_hash_bwd_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T})")
+    elif B > 0:
         with _dev_guard(x):
             rc = _lib.load().lffn_project_hash_bwd_f32(
                 _lib.ptr(x), _lib.ptr(diag), _lib.ptr(z), _lib.ptr(g_score), _lib.ptr(g_x), _lib.ptr(part_d),
@@ -562,6 +573,8 @@ def _project_hash_bwd_impl(x, diag, z, g_score, decay, residual):
     else:
         part_d.zero_(); part_b.zero_()
     g_d, g_b = _sum_partials(part_d.view(nparts, R * J * D), part_b)
+    if ln_weight is not None:
+        return g_x, g_d.view(R, J, D), g_b[:T * 8]
     return (g_x[0] if R == 1 else g_x.sum(0)), g_d.view(R, J, D), g_b[:T * 8]
 
 
@@ -569,8 +582,9 @@ _L.impl("project_hash_bwd", _project_hash_bwd_impl, "CUDA")
 
 
 @torch.library.register_fake("lookupffn::project_hash_bwd")
-def _(x, diag, z, g_score, decay, residual):
-    return torch.empty_like(x), torch.empty_like(diag), x.new_empty(z.shape[1])
+def _(x, diag, z, g_score, decay, residual, ln_weight=None, ln_bias=None, ln_eps=0.0):
+    g_x = torch.empty_like(x) if ln_weight is None else x.new_empty((diag.shape[0],) + tuple(x.shape))
+    return g_x, torch.empty_like(diag), x.new_empty(z.shape[1])
 
 
 _L.define("ln_project_hash(Tensor x, Tensor ln_weight, Tensor ln_bias, float eps, Tensor diag, Tensor? bias, "

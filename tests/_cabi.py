@@ -349,3 +349,23 @@ def sum_partials(parts_a, parts_b=None, chunks=1):
     if chunks == 1:
         return host(oa)[0], (None if ob is None else host(ob)[0])
     return host(oa), (None if ob is None else host(ob))
+
+
+def project_hash_bwd(x, diag, z, g_score, ln_w=None, ln_b=None, eps=1e-5, decay=0.7, nparts=64):
+    """-> g_x [R, B, H] (w.r.t. the LayerNorm output when ln_w is given), grad diag [R, J, D], grad bias [R*D]."""
+    xd, dd, zd, gd, lw, lb = dev(x), dev(diag), dev(z), dev(g_score), dev(ln_w), dev(ln_b)
+    B, H = x.shape
+    R, J, D = diag.shape
+    T = g_score.shape[1]
+    g_x = torch.full((R, B, H), float("nan"), dtype=torch.float32, device=DEV)
+    part_d = torch.full((nparts, R, J, D), float("nan"), dtype=torch.float32, device=DEV)
+    part_b = torch.full((nparts, R * D), float("nan"), dtype=torch.float32, device=DEV)
+    dc, rc = float(np.float32(decay)), float(np.float32(1 - decay))
+    if ln_w is None:
+        _call("lffn_project_hash_bwd_f32", p(xd), p(dd), p(zd), p(gd), p(g_x), p(part_d), p(part_b),
+              B, H, D, R, J, T, nparts, dc, rc)
+    else:
+        _call("lffn_ln_project_hash_bwd_f32", p(xd), p(lw), p(lb), float(np.float32(eps)), p(dd), p(zd), p(gd), p(g_x),
+              p(part_d), p(part_b), B, H, D, R, J, T, nparts, dc, rc)
+    torch.cuda.synchronize()
+    return host(g_x), part_d.double().sum(0).cpu().numpy(), part_b.double().sum(0).cpu().numpy()

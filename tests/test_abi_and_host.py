@@ -119,6 +119,10 @@ def test_argument_validation_of_the_backward_and_block_entry_points():
     assert lib.lffn_bh4_block_wgrad_f32(P, P, P, P, 0, 768, 1024, 1, 4, 64, None) == OK
     assert lib.lffn_project_hash_bwd_f32(P, P, P, P, P, P, P, 4, 64, 64, 1, 4, 8, 1, 0.7, 0.3, None) == U   # D < 256
     assert lib.lffn_project_hash_bwd_f32(P, P, P, P, P, P, P, 4, 768, 1024, 1, 5, 128, 1, 0.7, 0.3, None) == U  # J > 4
+    lb = lib.lffn_ln_project_hash_bwd_f32
+    assert lb(P, None, P, 1e-5, P, P, P, P, P, P, 4, 768, 1024, 1, 4, 128, 1, 0.7, 0.3, None) == A    # no LayerNorm weight
+    assert lb(P, P, P + 4, 1e-5, P, P, P, P, P, P, 4, 768, 1024, 1, 4, 128, 1, 0.7, 0.3, None) == A   # misaligned bias
+    assert lb(P, P, P, 1e-5, P, P, P, P, P, P, 4, 768, 1024, 1, 5, 128, 1, 0.7, 0.3, None) == U       # J > 4
     assert lib.lffn_lookup_scatter_sorted_f32(P, P, P, P, P, 1 << 30, 16, 4, 1024, 64, 0, None) == U    # S > 512
     assert lib.lffn_lookup_scatter_sorted_f32(P, P, P, P, P, 1 << 30, 16, 4, 16, 48, 0, None) == U      # Do % 32
     assert lib.lffn_lookup_scatter_sorted_f32(P, P, P, P, P, 64, 16, 4, 16, 64, 0, None) == A           # workspace too small

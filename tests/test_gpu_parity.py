@@ -519,6 +519,27 @@ def test_sum_partials_in_chunks_and_column_sums(P, n, chunks):
     assert np.abs(s - a.astype(np.float64).sum(0)).max() <= 1e-6 * np.abs(a).sum(0).max()
 
 
+@pytest.mark.parametrize("B,H,D,R,T", [(300, 768, 1024, 1, 128), (70, 256, 256, 2, 64), (33, 500, 512, 1, 40)])
+def test_ln_project_hash_bwd_matches_the_backward_on_the_normalised_input(B, H, D, R, T):
+    """LayerNorm formed on load inside the projection's backward: the same gradients as the plain
+    backward kernel fed with the LayerNorm output (and the z of the forward with LayerNorm inside)."""
+    rng = np.random.RandomState(B + H + T)
+    J = 4
+    x = (rng.randn(B, H) * 1.5 + 0.3).astype(np.float32)
+    ln_w = (1 + 0.1 * rng.randn(H)).astype(np.float32)
+    ln_b = (0.1 * rng.randn(H)).astype(np.float32)
+    diag = (rng.randn(R, J, D) / math.sqrt(D)).astype(np.float32)
+    bias = (0.05 * rng.randn(T * 8)).astype(np.float32)
+    g_score = rng.randn(B, T).astype(np.float32)
+    _, _, z = cabi.ln_project_hash(x, ln_w, ln_b, 1e-5, diag, bias, T)
+    h = oracle.layernorm(x.astype(np.float64), ln_w, ln_b, 1e-5).astype(np.float32)
+    want = cabi.project_hash_bwd(h, diag, z, g_score)
+    got = cabi.project_hash_bwd(x, diag, z, g_score, ln_w, ln_b, 1e-5)
+    for g, w in zip(got, want):
+        assert g.shape == w.shape and not np.isnan(g).any()
+        assert np.abs(g - w).max() <= 2e-5 * np.abs(w).max()
+
+
 def test_project_hash_near_zero_flip_count():
     # end to end against the float64 truth: flips may only happen where |z| is tiny
     rng = np.random.RandomState(9)
