@@ -66,7 +66,7 @@ WORKLOADS = {
 # (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); the summaries
 # are kept under profiles/.  None until measured for that workload.
 LDS_READ_PEAK_GBS = 76700.0     # microbenchmark: 125 bytes per clock per CU, 256 CUs
-MEASURED_TRAFFIC_BYTES = {"cfg2": 473980523, "cfg2b64": 474192048, "cfg3": 3170854613, "cfg3bf16": 2395468175,
+MEASURED_TRAFFIC_BYTES = {"cfg2": 499230616, "cfg2b64": 474192048, "cfg3": 3179615493, "cfg3bf16": 2393925657,
                           "cfg5": 944205370}
 
 
