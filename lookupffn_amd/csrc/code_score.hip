@@ -125,7 +125,7 @@ __global__ __launch_bounds__(256) void code_score_bwd_kernel(const float *__rest
 #pragma unroll
         for (int d = 0; d < K; ++d) {
             const float sg = v[d] > 0.f ? gp : (v[d] < 0.f ? -gp : 0.f);
-            o[d] = sg * (1.0f + S * 2.0f * e[d] / (1.0f + e[d]));
+            o[d] = sg * (1.0f + S * 2.0f * (e[d] * __builtin_amdgcn_rcpf(1.0f + e[d])));   // hardware reciprocal, 1 ulp
         }
 #pragma unroll
         for (int q = 0; q < K / 4; ++q)

@@ -586,10 +586,14 @@ __global__ __launch_bounds__(256) void project_hash_bwd_kernel(ProjectBwdArgs a)
             const float s_back = lane_xor<1>(s_run), p_back = lane_xor<1>(p_run);
             const float S = (lr & 1) ? s_run : s_back;
             const float P = (lr & 1) ? p_run : p_back;
+            // one division per group of four (P is the lane pair's), hardware reciprocals (1 ulp) for
+            // the per-value quotients: a gradient, compared at 1e-5
+            const float g_over_p = g / P;
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const float sg = zz[c] > 0.f ? 1.f : (zz[c] < 0.f ? -1.f : 0.f);
-                gz[j][c] = in_cols ? g * sg * (1.0f + S * 2.0f * ez[c] / (1.0f + ez[c])) / P : 0.f;
+                const float q = ez[c] * __builtin_amdgcn_rcpf(1.0f + ez[c]);
+                gz[j][c] = in_cols ? sg * (1.0f + S * 2.0f * q) * g_over_p : 0.f;
                 acc_b[j][c] += gz[j][c];
             }
         }
