@@ -533,7 +533,7 @@ __global__ __launch_bounds__(256 * HV / NH, HV == 1 ? 2 : 1) void bh4_block_kern
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
                             az[i] = fabsf(z[i]);
-                            fz[i] = 1.0f + expf(-2.0f * az[i]);
+                            fz[i] = 1.0f + exp_minus_2a(az[i]);
                         }
                         float s_loc = 0.f, p_loc = 1.f;
 #pragma unroll

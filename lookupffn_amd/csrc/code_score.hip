@@ -29,7 +29,7 @@ __global__ __launch_bounds__(256) void code_score_kernel(const float *__restrict
                 const float a = fabsf(v[c]);
                 code = (code << 1) | (v[c] > 0.f ? 1 : 0);
                 num = num + a;
-                den = den * (1.0f + expf(-2.0f * a));
+                den = den * (1.0f + exp_minus_2a(a));
             }
         }
     } else {
@@ -39,7 +39,7 @@ __global__ __launch_bounds__(256) void code_score_kernel(const float *__restrict
             const float a = fabsf(v);
             code = (code << 1) | (v > 0.f ? 1 : 0);
             num = num + a;
-            den = den * (1.0f + expf(-2.0f * a));
+            den = den * (1.0f + exp_minus_2a(a));
         }
     }
     codes[n] = code;
@@ -70,7 +70,7 @@ __global__ __launch_bounds__(256) void mix_code_score_kernel(const float *__rest
         const float a = fabsf(v);
         code = (code << 1) | (v > 0.f ? 1 : 0);
         num = num + a;
-        den = den * (1.0f + expf(-2.0f * a));
+        den = den * (1.0f + exp_minus_2a(a));
     };
     if constexpr (K > 0) {
         const int col0 = t * K;

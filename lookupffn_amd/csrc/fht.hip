@@ -373,7 +373,7 @@ __global__ __launch_bounds__(256) void project_kernel(ProjectArgs a) {
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                     az[c] = fabsf(z[c]);
-                    fz[c] = 1.0f + expf(-2.0f * az[c]);
+                    fz[c] = 1.0f + exp_minus_2a(az[c]);
                 }
                 float s_loc = 0.f, p_loc = 1.f;
                 score_chain(az, fz, s_loc, p_loc);                 // what an even lane hands over
