@@ -312,6 +312,13 @@ class LookupFFN(nn.Module):
         self.tables = nn.Parameter(0.02 * torch.randn(self.num_table, self.table_size, self.output_size))
         self.bias = nn.Parameter(0.001 * torch.randn(self.output_size))
 
+    def __getstate__(self):
+        # the cached parameter views are derived data: not pickled with the module
+        state = super().__getstate__() if hasattr(super(), "__getstate__") else self.__dict__.copy()
+        state = dict(state)
+        state.pop("_inference_cache", None)
+        return state
+
     def extra_repr(self):
         return (f"hidden_size={self.hidden_size}, num_table={self.num_table}, "
                 f"table_size={self.table_size}, output_size={self.output_size}")
