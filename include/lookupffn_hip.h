@@ -39,7 +39,7 @@ extern "C" {
 #define LFFN_ERR_UNSUPPORTED -2   /* a shape outside what the kernels are built for */
 #define LFFN_ERR_LAUNCH      -3   /* hipGetLastError() after the launch was not hipSuccess */
 
-#define LFFN_ABI_VERSION 2
+#define LFFN_ABI_VERSION 3
 
 /* ABI version of the loaded library (LFFN_ABI_VERSION at build time). */
 int lffn_version(void);

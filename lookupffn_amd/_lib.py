@@ -15,7 +15,7 @@ _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 # LOOKUPFFN_HIP_LIB points at another build of the same ABI (e.g. a tuning build)
 LIB_PATH = os.environ.get("LOOKUPFFN_HIP_LIB") or os.path.join(_PKG_DIR, "liblookupffn_hip.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 LFFN_OK = 0
 LFFN_ERR_BAD_ARG = -1
@@ -107,13 +107,13 @@ def load() -> ctypes.CDLL:
         lib.lffn_version.argtypes = []
         lib.lffn_error_string.restype = ctypes.c_char_p
         lib.lffn_error_string.argtypes = [ctypes.c_int]
+        if lib.lffn_version() != ABI_VERSION:          # first: an older library lacks some of the entry points below
+            raise LookupFFNLibraryError(
+                f"{LIB_PATH} has ABI version {lib.lffn_version()}, this package needs {ABI_VERSION}: rebuild it")
         for name, argtypes in SIGNATURES.items():
             fn = getattr(lib, name)
             fn.restype = ctypes.c_int
             fn.argtypes = argtypes
-        if lib.lffn_version() != ABI_VERSION:
-            raise LookupFFNLibraryError(
-                f"{LIB_PATH} has ABI version {lib.lffn_version()}, this package needs {ABI_VERSION}: rebuild it")
         _lib = lib
         return _lib
 
