@@ -341,6 +341,33 @@ def test_checkpoint_round_trip_and_folded_weight_cache(tmp_path):
         assert not torch.equal(b(x), out_a)
 
 
+@pytest.mark.parametrize("bs", [1, 64])
+def test_training_step_of_a_large_batch_is_the_sum_of_its_halves(bs):
+    """A size-independent property at the full width of the layer (768 -> 128 tables x 256 x 768) and
+    32768 tokens, where the backward takes the sorted scatter, the chunked column sums and the
+    kernels' partial sums: every parameter gradient of the batch equals the sum of the gradients of
+    its two halves, and the input gradient is their concatenation."""
+    torch.manual_seed(2)
+    layer = lookupffn_amd.LookupFFN(_config(hidden_size=768, ffn_num_table=128, block_size=bs), 768).to(DEV).train()
+    B = 32768
+    x = torch.randn(B, 768, device=DEV)
+    g = torch.randn(B, 768, device=DEV)
+
+    def grads(xs, gs):
+        for q in layer.parameters():
+            q.grad = None
+        xs = xs.clone().requires_grad_(True)
+        layer(xs).backward(gs)
+        return [xs.grad.clone()] + [q.grad.clone() for q in layer.parameters()]
+
+    full = grads(x, g)
+    first, second = grads(x[:B // 2], g[:B // 2]), grads(x[B // 2:], g[B // 2:])
+    names = ["x"] + [n for n, _ in layer.named_parameters()]
+    for n, f, a, b in zip(names, full, first, second):
+        want = torch.cat([a, b]) if n == "x" else a + b
+        assert ((f - want).abs().max() / want.abs().max()).item() <= 1e-5, n
+
+
 def test_one_launch_layer_follows_its_parameters():
     """Small batches take the one-launch form, which keeps views of the parameters between calls:
     they must follow in-place updates, a loaded state dict, a replaced parameter and a cast, and
