@@ -354,10 +354,13 @@ GatherPlan plan_gather(int64_t B, int64_t T, int64_t S, int64_t Do) {
     // token-major: every token reads its T rows from L2 / Infinity Cache, measured 9 TB/s
     GatherPlan best{0, 0, double(B) * double(T) * double(Do) * (BF16 ? 2 : 4) / 9e6 + 5.0};
     if (S > MAX_S || T < 4 || B * T >= (int64_t(1) << 31)) return best;
-    struct Option { int kind, np; double us_per_table; };
-    static const Option f32_opts[] = {{1, 4, 1.15}, {1, 8, 1.18}, {1, 13, 1.30}, {1, 16, 1.60},
-                                      {2, 4, 0.88}, {2, 8, 1.01}, {2, 13, 1.47}, {2, 16, 1.79}};
-    static const Option bf16_opts[] = {{1, 4, 1.21}, {1, 8, 1.32}, {2, 4, 0.97}, {2, 8, 1.20}};
+    // us_per_table: tables that fit the cache (measured at 128 x 256 x 768 fp32, 16384 tokens); us_big:
+    // table sets beyond it (512 x 256 x 1024 fp32 = 537 MB; the bf16 figures are the cached ones times
+    // 1.3 / 1.15).  Both with the team touch in the kernels.
+    struct Option { int kind, np; double us_per_table, us_big; };
+    static const Option f32_opts[] = {{1, 4, 1.16, 1.45}, {1, 8, 1.05, 1.13}, {1, 13, 1.29, 1.48}, {1, 16, 1.50, 1.56},
+                                      {2, 4, 0.74, 1.00}, {2, 8, 0.98, 1.31}, {2, 13, 1.41, 1.31}, {2, 16, 1.77, 1.77}};
+    static const Option bf16_opts[] = {{1, 4, 1.21, 1.57}, {1, 8, 1.32, 1.72}, {2, 4, 0.97, 1.12}, {2, 8, 1.20, 1.38}};
     const Option *opts = BF16 ? bf16_opts : f32_opts;
     const int nopts = BF16 ? 4 : 8;
     const bool big = double(T) * double(S) * double(Do) * (BF16 ? 2 : 4) > 200e6;
@@ -373,7 +376,7 @@ GatherPlan plan_gather(int64_t B, int64_t T, int64_t S, int64_t Do) {
         if (B * nslices > (int64_t(1) << 30)) continue;
         const int64_t tiles = (B + tok - 1) / tok;
         const int64_t rounds = (tiles * nslices + 255) / 256;
-        const double us = double(rounds) * double(T) * o.us_per_table * (big ? (o.kind == 1 ? 1.3 : 1.15) : 1.0);
+        const double us = double(rounds) * double(T) * (big ? o.us_big : o.us_per_table);
         if (us < best_us) { best_us = us; best = GatherPlan{o.kind, o.np, us}; }
     }
     return best;
@@ -437,6 +440,38 @@ __global__ __launch_bounds__(256) void gather_parts_reduce_kernel(const float *p
 }
 
 // Is (kind, np) a kernel that is built, and does the shape meet its preconditions?
+// Many tokens and tables that fit the 256 MB Infinity Cache are taken in pieces: in one launch over
+// all tokens the outputs, codes and scores streaming through push the tables out of the caches and
+// every round of workgroups fetches its slices from further away (131072 tokens at 128 x 256 x 768
+// fp32: 1745 us in one launch, 1357 in pieces).  A piece is what one round of 256 workgroups takes at
+// the tile size that is cheapest for the whole batch: 21 tiles of 832 tokens at 768 columns, 32
+// tiles of 1024 tokens at 512 columns (32768 tokens: 295 -> 211 us against pieces of 16384).
+// Returns the tokens per piece (a multiple of 64), or B when the batch goes in one launch.
+template <bool BF16>
+int64_t gather_pieces(int64_t B, int64_t T, int64_t S, int64_t Do) {
+    if (B < 2 * 16384 || double(T) * double(S) * double(Do) * (BF16 ? 2 : 4) > double(int64_t(192) << 20)) return B;
+    const GatherPlan whole = plan_gather<BF16>(B, T, S, Do);
+    if (whole.kind == 0) return B;
+    double best_us = 1e300;
+    int64_t best_each = B;
+    for (int kind = 1; kind <= 2; ++kind) {
+        const int cols = (kind == 1 ? 256 : 128) / (BF16 ? 2 : 4);
+        if (Do % cols != 0) continue;
+        const int64_t nslices = Do / cols;
+        if (nslices > 256) continue;
+        for (int np : {4, 8, 13, 16}) {
+            if (BF16 && np > 8) continue;
+            const int64_t piece = (256 / nslices) * int64_t(kind == 1 ? 64 : 128) * np;     // one round
+            const int64_t n = (B + piece - 1) / piece;
+            const int64_t each = ((B + n - 1) / n + 63) & ~int64_t(63);
+            const GatherPlan p = plan_gather<BF16>(each, T, S, Do);                        // what a piece will run as
+            const double us = double(n) * (p.us + 4.0);                                    // + a launch
+            if (us < best_us) { best_us = us; best_each = each; }
+        }
+    }
+    return best_each < B ? best_each : B;
+}
+
 template <bool BF16>
 bool plan_is_valid(const GatherPlan &p, int64_t B, int64_t T, int64_t S, int64_t Do) {
     if (p.kind == 0) return true;
@@ -461,14 +496,10 @@ int lookup_gather_entry(const int32_t *code, const float *score, const void *tab
     LFFN_REQUIRE(lffn_aligned16(tables) && lffn_aligned16(out) && (!bias || lffn_aligned16(bias)) &&
                      (!residual || lffn_aligned16(residual)), LFFN_ERR_BAD_ARG);
     if (B == 0) return LFFN_OK;
-    // Many tokens, tables that fit the 256 MB Infinity Cache: take the tokens in pieces of about
-    // 16384, one launch after the other.  In one launch over all tokens the outputs, codes and
-    // scores streaming through push the tables out of that cache and every workgroup fetches its
-    // slices from HBM again (65536 tokens at 128 x 256 x 768: 867 us in one launch, 4 x 176 apart).
-    constexpr int64_t PIECE = 16384;
-    if (kind_req < 0 && B >= 2 * PIECE && T * S * Do * (BF16 ? 2 : 4) <= (int64_t(192) << 20)) {
-        const int64_t n = (B + PIECE / 2) / PIECE;
-        const int64_t each = ((B + n - 1) / n + 63) & ~int64_t(63);
+    // Many tokens, tables that fit the 256 MB Infinity Cache: take the tokens in pieces, one launch
+    // after the other (gather_pieces).
+    const int64_t each = kind_req < 0 ? gather_pieces<BF16>(B, T, S, Do) : B;
+    if (each < B) {
         for (int64_t b0 = 0; b0 < B; b0 += each) {
             const int rc = lookup_gather_entry<BF16>(code + b0 * T, score + b0 * T, tables, bias,
                                                      residual ? residual + b0 * Do : nullptr, out + b0 * Do,
@@ -568,7 +599,8 @@ extern "C" int lffn_lookup_gather_workspace_bytes(int64_t B, int64_t T, int64_t 
     LFFN_REQUIRE(bytes, LFFN_ERR_BAD_ARG);
     *bytes = 0;
     if (B < 1 || T < 1 || Do < 1 || !lffn_is_pow2(S) || Do % 64 != 0 || B * T >= (int64_t(1) << 31)) return LFFN_OK;
-    if (B >= 2 * 16384) return LFFN_OK;                        // taken in pieces, none of which is split
+    if ((bf16 ? gather_pieces<true>(B, T, S, Do) : gather_pieces<false>(B, T, S, Do)) < B)
+        return LFFN_OK;                                        // taken in pieces, none of which is split
     const GatherPlan plan = bf16 ? plan_gather<true>(B, T, S, Do) : plan_gather<false>(B, T, S, Do);
     const SplitPlan sp = bf16 ? plan_split<true>(B, T, S, Do) : plan_split<false>(B, T, S, Do);
     if (sp.nparts > 1 && sp.us < 0.85 * plan.us) *bytes = int64_t(sp.nparts) * B * Do * 4;
