@@ -355,12 +355,11 @@ GatherPlan plan_gather(int64_t B, int64_t T, int64_t S, int64_t Do) {
     GatherPlan best{0, 0, double(B) * double(T) * double(Do) * (BF16 ? 2 : 4) / 9e6 + 5.0};
     if (S > MAX_S || T < 4 || B * T >= (int64_t(1) << 31)) return best;
     // us_per_table: tables that fit the cache (measured at 128 x 256 x 768 fp32, 16384 tokens); us_big:
-    // table sets beyond it (512 x 256 x 1024 fp32 = 537 MB; the bf16 figures are the cached ones times
-    // 1.3 / 1.15).  Both with the team touch in the kernels.
+    // table sets beyond it (512 x 256 x 1024: 537 MB fp32, 268 MB bf16).  All with the team touch in the kernels.
     struct Option { int kind, np; double us_per_table, us_big; };
     static const Option f32_opts[] = {{1, 4, 1.16, 1.45}, {1, 8, 1.05, 1.13}, {1, 13, 1.29, 1.48}, {1, 16, 1.50, 1.56},
                                       {2, 4, 0.74, 1.00}, {2, 8, 0.98, 1.31}, {2, 13, 1.41, 1.31}, {2, 16, 1.77, 1.77}};
-    static const Option bf16_opts[] = {{1, 4, 1.21, 1.57}, {1, 8, 1.32, 1.72}, {2, 4, 0.97, 1.12}, {2, 8, 1.20, 1.38}};
+    static const Option bf16_opts[] = {{1, 4, 1.10, 1.51}, {1, 8, 1.24, 1.34}, {2, 4, 0.87, 0.88}, {2, 8, 1.44, 1.37}};
     const Option *opts = BF16 ? bf16_opts : f32_opts;
     const int nopts = BF16 ? 4 : 8;
     const bool big = double(T) * double(S) * double(Do) * (BF16 ? 2 : 4) > 200e6;
@@ -398,8 +397,8 @@ SplitPlan plan_split(int64_t B, int64_t T, int64_t S, int64_t Do) {
     const int cols = BF16 ? 128 : 64;
     if (S > MAX_S || T < 32 || Do % cols != 0 || B < 256 || B * T >= (int64_t(1) << 31)) return best;
     struct Option { int np; double us_per_table; };
-    static const Option f32_opts[] = {{4, 1.15}, {8, 1.18}, {13, 1.30}};
-    static const Option bf16_opts[] = {{4, 1.21}, {8, 1.32}};
+    static const Option f32_opts[] = {{4, 1.16}, {8, 1.05}, {13, 1.29}};
+    static const Option bf16_opts[] = {{4, 1.10}, {8, 1.24}};
     const Option *opts = BF16 ? bf16_opts : f32_opts;
     const int nopts = BF16 ? 2 : 3;
     const int64_t nslices = Do / cols;
@@ -469,7 +468,11 @@ int64_t gather_pieces(int64_t B, int64_t T, int64_t S, int64_t Do) {
             if (us < best_us) { best_us = us; best_each = each; }
         }
     }
-    return best_each < B ? best_each : B;
+    // two rounds still go faster in one launch (32768 tokens, bf16 rows of 1024: 339 us against 382 in two
+    // pieces; fp32 rows of 768: 345 either way); from three rounds on the pieces win (65536 tokens: 693
+    // against 735, 131072: 1357 against 1745)
+    if ((B + best_each - 1) / best_each <= 2) return B;
+    return best_each;
 }
 
 template <bool BF16>

@@ -796,7 +796,7 @@ def test_lookup_gather_plan_and_planned_entry():
     # what the heuristic picks at the BASELINE.json shapes
     assert cabi.lookup_gather_plan(16384, 128, 256, 768) == (1, 832)            # config 2
     assert cabi.lookup_gather_plan(16384, 512, 256, 1024) == (1, 1024)          # config 3 fp32
-    assert cabi.lookup_gather_plan(16384, 512, 256, 1024, bf16=True) == (2, 1024)
+    assert cabi.lookup_gather_plan(16384, 512, 256, 1024, bf16=True) == (1, 512)
     assert cabi.lookup_gather_plan(256, 32, 256, 256) == (0, 0)                 # config 1: token-major
     assert cabi.lookup_gather_plan(16384, 128, 512, 768) == (0, 0)              # S > 256
     # every plan the heuristic can return is one of the built kernels
