@@ -66,7 +66,7 @@ WORKLOADS = {
 # (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); the summaries
 # are kept under profiles/.  None until measured for that workload.
 LDS_READ_PEAK_GBS = 76700.0     # microbenchmark: 125 bytes per clock per CU, 256 CUs
-MEASURED_TRAFFIC_BYTES = {"cfg2": 499747232, "cfg2b64": 499427315, "cfg3": 2840080784, "cfg3bf16": 2391081909,
+MEASURED_TRAFFIC_BYTES = {"cfg2": 499747232, "cfg2b64": 499427315, "cfg3": 2840080784, "cfg3bf16": 1382263937,
                           "cfg5": 943507857}
 
 
