@@ -178,6 +178,19 @@ def test_workspace_queries_are_host_side_plans():
     for shape in ((16384, 128, 256, 768), (65536, 128, 256, 768), (256, 32, 256, 256), (4096, 16, 256, 768),
                   (2048, 128, 512, 768), (2048, 128, 256, 100), (0, 128, 256, 768)):
         assert gather_ws(*shape) == 0, shape
+    # which gather kernel a shape gets is a host-side decision as well: (tables per LDS buffer, tokens per workgroup)
+    def plan(B, T, S, Do, bf16=0):
+        kind = ctypes.c_int32(-1)
+        tokens = lib.lffn_lookup_gather_plan(B, T, S, Do, bf16, ctypes.byref(kind))
+        return kind.value, tokens
+
+    assert plan(16384, 128, 256, 768) == (1, 832)               # RoBERTa-base: 240 workgroups in one round
+    assert plan(16384, 512, 256, 1024) == (1, 1024)             # 537 MB of tables: 256 workgroups in one round
+    assert plan(16384, 512, 256, 1024, 1) == (1, 512)           # the same in bf16 rows
+    assert plan(32768, 128, 256, 512) == (1, 1024)              # the reference's compare.py shape
+    assert plan(8192, 128, 256, 768) == (2, 1024)               # fewer tokens: two tables per buffer
+    assert plan(256, 32, 256, 256) == (0, 0)                    # too few tokens to stage tables: token-major
+    assert plan(16384, 128, 512, 768) == (0, 0)                 # tables too long for the LDS buffers
     # sorted scatter: pairs + offsets + transposed codes and scores + packed gradient, for at most 16384 tokens
     one = scatter_ws(16384, 128, 256, 768)
     assert one >= 16384 * 128 * 8 + 16384 * 768 * 4
