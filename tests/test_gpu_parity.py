@@ -817,6 +817,47 @@ def test_lookup_gather_plan_and_planned_entry():
     assert lib.lffn_lookup_gather_planned_f32(*big_s, 1, 512, None) == _lib.LFFN_ERR_UNSUPPORTED     # S > 256
 
 
+def test_every_gather_form_and_the_inner_product_on_random_shapes():
+    """Seeded sweep: every built table-major form (one or two tables per LDS buffer, every tile size,
+    fp32 and bf16 rows) forced onto shapes it would not be chosen for (odd table counts, batches that
+    end inside a tile or a wavefront, short tables, few tables), plus what the plan picks and the
+    inner product, all against the float64 sum."""
+    rng = np.random.RandomState(2024)
+
+    def bf16_bits(a):
+        u = a.astype(np.float32).view(np.uint32)
+        return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+    for it in range(24):
+        bf = it % 3 == 2
+        S = int(rng.choice([256, 256, 256, 128, 64, 16]))
+        T = int(rng.randint(4, 36))
+        Do = int(rng.choice([128, 256, 384, 768])) if bf else int(rng.choice([64, 128, 192, 256, 768]))
+        B = int(rng.choice([1, 7, 63, 65, 257, 833, 1000]))
+        tables = (0.1 * rng.randn(T, S, Do)).astype(np.float32)
+        code = rng.randint(0, S, size=(B, T)).astype(np.int32)
+        score = rng.rand(B, T).astype(np.float32)
+        bias = (0.01 * rng.randn(Do)).astype(np.float32)
+        tb = bf16_bits(tables) if bf else tables
+        tv = (tb.astype(np.uint32) << 16).view(np.float32) if bf else tables
+        rows = tv[np.arange(T)[None, :], code].astype(np.float64)                  # [B, T, Do]
+        want = bias.astype(np.float64) + np.einsum("bt,btd->bd", score.astype(np.float64), rows)
+        scale = np.abs(want).max()
+        plans = [None]
+        for kind in (1, 2):
+            cols = (256 if kind == 1 else 128) // (2 if bf else 4)
+            if Do % cols == 0:
+                plans += [(kind, (64 if kind == 1 else 128) * np_) for np_ in ((4, 8) if bf else (4, 8, 13, 16))]
+        for plan in plans:
+            got = cabi.lookup_gather(code, score, tb, bias, bf16=bf, plan=plan)
+            assert np.abs(got - want).max() <= 1e-5 * scale, (it, bf, B, T, S, Do, plan)
+        if not bf:
+            g = rng.randn(B, Do).astype(np.float32)
+            want_i = np.einsum("bd,btd->bt", g.astype(np.float64), rows)
+            got_i = cabi.lookup_inner(code, g, tables)
+            assert np.abs(got_i - want_i).max() <= 1e-5 * np.abs(want_i).max(), (it, B, T, S, Do)
+
+
 def test_gather_special_cases():
     rng = np.random.RandomState(30)
     tables, code, idx, w = _rand_gather(rng, 16, 8, 16, 128)
