@@ -51,6 +51,12 @@ def compute_code_score(hash_scores, training):
     """PL/compute_code_score/kernel.py:22-30: (code int32 [..., T], score float [..., T])."""
     if not hash_scores.is_cuda:
         raise RuntimeError("compute_code_score: lookupffn_amd runs on the GPU only (got a CPU tensor)")
+    if hash_scores.dtype in (torch.float16, torch.bfloat16):
+        # under autocast a dense projection hands over 16-bit z (the reference's torch formula takes
+        # any float dtype, PL/compute_code_score/kernel.py:43-55): widened here, exactly, so the code is
+        # that of the 16-bit values; the score comes back in float32 and autograd casts the gradient
+        # of z back to the 16-bit type
+        hash_scores = hash_scores.float()
     if hash_scores.dtype != torch.float32:
-        raise NotImplementedError(f"compute_code_score: dtype {hash_scores.dtype} (float32 is built)")
+        raise NotImplementedError(f"compute_code_score: dtype {hash_scores.dtype} (float32, float16 and bfloat16 are taken)")
     return ComputeCodeScore.apply(hash_scores)

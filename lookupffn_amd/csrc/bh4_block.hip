@@ -580,11 +580,8 @@ int launch_block(const BlockArgs &a, hipStream_t st) {
     constexpr int TOK = 16 * HV;
     const size_t lds_bytes = (size_t(TOK) * (BS * NB + PAD) + 2 * TOK + (HASH ? 2 * BS * NB : 0)) * sizeof(float);
     auto kern = bh4_block_kernel<NB, HASH, NH, BWD, HV>;
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)lds_bytes) != hipSuccess) {
-        (void)hipGetLastError();
-        return LFFN_ERR_LAUNCH;
-    }
+    static LdsGrant granted;      // one record per kernel instantiation
+    if (!lffn_grant_dynamic_lds(reinterpret_cast<const void *>(kern), lds_bytes, granted)) return LFFN_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)((a.B + TOK - 1) / TOK)), dim3(256 * HV / NH), lds_bytes, st, a);
     return lffn_launch_status();
 }

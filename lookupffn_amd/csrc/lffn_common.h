@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <type_traits>
 
 #include "../../include/lookupffn_hip.h"
@@ -46,6 +47,36 @@ __attribute__((visibility("hidden")))
 int lffn_internal_lookup_gather_pair(const int32_t *code, const float *score, const void *tables,
                                      const float *bias, const float *residual, float *out, int64_t B, int64_t T,
                                      int64_t S, int64_t Do, bool bf16, int np, void *stream);
+
+// Dynamic LDS beyond the default limit has to be granted to a kernel once per device
+// (hipFuncAttributeMaxDynamicSharedMemorySize).  `granted` is the caller's record for ONE kernel
+// instantiation (a function-local static array, zero-initialised): the largest size granted so far
+// on each device, so that the attribute call is made when a launch needs more than that and not on
+// every launch.  Devices beyond the record ask every time.
+constexpr int LFFN_MAX_DEVICES = 16;
+struct LdsGrant {
+    std::atomic<int> bytes[LFFN_MAX_DEVICES];
+};
+static inline bool lffn_grant_dynamic_lds(const void *kernel, size_t lds_bytes, LdsGrant &granted) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    const bool recorded = dev >= 0 && dev < LFFN_MAX_DEVICES;
+    if (recorded && granted.bytes[dev].load(std::memory_order_acquire) >= (int)lds_bytes) return true;
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    if (recorded) {
+        int seen = granted.bytes[dev].load(std::memory_order_relaxed);
+        while (seen < (int)lds_bytes &&
+               !granted.bytes[dev].compare_exchange_weak(seen, (int)lds_bytes, std::memory_order_release)) {
+        }
+    }
+    return true;
+}
 
 static inline int lffn_launch_status() {
     return hipGetLastError() == hipSuccess ? LFFN_OK : LFFN_ERR_LAUNCH;
@@ -157,7 +188,7 @@ __device__ __forceinline__ void l2_touch(const char *base, uint32_t lane_offset,
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
                  :
                  : "v"(lane_offset), "s"(base), "s"(lds_byte_addr)
-                 : "memory");
+                 : "memory", "m0");
 }
 
 // The line of a region of `nlines` 128-byte lines that lane `tid` of workgroup `member` of a team of

@@ -70,7 +70,7 @@ __device__ __forceinline__ void lds_dma16(const char *table, uint32_t lane_offse
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
                  : "v"(lane_offset), "s"(table), "s"(lds_byte_addr)
-                 : "memory");
+                 : "memory", "m0");
 }
 
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
@@ -320,11 +320,8 @@ int launch_lds_full(LdsGatherArgs a, hipStream_t stream) {
     a.per_xcd = (units + XCDS - 1) / XCDS;
     const size_t lds_bytes = size_t(2) * a.S * SEG_VECS * 16 + TOUCH_SINK_BYTES;      // two buffers + the touches' scratch
     auto kern = lookup_gather_lds_kernel<BF16, NP, FULL>;
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)lds_bytes) != hipSuccess) {
-        (void)hipGetLastError();
-        return LFFN_ERR_LAUNCH;
-    }
+    static LdsGrant granted;      // one record per kernel instantiation
+    if (!lffn_grant_dynamic_lds(reinterpret_cast<const void *>(kern), lds_bytes, granted)) return LFFN_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3(a.per_xcd * XCDS), dim3(WG), lds_bytes, stream, a);
     return lffn_launch_status();
 }

@@ -55,7 +55,7 @@ __device__ __forceinline__ void lds_dma16(const char *gptr, uint32_t lds_byte_ad
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                  :
                  : "v"(gptr), "s"(lds_byte_addr)
-                 : "memory");
+                 : "memory", "m0");
 }
 
 template <bool FULL>
@@ -227,11 +227,8 @@ int launch_inner_full(InnerArgs a, hipStream_t stream) {
     a.per_xcd = (units + XCDS - 1) / XCDS;
     const size_t lds_bytes = size_t(2) * a.S * SEG_VECS * 16 + TOUCH_SINK_BYTES;     // two buffers + the touches' scratch
     auto kern = lookup_inner_lds_kernel<NP, FULL>;
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)lds_bytes) != hipSuccess) {
-        (void)hipGetLastError();
-        return LFFN_ERR_LAUNCH;
-    }
+    static LdsGrant granted;      // one record per kernel instantiation
+    if (!lffn_grant_dynamic_lds(reinterpret_cast<const void *>(kern), lds_bytes, granted)) return LFFN_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3(a.per_xcd * XCDS), dim3(WG), lds_bytes, stream, a);
     return lffn_launch_status();
 }

@@ -173,11 +173,8 @@ extern "C" int lffn_lookup_scatter_f32(const int32_t *code, const float *score, 
     a.per_xcd = (int)((units + XCDS - 1) / XCDS);
     a.accumulate = accumulate;
     const size_t lds_bytes = size_t(S) * COLS * 8 + size_t(WAVES) * 64 * 8;
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(lookup_scatter_lds_kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess) {
-        (void)hipGetLastError();
-        return LFFN_ERR_LAUNCH;
-    }
+    static LdsGrant granted;      // one record per kernel instantiation
+    if (!lffn_grant_dynamic_lds(reinterpret_cast<const void *>(lookup_scatter_lds_kernel), lds_bytes, granted)) return LFFN_ERR_LAUNCH;
     hipLaunchKernelGGL(lookup_scatter_lds_kernel, dim3(a.per_xcd * XCDS), dim3(WG), lds_bytes, st, a);
     return lffn_launch_status();
 }

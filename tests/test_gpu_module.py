@@ -445,3 +445,139 @@ def test_layer_forward_under_graph_capture(tokens, tables, width):
             want = layer(x)                                # eager work between the replays
             torch.cuda.synchronize()
             assert torch.equal(got, want), i
+
+
+# ----------------------------------------------------------------------------- dense projection, autocast
+
+def _dense_reference_grads(layer, x, target, z_dtype=torch.float64):
+    """Autograd over the reference's formulas (PL/lookup.py:57-60,64-77,98-130 with
+    compute_code_score_torch and the index-multiply-sum gather) in float64 on the CPU."""
+    T, S, Do = layer.tables.shape
+    H = layer.hidden_size
+    ref = {k: v.detach().double().cpu().requires_grad_(True) for k, v in layer.named_parameters()}
+    xr = x.detach().double().cpu().requires_grad_(True)
+    h = torch.nn.functional.layer_norm(xr, (H,), ref["LayerNorm.weight"], ref["LayerNorm.bias"], 1e-5)
+    z = (h @ ref["hash.projection.weight"].T + ref["hash.projection.bias"]).reshape(-1, T, 8)
+    code, score = lookupffn_amd.compute_code_score_torch(z)
+    idx = code.long() + torch.arange(T)[None] * S
+    out = (ref["tables"].reshape(T * S, Do)[idx] * score[:, :, None]).sum(1) + ref["bias"]
+    ((out - target.double().cpu()) ** 2).sum().backward()
+    return out.detach(), code, ref, xr
+
+
+@pytest.mark.parametrize("H,T,Do", [(192, 32, 128), (512, 128, 512), (768, 128, 768)])
+def test_dense_projection_forward_matches_oracle(H, T, Do):
+    """projection_type="dense" (PL/lookup.py:57-60, cfgs/roberta/small-512/lookup-t128-s8-dense.py:25):
+    nn.Linear, then the code/score kernel and the gather kernel.  From the GPU's own z (rocBLAS rounds
+    the product differently from any CPU sum) everything after it is checked against the oracle; z
+    itself against the float64 product."""
+    torch.manual_seed(H + T + 1)
+    S = 256
+    layer = lookupffn_amd.LookupFFN(_config(hidden_size=H, ffn_num_table=T, projection_type="dense"), Do).eval().to(DEV)
+    assert isinstance(layer.hash.projection, torch.nn.Linear)
+    assert layer.hash.projection.weight.shape == (T * 8, H)
+    x = torch.randn(5, 41, H, device=DEV)
+    with torch.no_grad():
+        out = layer(x)
+        h = layer.LayerNorm(x.reshape(-1, H))
+        z = layer.hash.projection(h)
+        code, score = layer.hash(h)
+    p = layer.hash.projection
+    z64 = npf(h).astype(np.float64) @ npf(p.weight).astype(np.float64).T + npf(p.bias)
+    assert relmax(npf(z), z64) <= 1e-5
+    code_o, score_o = oracle.code_score(npf(z).reshape(-1, T, 8))
+    assert np.array_equal(npf(code).astype(np.int32), code_o)
+    np.testing.assert_allclose(npf(score), score_o, rtol=2e-6)
+    idx = code_o + (np.arange(T, dtype=np.int32) * S)[None]
+    want = oracle.gather_add(idx, npf(layer.tables).reshape(T * S, Do).astype(np.float64),
+                             score_o.astype(np.float64)) + npf(layer.bias)
+    assert relmax(npf(out).reshape(-1, Do), want) <= 1e-5
+    # against the float64 truth codes differ only where |z| is at rounding level
+    code64, _ = oracle.code_score(z64.reshape(-1, T, 8))
+    flips = (code64 != code_o)
+    if flips.any():
+        zmin = np.abs(z64.reshape(-1, T, 8)).min(-1)
+        assert zmin[flips].max() <= 1e-5 * np.abs(z64).max()
+
+
+@pytest.mark.parametrize("H,T,Do", [(192, 32, 64), (512, 128, 128)])
+def test_dense_projection_gradients_match_torch_autograd_of_reference_formulas(H, T, Do):
+    torch.manual_seed(9 + H + T)
+    layer = lookupffn_amd.LookupFFN(_config(hidden_size=H, ffn_num_table=T, projection_type="dense"), Do).to(DEV).train()
+    x = torch.randn(24, H, device=DEV, requires_grad=True)
+    target = torch.randn(24, Do, device=DEV)
+    out = layer(x)
+    ((out - target) ** 2).sum().backward()
+    out_r, code_r, ref, xr = _dense_reference_grads(layer, x, target)
+    with torch.no_grad():
+        code_g, _ = layer.hash(layer.LayerNorm(x))
+    if not np.array_equal(npf(code_g).astype(np.int64), code_r.numpy().astype(np.int64)):
+        pytest.skip("a sign flipped between fp32 and fp64 projections for this seed")
+    assert relmax(npf(out), out_r.numpy()) <= 2e-5
+    for k, v in layer.named_parameters():
+        assert v.grad is not None and relmax(npf(v.grad), ref[k].grad.numpy()) <= 2e-4, k
+    assert relmax(npf(x.grad), xr.grad.numpy()) <= 2e-4
+
+
+def test_compute_code_score_takes_16_bit_z():
+    """Under autocast nn.Linear returns float16: the code is that of the 16-bit values (widening is
+    exact), the score is float32, the gradient comes back in the dtype of z."""
+    torch.manual_seed(3)
+    for dt in (torch.float16, torch.bfloat16):
+        z = torch.randn(50, 12, 8, device=DEV).to(dt).requires_grad_(True)
+        code, score = lookupffn_amd.compute_code_score(z, training=True)
+        assert code.dtype == torch.int32 and score.dtype == torch.float32
+        code_o, score_o = oracle.code_score(npf(z))
+        assert np.array_equal(npf(code).astype(np.int32), code_o)
+        np.testing.assert_allclose(npf(score), score_o, rtol=2e-6)
+        gs = torch.randn(50, 12, device=DEV)
+        score.backward(gs)
+        assert z.grad.dtype == dt
+        want = oracle.code_score_bwd(npf(z).astype(np.float64), npf(gs).astype(np.float64))
+        assert relmax(npf(z.grad), want) <= (2e-3 if dt == torch.float16 else 1e-2)
+
+
+@pytest.mark.parametrize("projection,bs", [("bh4", 64), ("bh4", 1), ("dense", 1)])
+def test_layer_under_autocast_float16(projection, bs):
+    """The reference trains with precision=16 (cfgs/roberta/small-512/lookup-t128-s8-bh4.py:15-34:
+    hidden 512, 128 tables of 256, block size 64).  Forward + backward of the layer under
+    torch.autocast(float16) against the same step in float32: the custom operators keep float32
+    whatever autocast says, so the BH4 forms agree to rounding; with the dense projection z is a
+    float16 product, so codes may differ where |z| is below half precision and only tokens whose
+    codes all agree are compared."""
+    torch.manual_seed(21)
+    H, T, Do, B = 512, 128, 512, 96
+    layer = lookupffn_amd.LookupFFN(_config(hidden_size=H, ffn_num_table=T, projection_type=projection,
+                                            block_size=bs), Do).to(DEV).train()
+    x = torch.randn(B, H, device=DEV)
+    target = torch.randn(B, Do, device=DEV)
+
+    def step(autocast):
+        layer.zero_grad(set_to_none=True)
+        xi = x.clone().requires_grad_(True)
+        with torch.autocast("cuda", dtype=torch.float16, enabled=autocast):
+            out = layer(xi)
+            h = layer.LayerNorm(xi)
+            code, _ = layer.hash(h)
+        loss = ((out.float() - target) ** 2).sum()
+        loss.backward()
+        return out.detach(), code.detach(), xi.grad.detach(), {k: v.grad.detach().clone() for k, v in layer.named_parameters()}
+
+    out32, code32, gx32, gp32 = step(False)
+    out16, code16, gx16, gp16 = step(True)
+    assert out16.dtype == torch.float32 and out16.shape == (B, Do)
+    assert all(torch.isfinite(v).all() for v in gp16.values()) and torch.isfinite(gx16).all()
+    if projection == "bh4":
+        assert torch.equal(code16, code32)
+        assert relmax(npf(out16), npf(out32)) <= 1e-5
+        assert relmax(npf(gx16), npf(gx32)) <= 1e-4
+        for k in gp32:
+            assert relmax(npf(gp16[k]), npf(gp32[k])) <= 1e-4, k
+    else:
+        agree = (code16 == code32).all(dim=1).cpu().numpy()
+        frac_codes = (code16 == code32).float().mean().item()
+        assert frac_codes > 0.99                              # float16 z: a few signs flip near zero
+        if agree.any():
+            # same rows gathered; the scores come from float16 z, so they differ at half precision
+            assert relmax(npf(out16)[agree], npf(out32)[agree]) <= 2e-2
+            assert relmax(npf(gx16)[agree], npf(gx32)[agree]) <= 5e-2

@@ -1095,3 +1095,104 @@ def test_scatter_duplicates_zipf():
     g = rng.randn(B, Do).astype(np.float32)
     want = oracle.scatter_add(idx, g.astype(np.float64), w.astype(np.float64), T * S)
     assert relmax(cabi.scatter_add(idx, g, w, T * S), want) <= 1e-5
+
+
+# ----------------------------------------------------------------------------- config 3 at full size
+
+@pytest.fixture(scope="module")
+def config3():
+    """BASELINE.json config 3: 16384 tokens, 512 tables x 256 entries x 1024 columns (537 MB of fp32
+    rows, more than the Infinity Cache holds; 268 MB as bf16), weights uniform (0, 1]."""
+    rng = np.random.default_rng(33)
+    B, T, S, Do = 16384, 512, 256, 1024
+    tables = rng.standard_normal((T, S, Do), dtype=np.float32)
+    tables *= np.float32(0.02)
+    code = rng.integers(0, S, size=(B, T), dtype=np.int32)
+    idx = code + (np.arange(T, dtype=np.int32) * S)[None]
+    w = (1.0 - rng.random((B, T), dtype=np.float32)).astype(np.float32)
+    bias = (0.001 * rng.standard_normal(Do)).astype(np.float32)
+    # a random sample of tokens, the first few and the whole tail of the last tile
+    sub = np.unique(np.concatenate([rng.choice(B, 64, replace=False), np.arange(B - 40, B), np.arange(0, 8)]))
+    # sum_b w[b,t] over the tokens with code s: what the all-token checksums are formed from
+    cnt = np.zeros((T, S), np.float64)
+    np.add.at(cnt, (np.broadcast_to(np.arange(T), (B, T)), code), w.astype(np.float64))
+    return dict(B=B, T=T, S=S, Do=Do, tables=tables, code=code, idx=idx, w=w, bias=bias, sub=sub, cnt=cnt)
+
+
+def _rows64(src_f32, idx):
+    """The rows a sample of tokens reads, as a compact float64 table with re-numbered indices."""
+    uniq, inv = np.unique(idx, return_inverse=True)
+    return src_f32[uniq].astype(np.float64), inv.reshape(idx.shape).astype(np.int32)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_config3_gather_full_size(config3, bf16):
+    c = config3
+    B, T, S, Do = c["B"], c["T"], c["S"], c["Do"]
+    plan = cabi.lookup_gather_plan(B, T, S, Do, bf16)
+    assert plan[0] in (1, 2), plan                       # a table-major LDS kernel, the planner's own choice
+    flat = c["tables"].reshape(T * S, Do)
+    src = oracle.bf16_round(flat) if bf16 else flat
+    wide = oracle.bf16_widen(src) if bf16 else flat     # the values the kernel multiplies
+    got = cabi.lookup_gather(c["code"], c["w"], src.reshape(T, S, Do), c["bias"], bf16=bf16)
+    assert not np.isnan(got).any()
+    sub = c["sub"]
+    rows, ridx = _rows64(wide, c["idx"][sub])
+    want = oracle.gather_add(ridx, rows, c["w"][sub].astype(np.float64)) + c["bias"]
+    assert relmax(got[sub], want) <= 1e-5
+    if bf16:
+        rows32, _ = _rows64(flat, c["idx"][sub])
+        assert relmax(got[sub], oracle.gather_add(ridx, rows32, c["w"][sub].astype(np.float64)) + c["bias"]) <= 1e-2
+    # every token against the token-major kernel (same rows, the same order of additions)
+    assert relmax(got, cabi.gather_add(c["idx"], src, c["w"], bf16=bf16).astype(np.float64) + c["bias"]) <= 2e-6
+    # checksum over all tokens: sum_b out[b] = B * bias + sum_{t,s} cnt[t,s] * tables[t,s]
+    want_sum = B * c["bias"].astype(np.float64)
+    for t0 in range(0, T, 64):
+        want_sum = want_sum + np.einsum("ts,tsd->d", c["cnt"][t0:t0 + 64], wide[t0 * S:(t0 + 64) * S].reshape(64, S, Do).astype(np.float64))
+    assert relmax(got.astype(np.float64).sum(0), want_sum) <= 1e-5
+    # a second launch gives the same bits (fixed order of additions)
+    assert np.array_equal(got, cabi.lookup_gather(c["code"], c["w"], src.reshape(T, S, Do), c["bias"], bf16=bf16))
+
+
+def test_config3_inner_product_full_size(config3):
+    c = config3
+    B, T, S, Do = c["B"], c["T"], c["S"], c["Do"]
+    rng = np.random.default_rng(34)
+    g = rng.standard_normal((B, Do), dtype=np.float32)
+    got = cabi.lookup_inner(c["code"], g, c["tables"])
+    assert not np.isnan(got).any()
+    sub = c["sub"]
+    flat = c["tables"].reshape(T * S, Do)
+    rows, ridx = _rows64(flat, c["idx"][sub])
+    want = oracle.indexed_inner_product(ridx, g[sub].astype(np.float64), rows)
+    assert relmax(got[sub], want) <= 1e-5
+    # every (token, table) against the token-major kernel
+    assert relmax(got, cabi.indexed_inner_product(c["idx"], g, flat)) <= 1e-5
+    # duality with the forward: <G(w), g> = sum_bt w[b,t] * grad_score[b,t]
+    fwd = cabi.lookup_gather(c["code"], c["w"], c["tables"], None)
+    lhs = float((fwd.astype(np.float64) * g).sum())
+    rhs = float((got.astype(np.float64) * c["w"]).sum())
+    assert abs(lhs - rhs) <= 1e-5 * max(abs(lhs), 1.0) * 10
+
+
+def test_config3_scatter_full_size(config3):
+    c = config3
+    B, T, S, Do = c["B"], c["T"], c["S"], c["Do"]
+    rng = np.random.default_rng(35)
+    g = rng.standard_normal((B, Do), dtype=np.float32)
+    got = cabi.lookup_scatter_sorted(c["code"], c["w"], g, S)
+    assert not np.isnan(got).any()
+    # column sums: sum_s grad[t,s,:] = sum_b w[b,t] g[b,:]
+    want_sum = c["w"].astype(np.float64).T @ g.astype(np.float64)
+    assert relmax(got.astype(np.float64).sum(1), want_sum) <= 1e-5
+    # a few tables in full against the oracle
+    for t in (0, 255, 511):
+        want_t = oracle.scatter_add(c["code"][:, t:t + 1], g.astype(np.float64), c["w"][:, t:t + 1].astype(np.float64), S)
+        assert relmax(got[t], want_t) <= 1e-5
+    # the LDS form on the same inputs
+    assert relmax(got, cabi.lookup_scatter(c["code"], c["w"], g, S)) <= 1e-5
+    # duality with the forward: <G(w), g> = <grad_tables, tables>
+    fwd = cabi.lookup_gather(c["code"], c["w"], c["tables"], None)
+    lhs = float((fwd.astype(np.float64) * g).sum())
+    rhs = float(np.einsum("tsd,tsd->", got.astype(np.float64), c["tables"].astype(np.float64)))
+    assert abs(lhs - rhs) <= 1e-5 * max(abs(lhs), 1.0) * 10
