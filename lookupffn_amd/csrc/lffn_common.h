@@ -185,10 +185,13 @@ constexpr int TOUCH_SINK_BYTES = 256;
 constexpr int WAIT_VMCNT_0 = 0x0F70;
 constexpr int WAIT_VMCNT_1 = 0x0F71;
 __device__ __forceinline__ void l2_touch(const char *base, uint32_t lane_offset, uint32_t lds_byte_addr) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
-                 :
+    // M0 is put back: the compiler reserves it for its own use and does not honour a clobber
+    // declaration of it, so the statement must leave it as it found it
+    uint32_t saved_m0;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2\n\ts_mov_b32 m0, %0"
+                 : "=&s"(saved_m0)
                  : "v"(lane_offset), "s"(base), "s"(lds_byte_addr)
-                 : "memory", "m0");
+                 : "memory");
 }
 
 // The line of a region of `nlines` 128-byte lines that lane `tid` of workgroup `member` of a team of

@@ -67,10 +67,13 @@ struct LdsGatherArgs {
 __device__ __forceinline__ void lds_dma16(const char *table, uint32_t lane_offset, uint32_t lds_byte_addr) {
     // scalar base + 32-bit lane offset: the lane offsets are the same for every table, so they
     // stay in registers and a table costs no address arithmetic on the vector unit
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :
+    // M0 is put back: the compiler reserves it for its own use and does not honour a clobber
+    // declaration of it, so the statement must leave it as it found it
+    uint32_t saved_m0;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b32 m0, %0"
+                 : "=&s"(saved_m0)
                  : "v"(lane_offset), "s"(table), "s"(lds_byte_addr)
-                 : "memory", "m0");
+                 : "memory");
 }
 
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));

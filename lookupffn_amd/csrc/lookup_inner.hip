@@ -52,10 +52,13 @@ struct InnerArgs {
 // the copy with the LDS reads of the other buffer; the caller waits with vmcnt(0)
 // before the barrier that publishes the buffer.
 __device__ __forceinline__ void lds_dma16(const char *gptr, uint32_t lds_byte_addr) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                 :
+    // M0 is put back: the compiler reserves it for its own use and does not honour a clobber
+    // declaration of it, so the statement must leave it as it found it
+    uint32_t saved_m0;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
+                 : "=&s"(saved_m0)
                  : "v"(gptr), "s"(lds_byte_addr)
-                 : "memory", "m0");
+                 : "memory");
 }
 
 template <bool FULL>
