@@ -14,7 +14,8 @@
  * Conventions
  *   - Every pointer is a DEVICE pointer to a contiguous row-major array that the
  *     caller owns.  The library allocates nothing, frees nothing and keeps no
- *     state between calls.
+ *     results between calls (it remembers, per device, which kernels were granted
+ *     large LDS sizes and where its one static scratch array lives).
  *   - Forward outputs are fully overwritten (no zero-initialisation needed).
  *     Only lffn_scatter_add_f32 accumulates into its output.
  *   - Calls are asynchronous on `stream` (NULL = the legacy default stream) and
@@ -38,8 +39,9 @@ extern "C" {
 #define LFFN_ERR_BAD_ARG     -1   /* null pointer, negative size, misaligned pointer */
 #define LFFN_ERR_UNSUPPORTED -2   /* a shape outside what the kernels are built for */
 #define LFFN_ERR_LAUNCH      -3   /* hipGetLastError() after the launch was not hipSuccess */
+#define LFFN_ERR_SCRATCH     -4   /* an entry point that allocates nothing: the shape exceeds its static scratch */
 
-#define LFFN_ABI_VERSION 3
+#define LFFN_ABI_VERSION 4
 
 /* ABI version of the loaded library (LFFN_ABI_VERSION at build time). */
 int lffn_version(void);
@@ -208,6 +210,26 @@ int lffn_sum_partials_f32(const float *parts_a, float *out_a, int64_t n_a, const
 int lffn_layer_norm_bwd_f32(const float *x, const float *ln_weight, float ln_eps, const float *g_y, float *g_x,
                             float *part_weight, float *part_bias, int64_t B, int64_t H, int64_t R,
                             int64_t num_partials, void *stream);
+
+/*
+ * lffn_layer_norm_bwd_f32 for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): the partial sums go to a buffer
+ * the library itself holds (a static device array of 4 MiB: 2 x 512 partials x 1024 columns of fp32,
+ * present on every GPU the library runs on for the life of the process) and the column sums are
+ * finished here, so the caller passes only inputs and outputs:
+ *   g_x [B, H] as lffn_layer_norm_bwd_f32;  g_weight [H] = sum_b g * x^;  g_bias [H] = sum_b g
+ * with min(512, max(1, ceil(B / 4))) partials, added up by lffn_sum_partials_f32 (chunks = 1): the
+ * results are bit-identical to those two calls with that many partials.  No hipMalloc, hipFree or
+ * other allocating call is made.  Shapes whose partials exceed the buffer (H > 1024) return
+ * LFFN_ERR_SCRATCH.  The buffer keeps the last call's contents; every call overwrites all it reads, so
+ * nothing needs clearing.  All calls on one GPU share the one buffer: calls that overlap on a GPU
+ * (two streams, two threads) race.  ln_weight may be null (no affine; g_weight is still written).
+ * No counterpart in the reference (it has no entry point of this kind; the operator is the LayerNorm
+ * backward autograd records for PL/lookup.py:99).
+ */
+int lffn_layer_norm_bwd_noalloc_f32(const float *x, const float *ln_weight, float ln_eps, const float *g_y,
+                                    float *g_x, float *g_weight, float *g_bias, int64_t B, int64_t H, int64_t R,
+                                    void *stream);
 
 /*
  * The whole layer in one launch, for small batches without gradient (PL/lookup.py:99-108):

@@ -15,12 +15,13 @@ _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 # LOOKUPFFN_HIP_LIB points at another build of the same ABI (e.g. a tuning build)
 LIB_PATH = os.environ.get("LOOKUPFFN_HIP_LIB") or os.path.join(_PKG_DIR, "liblookupffn_hip.so")
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 LFFN_OK = 0
 LFFN_ERR_BAD_ARG = -1
 LFFN_ERR_UNSUPPORTED = -2
 LFFN_ERR_LAUNCH = -3
+LFFN_ERR_SCRATCH = -4
 
 _vp = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -46,6 +47,7 @@ SIGNATURES = {
     "lffn_lookup_ffn_fused_f32": [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
                                   _i64, _i64, _i64, ctypes.c_float, ctypes.c_float, _vp],
     "lffn_layer_norm_bwd_f32": [_vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
+    "lffn_layer_norm_bwd_noalloc_f32": [_vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "lffn_bh4_block_wgrad_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp],
     "lffn_bh4_fold_f32": [_vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "lffn_bh4_block_f32": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp],

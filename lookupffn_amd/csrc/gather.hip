@@ -453,6 +453,7 @@ extern "C" const char *lffn_error_string(int code) {
         case LFFN_ERR_BAD_ARG: return "bad argument (null or misaligned pointer, negative or inconsistent size)";
         case LFFN_ERR_UNSUPPORTED: return "shape not supported by the gfx950 kernels";
         case LFFN_ERR_LAUNCH: return "kernel launch failed";
+        case LFFN_ERR_SCRATCH: return "the shape needs more scratch memory than the library's static buffer holds";
         default: return "unknown error code";
     }
 }

@@ -164,6 +164,34 @@ __global__ __launch_bounds__(256) void sum_partials_kernel(SumPartialsArgs a) {
 
 }  // namespace
 
+// Scratch of lffn_layer_norm_bwd_noalloc_f32: the per-workgroup partial sums of the weight and bias
+// gradients, [2][num_partials][H] with num_partials <= LN_NOALLOC_PARTIALS and H <= 256 * NJ_MAX.  Held
+// by every GPU the library runs on until the process ends.  In host code this name is only a handle
+// for hipGetSymbolAddress, never a device address.
+constexpr int LN_NOALLOC_PARTIALS = 512;
+constexpr size_t LN_NOALLOC_FLOATS = size_t(2) * LN_NOALLOC_PARTIALS * 256 * NJ_MAX;      // 4 MiB
+static __device__ __align__(256) float ln_noalloc_scratch[LN_NOALLOC_FLOATS];
+
+// The device address of ln_noalloc_scratch on the current device, looked up once per device (each GPU
+// holds its own copy of the array at its own address).  Null when the lookup fails.
+static float *ln_noalloc_scratch_ptr() {
+    static std::atomic<float *> known[LFFN_MAX_DEVICES];
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= LFFN_MAX_DEVICES) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    float *p = known[dev].load(std::memory_order_acquire);
+    if (p) return p;
+    void *sym = nullptr;
+    if (hipGetSymbolAddress(&sym, HIP_SYMBOL(ln_noalloc_scratch)) != hipSuccess || !sym) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    known[dev].store(static_cast<float *>(sym), std::memory_order_release);     // two threads racing store the same address
+    return static_cast<float *>(sym);
+}
+
 extern "C" int lffn_sum_partials_f32(const float *parts_a, float *out_a, int64_t n_a, const float *parts_b,
                                      float *out_b, int64_t n_b, int64_t num_partials, int64_t chunks,
                                      void *stream) {
@@ -208,4 +236,23 @@ extern "C" int lffn_layer_norm_bwd_f32(const float *x, const float *ln_weight, f
     else if (H <= 768) hipLaunchKernelGGL((layer_norm_bwd_kernel<3>), grid, dim3(256), 0, st, a);
     else hipLaunchKernelGGL((layer_norm_bwd_kernel<4>), grid, dim3(256), 0, st, a);
     return lffn_launch_status();
+}
+
+extern "C" int lffn_layer_norm_bwd_noalloc_f32(const float *x, const float *ln_weight, float ln_eps, const float *g_y,
+                                               float *g_x, float *g_weight, float *g_bias, int64_t B, int64_t H,
+                                               int64_t R, void *stream) {
+    LFFN_REQUIRE(B >= 0 && H >= 1, LFFN_ERR_BAD_ARG);
+    // as many partials as workgroups that have a row, at most LN_NOALLOC_PARTIALS
+    const int64_t want = (B + 3) / 4;
+    const int64_t num_partials = want < 1 ? 1 : (want > LN_NOALLOC_PARTIALS ? LN_NOALLOC_PARTIALS : want);
+    LFFN_REQUIRE(size_t(2) * size_t(num_partials) * size_t(H) <= LN_NOALLOC_FLOATS, LFFN_ERR_SCRATCH);
+    LFFN_REQUIRE(g_weight && g_bias && lffn_aligned16(g_weight) && lffn_aligned16(g_bias), LFFN_ERR_BAD_ARG);
+    float *scratch = ln_noalloc_scratch_ptr();
+    LFFN_REQUIRE(scratch, LFFN_ERR_LAUNCH);
+    float *part_w = scratch, *part_b = scratch + num_partials * H;
+    // every one of the num_partials workgroups writes its row of both arrays, so nothing of the last
+    // call's contents is read and nothing needs clearing
+    const int rc = lffn_layer_norm_bwd_f32(x, ln_weight, ln_eps, g_y, g_x, part_w, part_b, B, H, R, num_partials, stream);
+    if (rc != LFFN_OK) return rc;
+    return lffn_sum_partials_f32(part_w, g_weight, H, part_b, g_bias, H, num_partials, 1, stream);
 }
