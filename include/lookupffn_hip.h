@@ -387,16 +387,27 @@ int lffn_lookup_gather_residual_bf16(const int32_t *code, const float *score, co
                                      int64_t B, int64_t T, int64_t S, int64_t Do, void *stream);
 
 /*
- * The same gather with a caller-provided workspace, for batches of a few thousand tokens: too
- * few (token tile, column slice) units to fill the chip at the tile sizes that make staging
- * tables in LDS pay.  Several workgroups then share a unit, each adding a range of the tables
- * into its own partial output in the workspace, and a second kernel adds the partials, in table
- * order, with bias and residual (results are reproducible, and equal to the one-part kernel's
- * up to the association of the fp32 sums).  lffn_lookup_gather_workspace_bytes sets *bytes to
- * the workspace that pays for a shape, or to 0 when the plain entry points are as fast
- * (16384 tokens and more at the RoBERTa-base tables, or very few tokens); with a null or too
- * small workspace the _ws entry points behave exactly like lffn_lookup_gather_residual_*.
- * residual may be null.  Same replacement as lffn_lookup_gather_f32 (PL/lookup.py:120-130, 108).
+ * The same gather with a caller-provided workspace, which two forms use:
+ *  - many tokens, fp32 rows, S = 256, an even number of tables (16384 tokens at the RoBERTa-base
+ *    tables): the four-lanes-per-token kernel.  A small kernel first packs the (code, score) pairs
+ *    into a stream of 12-byte records in the workspace (6 bytes per (token, table)), laid out so
+ *    that a wavefront of the gather kernel reads its records as one contiguous block; the gather
+ *    kernel walks 128-byte column slices, two tables per LDS buffer, 1024 to 2048 tokens per
+ *    workgroup.  Within a table pair a token adds the two rows in an order that depends on its
+ *    index (bit 1), so results equal lffn_lookup_gather_f32's up to the association of the fp32
+ *    sums; they are reproducible from run to run;
+ *  - a few thousand tokens: too few (token tile, column slice) units to fill the chip at the tile
+ *    sizes that make staging tables in LDS pay.  Several workgroups then share a unit, each adding
+ *    a range of the tables into its own partial output in the workspace, and a second kernel adds
+ *    the partials, in table order, with bias and residual (reproducible, and equal to the one-part
+ *    kernel's up to the association of the fp32 sums).
+ * lffn_lookup_gather_workspace_bytes sets *bytes to the workspace that pays for a shape, or to 0
+ * when the plain entry points are as fast (very few tokens, bf16 rows at 16384 tokens and more,
+ * tables beyond the 256 MB memory-side cache); with a null or too small workspace the _ws entry
+ * points behave exactly like lffn_lookup_gather_residual_*.  The workspace is scratch: 16-byte
+ * aligned device memory, contents undefined afterwards; calls that share one must be ordered on
+ * the stream.  residual may be null.
+ * Same replacement as lffn_lookup_gather_f32 (PL/lookup.py:120-130, 108).
  */
 int lffn_lookup_gather_workspace_bytes(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t bf16, int64_t *bytes);
 int lffn_lookup_gather_ws_f32(const int32_t *code, const float *score, const float *tables, const float *bias,
@@ -412,7 +423,9 @@ int lffn_lookup_gather_ws_bf16(const int32_t *code, const float *score, const ui
  * tables through LDS, or 0 when the token-major kernel is used (small batches,
  * S > 256); *tables_per_buffer (may be NULL) receives 0 (token-major), 1 (256-byte
  * column slices, one table per LDS buffer) or 2 (128-byte slices, two tables per
- * buffer).  Pure host function, no GPU work; negative on bad arguments.
+ * buffer).  (The workspace entry points may run a form this function does not report:
+ * 3, the four-lanes-per-token kernel.)  Pure host function, no GPU work; negative on
+ * bad arguments.
  * No counterpart in the reference (its gather has one kernel, gather_fp32.cu:6-36).
  */
 int lffn_lookup_gather_plan(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t bf16,
@@ -422,11 +435,13 @@ int lffn_lookup_gather_plan(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t
  * lffn_lookup_gather_{f32,bf16} with the kernel named by the caller instead of
  * chosen by lffn_lookup_gather_plan (for tuning, and so that every built kernel
  * can be tested on any shape): tables_per_buffer 0, 1 or 2 as reported by the plan
- * function; tokens_per_workgroup a multiple of 64 (one table per buffer: 256, 512,
- * 832, 1024; bf16 256, 512) or of 128 (two tables per buffer: 512, 1024, 1664,
- * 2048; bf16 512, 1024), ignored for 0.  LFFN_ERR_UNSUPPORTED if that kernel is not
- * built or the shape does not meet its conditions (S <= 256, Do a multiple of the
- * slice width).  No counterpart in the reference.
+ * function, or 3 for the four-lanes-per-token kernel (fp32 only; here without the
+ * record stream: it reads code and score itself); tokens_per_workgroup a multiple of
+ * 64 (one table per buffer: 256, 512, 832, 1024; bf16 256, 512), of 128 (two tables
+ * per buffer: 512, 1024, 1664, 2048; bf16 512, 1024) or of 256 (form 3: 1024, 1536,
+ * 1792, 2048), ignored for 0.  LFFN_ERR_UNSUPPORTED if that kernel is not built or the
+ * shape does not meet its conditions (S <= 256, Do a multiple of the slice width; form
+ * 3: S = 256, T even).  No counterpart in the reference.
  */
 int lffn_lookup_gather_planned_f32(const int32_t *code, const float *score, const float *tables,
                                    const float *bias, float *out,

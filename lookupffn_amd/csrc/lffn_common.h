@@ -78,6 +78,14 @@ static inline bool lffn_grant_dynamic_lds(const void *kernel, size_t lds_bytes, 
     return true;
 }
 
+// lookup_gather_quad.hip: the two-tables-per-buffer LDS gather with four lanes per token, fp32 rows (not exported)
+__attribute__((visibility("hidden")))
+int lffn_internal_lookup_gather_quad(const int32_t *code, const float *score, const void *tables,
+                                     const float *bias, const float *residual, float *out, int64_t B, int64_t T,
+                                     int64_t S, int64_t Do, int np, void *workspace, void *stream);
+__attribute__((visibility("hidden")))
+int64_t lffn_internal_quad_stream_bytes(int64_t B, int64_t T);
+
 static inline int lffn_launch_status() {
     return hipGetLastError() == hipSuccess ? LFFN_OK : LFFN_ERR_LAUNCH;
 }

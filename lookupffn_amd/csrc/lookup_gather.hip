@@ -349,6 +349,11 @@ struct GatherPlan {
     double us;             // predicted time
 };
 
+// microseconds per (table pair, pass of 256 tokens) of the four-lanes-per-token kernel, measured on MI355X
+// at 16384 tokens: 128 x 256 x 768 fp32 tables (cached) and 512 x 256 x 1024 (537 MB, beyond the cache)
+constexpr double QUAD_MARGIN = 0.92;      // the form must promise this much to be worth its workspace
+constexpr double QUAD_US_PER_PAIR_PASS = 0.28, QUAD_US_PER_PAIR_PASS_BIG = 0.40;
+
 template <bool BF16>
 GatherPlan plan_gather(int64_t B, int64_t T, int64_t S, int64_t Do) {
     // token-major: every token reads its T rows from L2 / Infinity Cache, measured 9 TB/s
@@ -377,6 +382,29 @@ GatherPlan plan_gather(int64_t B, int64_t T, int64_t S, int64_t Do) {
         const int64_t rounds = (tiles * nslices + 255) / 256;
         const double us = double(rounds) * double(T) * (big ? o.us_big : o.us_per_table);
         if (us < best_us) { best_us = us; best = GatherPlan{o.kind, o.np, us}; }
+    }
+    return best;
+}
+
+// The four-lanes-per-token form (lookup_gather_quad.hip; needs a workspace for its record stream): 128-byte
+// slices, 256*np tokens per workgroup, one round costs T/2 pairs x np passes x a measured cost per
+// (pair, pass) plus the packing kernel.  fp32 rows and an even number of tables only.
+template <bool BF16>
+GatherPlan plan_quad(int64_t B, int64_t T, int64_t S, int64_t Do) {
+    GatherPlan best{0, 0, 1e300};
+    if (BF16 || S != MAX_S || T < 8 || T % 2 != 0 || Do % 32 != 0 || B * T >= (int64_t(1) << 31) ||
+        2 * S * Do * 4 >= (int64_t(1) << 32))
+        return best;
+    const int64_t nslices = Do / 32;
+    if (((B + 1023) / 1024) * nslices < 192 || B * nslices > (int64_t(1) << 30)) return best;
+    const bool big = double(T) * double(S) * double(Do) * 4 > 200e6;
+    for (int np : {4, 6, 7, 8}) {
+        const int64_t tiles = (B + 256 * np - 1) / (256 * np);
+        const int64_t rounds = (tiles * nslices + 255) / 256;
+        const double per = big ? QUAD_US_PER_PAIR_PASS_BIG : QUAD_US_PER_PAIR_PASS;
+        const double us = double(rounds) * double(T / 2) * np * per +
+                          double(B) * double(T) * 14.0 / 3e6 + 4.0;      // packing: 8 bytes read, 6 written per (token, table)
+        if (us < best.us) best = GatherPlan{3, np, us};
     }
     return best;
 }
@@ -478,6 +506,10 @@ int64_t gather_pieces(int64_t B, int64_t T, int64_t S, int64_t Do) {
 template <bool BF16>
 bool plan_is_valid(const GatherPlan &p, int64_t B, int64_t T, int64_t S, int64_t Do) {
     if (p.kind == 0) return true;
+    if (p.kind == 3)        // four lanes per token: fp32 rows, an even number of tables, 32-bit offsets inside a table pair
+        return !BF16 && (p.np == 4 || p.np == 6 || p.np == 7 || p.np == 8) && S == MAX_S && T >= 2 && T % 2 == 0 &&
+               Do % 32 == 0 && B * T < (int64_t(1) << 31) && 2 * S * Do * 4 < (int64_t(1) << 32) &&
+               B * (Do / 32) <= (int64_t(1) << 30);
     if (p.kind != 1 && p.kind != 2) return false;
     const bool np_ok = BF16 ? (p.np == 4 || p.np == 8) : (p.np == 4 || p.np == 8 || p.np == 13 || p.np == 16);
     const int cols = (p.kind == 1 ? 256 : 128) / (BF16 ? 2 : 4);
@@ -504,17 +536,28 @@ int lookup_gather_entry(const int32_t *code, const float *score, const void *tab
     const int64_t each = kind_req < 0 ? gather_pieces<BF16>(B, T, S, Do) : B;
     if (each < B) {
         for (int64_t b0 = 0; b0 < B; b0 += each) {
+            // (a workspace serves every piece in turn: the launches are ordered on the stream)
             const int rc = lookup_gather_entry<BF16>(code + b0 * T, score + b0 * T, tables, bias,
                                                      residual ? residual + b0 * Do : nullptr, out + b0 * Do,
-                                                     B - b0 < each ? B - b0 : each, T, S, Do, -1, 0, stream);
+                                                     B - b0 < each ? B - b0 : each, T, S, Do, -1, 0, stream, workspace,
+                                                     workspace_bytes);
             if (rc != LFFN_OK) return rc;
         }
         return LFFN_OK;
     }
     GatherPlan plan;
+    void *quad_ws = nullptr;
     if (kind_req < 0) {
         plan = plan_gather<BF16>(B, T, S, Do);
         if (workspace) {
+            const GatherPlan qp = plan_quad<BF16>(B, T, S, Do);
+            if (qp.kind == 3 && qp.us < QUAD_MARGIN * plan.us && workspace_bytes >= lffn_internal_quad_stream_bytes(B, T)) {
+                LFFN_REQUIRE(lffn_aligned16(workspace), LFFN_ERR_BAD_ARG);
+                plan = qp;
+                quad_ws = workspace;
+            }
+        }
+        if (workspace && plan.kind != 3) {
             const SplitPlan sp = plan_split<BF16>(B, T, S, Do);
             if (sp.nparts > 1 && sp.us < 0.85 * plan.us && workspace_bytes >= int64_t(sp.nparts) * B * Do * 4) {
                 LFFN_REQUIRE(lffn_aligned16(workspace), LFFN_ERR_BAD_ARG);
@@ -542,13 +585,17 @@ int lookup_gather_entry(const int32_t *code, const float *score, const void *tab
         }
     } else {
         plan.kind = kind_req;
-        const int per_np = kind_req == 1 ? 64 : 128;
+        const int per_np = kind_req == 1 ? 64 : (kind_req == 3 ? 256 : 128);
         plan.np = kind_req == 0 ? 0 : tokens_req / per_np;
         LFFN_REQUIRE(kind_req == 0 || (tokens_req > 0 && tokens_req % per_np == 0), LFFN_ERR_BAD_ARG);
         LFFN_REQUIRE(plan_is_valid<BF16>(plan, B, T, S, Do), LFFN_ERR_UNSUPPORTED);
     }
     if (plan.kind == 0)
         return lffn_internal_lookup_gather_token_major(code, score, tables, bias, residual, out, B, T, S, Do, BF16, stream);
+    if (plan.kind == 3) {
+        if constexpr (BF16) return LFFN_ERR_UNSUPPORTED;
+        return lffn_internal_lookup_gather_quad(code, score, tables, bias, residual, out, B, T, S, Do, plan.np, quad_ws, stream);
+    }
     if (plan.kind == 2)
         return lffn_internal_lookup_gather_pair(code, score, tables, bias, residual, out, B, T, S, Do, BF16, plan.np, stream);
     const int np = plan.np;
@@ -602,9 +649,22 @@ extern "C" int lffn_lookup_gather_workspace_bytes(int64_t B, int64_t T, int64_t 
     LFFN_REQUIRE(bytes, LFFN_ERR_BAD_ARG);
     *bytes = 0;
     if (B < 1 || T < 1 || Do < 1 || !lffn_is_pow2(S) || Do % 64 != 0 || B * T >= (int64_t(1) << 31)) return LFFN_OK;
-    if ((bf16 ? gather_pieces<true>(B, T, S, Do) : gather_pieces<false>(B, T, S, Do)) < B)
-        return LFFN_OK;                                        // taken in pieces, none of which is split
+    const int64_t each = bf16 ? gather_pieces<true>(B, T, S, Do) : gather_pieces<false>(B, T, S, Do);
+    if (each < B) {                                            // taken in pieces, none of which is split
+        if (!bf16) {
+            const GatherPlan pp = plan_gather<false>(each, T, S, Do), pq = plan_quad<false>(each, T, S, Do);
+            if (pq.kind == 3 && pq.us < QUAD_MARGIN * pp.us) *bytes = lffn_internal_quad_stream_bytes(each, T);
+        }
+        return LFFN_OK;
+    }
     const GatherPlan plan = bf16 ? plan_gather<true>(B, T, S, Do) : plan_gather<false>(B, T, S, Do);
+    if (!bf16) {
+        const GatherPlan pq = plan_quad<false>(B, T, S, Do);
+        if (pq.kind == 3 && pq.us < QUAD_MARGIN * plan.us) {
+            *bytes = lffn_internal_quad_stream_bytes(B, T);
+            return LFFN_OK;
+        }
+    }
     const SplitPlan sp = bf16 ? plan_split<true>(B, T, S, Do) : plan_split<false>(B, T, S, Do);
     if (sp.nparts > 1 && sp.us < 0.85 * plan.us) *bytes = int64_t(sp.nparts) * B * Do * 4;
     return LFFN_OK;
@@ -651,5 +711,5 @@ extern "C" int lffn_lookup_gather_plan(int64_t B, int64_t T, int64_t S, int64_t 
     if (B < 0 || T < 0 || Do < 1 || !lffn_is_pow2(S) || Do % 64 != 0) return LFFN_ERR_BAD_ARG;
     const GatherPlan plan = bf16 ? plan_gather<true>(B, T, S, Do) : plan_gather<false>(B, T, S, Do);
     if (tables_per_buffer) *tables_per_buffer = plan.kind;
-    return plan.kind == 0 ? 0 : (plan.kind == 1 ? 64 : 128) * plan.np;
+    return plan.kind == 0 ? 0 : (plan.kind == 1 ? 64 : (plan.kind == 3 ? 256 : 128)) * plan.np;
 }

@@ -775,8 +775,77 @@ def test_lookup_gather_table_split_matches_oracle(B, T, S, Do, bf16):
 
 
 def test_lookup_gather_workspace_query_is_zero_where_the_plain_form_is_as_fast():
-    for shape in ((16384, 128, 256, 768), (65536, 128, 256, 768), (8, 128, 256, 768), (4096, 16, 256, 768), (0, 4, 16, 64)):
+    for shape in ((16384, 512, 256, 1024), (8, 128, 256, 768), (4096, 16, 256, 768), (0, 4, 16, 64),
+                  (16384, 128, 128, 768), (16384, 127, 256, 768)):
         assert cabi.lookup_gather_workspace_bytes(*shape) == 0, shape
+    for shape in ((16384, 128, 256, 768), (65536, 128, 256, 768), (16384, 512, 256, 1024)):
+        assert cabi.lookup_gather_workspace_bytes(*shape, bf16=True) == 0, shape
+
+
+# The four-lanes-per-token kernel (form 3), every tile size that is built, reading code and score
+# itself (the planned entry point passes no workspace).  (B, T, 256, Do): token counts that end inside
+# a tile, a wavefront and a quad; table counts that leave a chunk of 8 short (2, 4 and 6 tables).
+QUAD_PLANS = [(3, 1024), (3, 1536), (3, 1792), (3, 2048)]
+QUAD_SHAPES = [(3000, 20, 256, 256), (4133, 6, 256, 384), (1793, 34, 256, 128), (1, 2, 256, 64), (2050, 8, 256, 192)]
+
+
+@pytest.mark.parametrize("plan", QUAD_PLANS)
+@pytest.mark.parametrize("B,T,S,Do", QUAD_SHAPES)
+def test_lookup_gather_quad_kernels_match_oracle(B, T, S, Do, plan):
+    rng = np.random.RandomState(B + T + S + Do + plan[1])
+    tables, code, idx, w = _rand_gather(rng, B, T, S, Do)
+    bias = (0.001 * rng.randn(Do)).astype(np.float32)
+    flat = tables.reshape(T * S, Do)
+    got = cabi.lookup_gather(code, w, tables, bias, plan=plan)
+    assert not np.isnan(got).any()
+    want = oracle.gather_add(idx, flat.astype(np.float64), w.astype(np.float64)) + bias
+    assert relmax(got, want) <= 1e-5
+    dirty = (code + S * rng.randint(0, 5, size=code.shape)).astype(np.int32)      # bits above log2(S) are ignored
+    assert np.array_equal(cabi.lookup_gather(dirty, w, tables, bias, plan=plan), got)
+    assert relmax(cabi.lookup_gather(code, w, tables, None, plan=plan), want - bias) <= 1e-5
+
+
+def test_lookup_gather_quad_refusals():
+    from lookupffn_amd import _lib
+    lib = _lib.load()
+    # (code, score, tables, bias, out, B, T, S, Do): refused before any launch, so the pointers are never used
+    assert lib.lffn_lookup_gather_planned_f32(256, 256, 256, None, 256, 3000, 21, 256, 256, 3, 1024, None) == _lib.LFFN_ERR_UNSUPPORTED   # odd T
+    assert lib.lffn_lookup_gather_planned_f32(256, 256, 256, None, 256, 3000, 20, 128, 256, 3, 1024, None) == _lib.LFFN_ERR_UNSUPPORTED   # S != 256
+    assert lib.lffn_lookup_gather_planned_f32(256, 256, 256, None, 256, 3000, 20, 256, 256, 3, 1280, None) == _lib.LFFN_ERR_UNSUPPORTED   # 5 passes: not built
+    assert lib.lffn_lookup_gather_planned_f32(256, 256, 256, None, 256, 3000, 20, 256, 256, 3, 1000, None) == _lib.LFFN_ERR_BAD_ARG
+    assert lib.lffn_lookup_gather_planned_bf16(256, 256, 256, None, 256, 3000, 20, 256, 256, 3, 1024, None) == _lib.LFFN_ERR_UNSUPPORTED  # fp32 only
+
+
+# (B, T, S, Do): shapes for which the workspace query asks for the record stream of form 3: config 2,
+# a token count that ends inside a tile and a quad, a table count that leaves the last chunk of 8 short,
+# and enough tokens that the entry point takes them in pieces (one workspace serves every piece)
+QUAD_WS_SHAPES = [(16384, 128, 256, 768), (16001, 32, 256, 768), (20000, 30, 256, 512), (70001, 16, 256, 768)]
+
+
+@pytest.mark.parametrize("B,T,S,Do", QUAD_WS_SHAPES)
+def test_lookup_gather_record_stream_form_matches_oracle(B, T, S, Do):
+    rng = np.random.RandomState(B + T + Do)
+    tables, code, idx, w = _rand_gather(rng, B, T, S, Do)
+    bias = (0.001 * rng.randn(Do)).astype(np.float32)
+    res = rng.randn(B, Do).astype(np.float32)
+    flat = tables.reshape(T * S, Do)
+    nbytes = cabi.lookup_gather_workspace_bytes(B, T, S, Do)
+    assert nbytes > 0 and nbytes % 48 == 0 and nbytes < B * Do * 4           # the record stream, not the table split
+    got = cabi.lookup_gather_ws(code, w, tables, bias, residual=res)
+    assert not np.isnan(got).any()
+    sub = np.unique(np.concatenate([rng.choice(B, 128, replace=False), np.arange(B - 70, B), np.arange(0, 8)]))
+    want = oracle.gather_add(idx[sub], flat.astype(np.float64), w[sub].astype(np.float64))
+    assert relmax(got[sub], want + bias + res[sub]) <= 1e-5
+    # every token against the plain entry point (same rows, the two tables of a pair added in either order)
+    plain = cabi.lookup_gather(code, w, tables, bias, residual=res)
+    assert relmax(got, plain) <= 2e-6
+    # reproducible; a second call may reuse the workspace
+    assert np.array_equal(got, cabi.lookup_gather_ws(code, w, tables, bias, residual=res))
+    # without a workspace, or with one that is too small, the entry point is the plain one
+    assert np.array_equal(cabi.lookup_gather_ws(code, w, tables, bias, residual=res, ws_bytes=0), plain)
+    assert np.array_equal(cabi.lookup_gather_ws(code, w, tables, bias, residual=res, ws_bytes=nbytes - 48), plain)
+    # no bias, no residual
+    assert relmax(cabi.lookup_gather_ws(code, w, tables, None)[sub], want) <= 1e-5
 
 
 @pytest.mark.parametrize("plan", F32_PLANS)
@@ -811,7 +880,8 @@ def test_lookup_gather_plan_and_planned_entry():
     args = (256, 256, 256, None, 256, 3000, 20, 256, 256)
     assert lib.lffn_lookup_gather_planned_f32(*args, 1, 320, None) == _lib.LFFN_ERR_UNSUPPORTED      # 5 passes: not built
     assert lib.lffn_lookup_gather_planned_f32(*args, 1, 100, None) == _lib.LFFN_ERR_BAD_ARG          # not a multiple of 64
-    assert lib.lffn_lookup_gather_planned_f32(*args, 3, 512, None) == _lib.LFFN_ERR_UNSUPPORTED      # no such kernel
+    assert lib.lffn_lookup_gather_planned_f32(*args, 3, 512, None) == _lib.LFFN_ERR_UNSUPPORTED      # two passes: not built
+    assert lib.lffn_lookup_gather_planned_f32(*args, 4, 512, None) == _lib.LFFN_ERR_UNSUPPORTED      # no such kernel
     assert lib.lffn_lookup_gather_planned_bf16(*args, 2, 2048, None) == _lib.LFFN_ERR_UNSUPPORTED    # fp32 only
     big_s = (256, 256, 256, None, 256, 3000, 20, 512, 256)
     assert lib.lffn_lookup_gather_planned_f32(*big_s, 1, 512, None) == _lib.LFFN_ERR_UNSUPPORTED     # S > 256
