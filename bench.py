@@ -7,10 +7,16 @@ is already resident in HBM: fused LayerNorm+projection+hash kernel -> gather-add
 kernel (+bias), i.e. LookupFFN.forward in eval mode.  Prints ONE JSON line:
 
   value        whole-layer forward tokens/s (BASELINE.json's metric, config 2 by default)
-  roofline     the gather-add kernel: algorithmic ("logical") bytes per launch
-               = B*T*Do*e + B*T*8 + B*Do*4, divided by the kernel's average
-               duration measured with HIP events on the launch stream inside the
-               timed region, against the 8 TB/s HBM peak
+  roofline     the gather-add kernel against the bound that binds it.  The table-major
+               kernels serve every row read from LDS, so the bound is the LDS read
+               path: achieved = B*T*Do*e row bytes per launch / the kernel's average
+               duration (HIP events on the launch stream, inside the timed region),
+               peak = 256 B/clk/CU x 256 CUs x 2.4 GHz.  Beside it: the compulsory
+               HBM bytes (tables + codes + scores + output, each once) and the
+               fabric traffic measured with rocprofv3 --pmc, as fractions of 8 TB/s,
+               and the "logical" rate (every row read counted as memory traffic)
+               as logical_gbps.  Small shapes run the token-major form (rows from
+               L2): there the bound is "hbm" and achieved counts the compulsory bytes.
   cpu_baseline the CPU oracle (OpenMP C restatement of the reference's layer) on a
                bounded sample of the same workload, on the host cores of this box
 
@@ -62,12 +68,41 @@ WORKLOADS = {
                  desc="config 5: backward at the config-2 shape, codes Zipf(s=1.1) over 256 entries"),
 }
 
-# HBM bytes per launch of the gather kernel measured with rocprofv3 --pmc
-# (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); the summaries
-# are kept under profiles/.  None until measured for that workload.
-LDS_READ_PEAK_GBS = 76700.0     # microbenchmark: 125 bytes per clock per CU, 256 CUs
-MEASURED_TRAFFIC_BYTES = {"cfg2": 499747232, "cfg2b64": 499427315, "cfg3": 2840080784, "cfg3bf16": 1382263937,
-                          "cfg5": 943507857}
+# LDS read path of CDNA4: 256 bytes per clock per CU; 256 CUs at the 2.4 GHz peak engine clock.
+# (A read-only probe on this part reaches 180 B/clk/CU with linear ds_read_b128 from 16 wavefronts
+# per CU and 145 B/clk/CU with 16 lanes per randomly chosen 256-byte row, the gather's pattern.)
+LDS_READ_PEAK_GBS = 256 * 256 * 2.4
+LDS_PEAK_BASIS = ("256 B/clk/CU x 256 CUs x 2.4 GHz; a read-only ds_read_b128 probe on this part reaches 180 B/clk/CU "
+                  "(linear) and 145 B/clk/CU (16 lanes per random 256-byte row, this kernel's pattern)")
+# L2 read path: 16 channels x 128 B/clk per XCD, 8 XCDs, 2.4 GHz
+L2_READ_PEAK_GBS = 16 * 128 * 8 * 2.4
+# HBM-side bytes per launch of the gather (cfg5: scatter) kernels measured with rocprofv3 --pmc
+# (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size), and the kernel form they were
+# measured on; the summaries are kept under profiles/.  Reported only while the library still runs
+# that form for the workload (a figure for another kernel would be stale).
+MEASURED_TRAFFIC = {
+    "cfg2": {"bytes": 281335769, "form": "record stream (four lanes per token)"},
+}
+
+
+def measured_traffic(workload, form):
+    rec = MEASURED_TRAFFIC.get(workload)
+    return rec["bytes"] if rec and rec["form"] == form else None
+
+
+def gather_form(B, T, S, Do, bf16):
+    """Which gather kernel the library runs for a shape, as a short string (host-side queries only)."""
+    import ctypes
+
+    from lookupffn_amd import _lib
+    lib = _lib.load()
+    ws = ctypes.c_int64(0)
+    _lib.check(lib.lffn_lookup_gather_workspace_bytes(B, T, S, Do, int(bf16), ctypes.byref(ws)), "workspace query")
+    kind = ctypes.c_int32(-1)
+    tokens = lib.lffn_lookup_gather_plan(B, T, S, Do, int(bf16), ctypes.byref(kind))
+    if ws.value > 0:
+        return "record stream (four lanes per token)" if ws.value < B * Do * 4 else "table split"
+    return "token-major" if kind.value == 0 else f"{kind.value} table(s) per LDS buffer, {tokens} tokens per workgroup"
 
 
 def build_layer(wl, device):
@@ -225,6 +260,8 @@ def main_backward(args):
     scatter_ms = sum(a.elapsed_time(b) for a, b in evs) / args.steps
     scatter_bytes = B * T * Do * 4 * 2 + B * T * 8 + B * Do * 4
     achieved = scatter_bytes / (scatter_ms * 1e-3) / 1e9
+    row_bytes = B * T * Do * 4                                            # gradient rows read, one per (token, table)
+    compulsory = T * S * Do * 4 + B * T * 8 + B * Do * 4                  # tables written, codes + scores + g read, each once
 
     def timed(fn, n=10):
         fn(); torch.cuda.synchronize()
@@ -246,10 +283,16 @@ def main_backward(args):
         "config": {"workload": wl["desc"], "tokens": B, "tables": T, "table_size": S, "d_out": Do,
                    "step": "inner product (grad score) + scatter-add (grad tables) + one kernel: score "
                            "derivative, transposed BH4(block 1)x4, grad of diagonals and bias"},
-        "roofline": {"bound": "hbm", "kernel": "lookup_scatter (three launches: transpose/pack, sort, sorted accumulate)", "achieved": achieved,
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get("cfg5"),
-                     "algorithmic_bytes": scatter_bytes, "avg_kernel_ms": scatter_ms},
+        # the sorted scatter reads every (token, table)'s 3 KB gradient row from L2 into registers (the
+        # gradient matrix stays in the L2s) and writes each table row once: its bound is the L2 read path
+        "roofline": {"bound": "l2", "kernel": "lookup_scatter (three launches: transpose/pack, sort, sorted accumulate)",
+                     "achieved": row_bytes / (scatter_ms * 1e-3) / 1e9, "peak": L2_READ_PEAK_GBS, "unit": "GB/s",
+                     "frac": row_bytes / (scatter_ms * 1e-3) / 1e9 / L2_READ_PEAK_GBS,
+                     "peak_basis": "16 channels x 128 B/clk per XCD x 8 XCDs x 2.4 GHz",
+                     "traffic": measured_traffic("cfg5", "sorted"),
+                     "row_read_bytes": row_bytes, "avg_kernel_ms": scatter_ms,
+                     "hbm": {"compulsory_bytes": compulsory, "frac_of_peak": compulsory / (scatter_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
+                     "logical_gbps": achieved, "algorithmic_bytes": scatter_bytes},
         "stages_ms": {"lookup_inner": inner_ms, "scatter_add": scatter_ms, "project_hash_bwd": bwd_proj_ms},
     }
     if not args.no_cpu_baseline:
@@ -470,7 +513,27 @@ def main():
         t1 = time.perf_counter()
         sec = t1 - t0
     gather_ms = sum(a.elapsed_time(b) for a, b in timed_evs) / len(timed_evs)
-    achieved = gather_bytes / (gather_ms * 1e-3) / 1e9
+    logical_gbps = gather_bytes / (gather_ms * 1e-3) / 1e9
+    row_bytes = B * T * Do * esz                                          # one row per (token, table)
+    compulsory = T * S * Do * esz + B * T * 8 + B * Do * 4                # tables, codes + scores, output: each once
+    form = "whole layer in one launch (rows from L2)" if fused_layer else gather_form(B, T, S, Do, wl["bf16"])
+    lds_bound = not fused_layer and form != "token-major"
+    traffic = measured_traffic(args.workload, form)
+    hbm = {"compulsory_bytes": compulsory, "frac_of_peak": compulsory / (gather_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+           "measured_traffic_bytes": traffic,
+           "measured_frac_of_peak": None if traffic is None else traffic / (gather_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    if lds_bound:
+        achieved = row_bytes / (gather_ms * 1e-3) / 1e9
+        roofline = {"bound": "lds", "kernel": "lookup_gather: " + form, "achieved": achieved, "peak": LDS_READ_PEAK_GBS,
+                    "unit": "GB/s", "frac": achieved / LDS_READ_PEAK_GBS, "peak_basis": LDS_PEAK_BASIS, "traffic": traffic,
+                    "row_read_bytes": row_bytes, "avg_kernel_ms": gather_ms, "hbm": hbm,
+                    "logical_gbps": logical_gbps, "algorithmic_bytes": gather_bytes}
+    else:
+        achieved = compulsory / (gather_ms * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "kernel": ("lookup_ffn_fused: " if fused_layer else "lookup_gather: ") + form,
+                    "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                    "traffic": traffic, "avg_kernel_ms": gather_ms, "hbm": hbm,
+                    "logical_gbps": logical_gbps, "algorithmic_bytes": gather_bytes}
 
     # stage breakdown (outside the timed region)
     def timed(fn, n=20):
@@ -528,15 +591,7 @@ def main():
                             "outside the step); one kernel: gather-add + bias") if block else
                            ("one kernel: LayerNorm + BH4(block 1)x4 + mix + hash + gather-add + bias" if fused_layer else
                             "one kernel: LayerNorm + BH4(block 1)x4 + mix + hash; one kernel: gather-add + bias")},
-        "roofline": {"bound": "hbm", "kernel": "lookup_ffn_fused (the whole layer)" if fused_layer else "lookup_gather",
-                     "achieved": achieved, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-                     "algorithmic_bytes": gather_bytes, "avg_kernel_ms": gather_ms,
-                     # the rows are read from LDS, whose measured read rate (conflict-free ds_read_b128 on
-                     # every CU) is 76.7 TB/s on this part: the bound that actually applies to this kernel
-                     "lds": {"row_read_bytes": B * T * Do * esz, "peak": LDS_READ_PEAK_GBS, "unit": "GB/s",
-                             "frac": B * T * Do * esz / (gather_ms * 1e-3) / 1e9 / LDS_READ_PEAK_GBS}},
+        "roofline": roofline,
         "stages_ms": ({"whole_layer": gather_ms} if fused_layer else
                       {("layernorm_bh4block_hash" if block else "layernorm_project_hash"): hash_ms,
                        "gather_add": gather_ms}),
