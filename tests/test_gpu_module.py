@@ -3,6 +3,7 @@
 forward against the CPU oracle, gradients against the oracle's backward routines
 and against torch autograd of the reference's slow formulas.
 """
+import math
 from argparse import Namespace
 
 import numpy as np
@@ -297,6 +298,68 @@ def test_encoder_layers_match_float64_composition():
             assert (err <= 5e-5).mean() >= 0.9, err
             h = got
         assert relmax(npf(model.encoder.LayerNorm(h)), npf(out)) <= 1e-6
+
+
+@torch.no_grad()
+def test_encoder_full_size_ffn_outputs_match_oracle():
+    """BASELINE config 4 at its real layer shape: 12 layers, hidden 768, 12 heads, sequence 512, every FFN a
+    LookupFFN with 128 tables x 256 x 768 (PL/layer.py:66-78, PL/encoder.py:9-37), on a batch of 2 sequences.
+    Every layer's FFN output (residual included, as EncoderLayer.forward asks for it) is checked against the
+    oracle's layer evaluated on the GPU's own FFN input, so a code that flips in one layer does not compound;
+    the attention half of every layer is checked against torch's float64 evaluation of the literal formula."""
+    torch.manual_seed(12)
+    H, heads, L, Bq, nl = 768, 12, 512, 2, 12
+    cfg = Namespace(hidden_size=H, num_attention_heads=heads, attention_head_size=H // heads, attention_probs_dropout_prob=0.1,
+                    hidden_dropout_prob=0.1, layer_norm_eps=1e-5, num_hidden_layers=nl, vocab_size=50265,
+                    max_position_embeddings=L, type_vocab_size=1, pad_token_id=1,
+                    ffn_num_table=128, ffn_table_size=256, projection_type="bh4", block_size=1)
+    model = lookupffn_amd.Lookup(cfg).eval()
+    with torch.no_grad():
+        for layer in model.encoder.layer:           # tables and biases away from their zero / constant initial values
+            layer.FFN.tables.normal_(0.0, 0.02)
+            layer.FFN.bias.normal_(0.0, 0.01)
+    model = model.to(DEV)
+    ids = torch.randint(0, cfg.vocab_size, (Bq, L), device=DEV)
+    pos = torch.arange(L, device=DEV)[None].expand(Bq, L).contiguous()
+    mask = torch.ones(Bq, L, device=DEV)
+    mask[1, 400:] = 0
+    seen = []
+    hooks = [layer.FFN.register_forward_hook(lambda m, args, kwargs, out: seen.append((args[0], kwargs.get("residual"), out)),
+                                             with_kwargs=True)
+             for layer in model.encoder.layer]
+    with torch.no_grad():
+        out, _ = model(ids, torch.zeros_like(ids), pos, mask)
+        h = model.embeddings(ids, torch.zeros_like(ids), pos)
+    for hk in hooks:
+        hk.remove()
+    assert out.shape == (Bq, L, H) and len(seen) == nl
+    worst = []
+    for layer, (x_in, res, y) in zip(model.encoder.layer, seen):
+        # the attention half, float64, from the layer's input h
+        att = layer.attention
+        x64 = h.double().cpu()
+        a = torch.nn.functional.layer_norm(x64, (H,), att.LayerNorm.weight.double().cpu(), att.LayerNorm.bias.double().cpu(), 1e-5)
+        lin = lambda m, t: t @ m.weight.double().cpu().T + m.bias.double().cpu()
+        hd = lambda t: t.view(Bq, L, heads, H // heads).permute(0, 2, 1, 3)
+        q, k, v = hd(lin(att.query, a)), hd(lin(att.key, a)), hd(lin(att.value, a))
+        probs = torch.softmax(q @ k.transpose(-1, -2) / math.sqrt(H // heads) - 1000.0 * (1.0 - mask.double().cpu()[:, None, None, :]), dim=-1)
+        attn_out = lin(att.dense, (probs @ v).permute(0, 2, 1, 3).reshape(Bq, L, H)) + x64
+        assert relmax(npf(x_in), attn_out.numpy()) <= 2e-5
+        assert res is x_in                                       # the residual add runs inside the gather kernel
+        # the FFN half against the oracle, from the GPU's own FFN input
+        ffn = layer.FFN
+        p = ffn.hash.projection
+        x2 = npf(x_in).reshape(-1, H).astype(np.float64)
+        want = oracle.lookup_ffn(x2, npf(ffn.LayerNorm.weight), npf(ffn.LayerNorm.bias), 1e-5, npf(p.weight), npf(p.bias),
+                                 npf(ffn.tables), npf(ffn.bias), decay=0.7) + x2
+        err = np.abs(npf(y).reshape(-1, H) - want).max(axis=1) / np.abs(want).max()
+        # a token whose projection sits on a sign boundary may take another table row on the GPU
+        # (LayerNorm sums are associated differently): all but a few tokens agree to rounding
+        assert (err <= 2e-5).mean() >= 0.98, (err > 2e-5).sum()
+        worst.append(np.median(err))
+        h = y
+    assert max(worst) <= 2e-6
+    assert relmax(npf(model.encoder.LayerNorm(h)), npf(out)) <= 1e-6
 
 
 def test_hadamard_half_dispatch():
