@@ -41,7 +41,7 @@ extern "C" {
 #define LFFN_ERR_LAUNCH      -3   /* hipGetLastError() after the launch was not hipSuccess */
 #define LFFN_ERR_SCRATCH     -4   /* an entry point that allocates nothing: the shape exceeds its static scratch */
 
-#define LFFN_ABI_VERSION 4
+#define LFFN_ABI_VERSION 5
 
 /* ABI version of the loaded library (LFFN_ABI_VERSION at build time). */
 int lffn_version(void);
@@ -390,8 +390,8 @@ int lffn_lookup_gather_residual_bf16(const int32_t *code, const float *score, co
  * The same gather with a caller-provided workspace, which two forms use:
  *  - many tokens, fp32 rows, S = 256, an even number of tables (16384 tokens at the RoBERTa-base
  *    tables): the four-lanes-per-token kernel.  A small kernel first packs the (code, score) pairs
- *    into a stream of 12-byte records in the workspace (6 bytes per (token, table)), laid out so
- *    that a wavefront of the gather kernel reads its records as one contiguous block; the gather
+ *    into a stream of 12-byte records in the workspace (6 bytes per (token, table)), one row of
+ *    records per table pair, which the gather kernel copies into LDS a pair ahead; the gather
  *    kernel walks 128-byte column slices, two tables per LDS buffer, 1024 to 2048 tokens per
  *    workgroup.  Within a table pair a token adds the two rows in an order that depends on its
  *    index (bit 1), so results equal lffn_lookup_gather_f32's up to the association of the fp32
@@ -435,18 +435,24 @@ int lffn_lookup_gather_plan(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t
  * lffn_lookup_gather_{f32,bf16} with the kernel named by the caller instead of
  * chosen by lffn_lookup_gather_plan (for tuning, and so that every built kernel
  * can be tested on any shape): tables_per_buffer 0, 1 or 2 as reported by the plan
- * function, or 3 for the four-lanes-per-token kernel (fp32 only; here without the
- * record stream: it reads code and score itself); tokens_per_workgroup a multiple of
- * 64 (one table per buffer: 256, 512, 832, 1024; bf16 256, 512), of 128 (two tables
- * per buffer: 512, 1024, 1664, 2048; bf16 512, 1024) or of 256 (form 3: 1024, 1536,
- * 1792, 2048), ignored for 0.  LFFN_ERR_UNSUPPORTED if that kernel is not built or the
- * shape does not meet its conditions (S <= 256, Do a multiple of the slice width; form
- * 3: S = 256, T even).  No counterpart in the reference.
+ * function; tokens_per_workgroup a multiple of 64 (one table per buffer: 256, 512,
+ * 832, 1024; bf16 256, 512) or of 128 (two tables per buffer: 512, 1024, 1664, 2048;
+ * bf16 512, 1024), ignored for 0.  LFFN_ERR_UNSUPPORTED if that kernel is not built or
+ * the shape does not meet its conditions (S <= 256, Do a multiple of the slice width).
+ * lffn_lookup_gather_ws_planned_f32 also takes residual and a workspace and with them
+ * form 3, the four-lanes-per-token kernel (tokens_per_workgroup 1024, 1536, 1792 or
+ * 2048; S = 256, T even, Do a multiple of 32; the workspace must hold the record
+ * stream, 6 * T * (B + 2048) bytes, or the call is refused with LFFN_ERR_UNSUPPORTED).
+ * No counterpart in the reference.
  */
 int lffn_lookup_gather_planned_f32(const int32_t *code, const float *score, const float *tables,
                                    const float *bias, float *out,
                                    int64_t B, int64_t T, int64_t S, int64_t Do,
                                    int32_t tables_per_buffer, int32_t tokens_per_workgroup, void *stream);
+int lffn_lookup_gather_ws_planned_f32(const int32_t *code, const float *score, const float *tables,
+                                      const float *bias, const float *residual, float *out, void *workspace,
+                                      int64_t workspace_bytes, int64_t B, int64_t T, int64_t S, int64_t Do,
+                                      int32_t tables_per_buffer, int32_t tokens_per_workgroup, void *stream);
 int lffn_lookup_gather_planned_bf16(const int32_t *code, const float *score, const uint16_t *tables,
                                     const float *bias, float *out,
                                     int64_t B, int64_t T, int64_t S, int64_t Do,

@@ -349,10 +349,12 @@ struct GatherPlan {
     double us;             // predicted time
 };
 
-// microseconds per (table pair, pass of 256 tokens) of the four-lanes-per-token kernel, measured on MI355X
-// at 16384 tokens: 128 x 256 x 768 fp32 tables (cached) and 512 x 256 x 1024 (537 MB, beyond the cache)
+// The four-lanes-per-token kernel: microseconds per table pair of a workgroup = a fixed part (the 64 KB
+// copy, the records, the barrier) + a part per pass of 256 tokens.  Measured on MI355X at 4, 6, 7 and 8
+// passes: 1.40, 1.74, 1.93, 2.18 us, the same for 128 x 256 x 768 fp32 tables (in the memory-side
+// cache) and 512 x 256 x 1024 (537 MB, beyond it: the touch by turns hides the difference).
 constexpr double QUAD_MARGIN = 0.92;      // the form must promise this much to be worth its workspace
-constexpr double QUAD_US_PER_PAIR_PASS = 0.28, QUAD_US_PER_PAIR_PASS_BIG = 0.40;
+constexpr double QUAD_US_PER_PAIR = 0.62, QUAD_US_PER_PAIR_PASS = 0.195;
 
 template <bool BF16>
 GatherPlan plan_gather(int64_t B, int64_t T, int64_t S, int64_t Do) {
@@ -387,22 +389,20 @@ GatherPlan plan_gather(int64_t B, int64_t T, int64_t S, int64_t Do) {
 }
 
 // The four-lanes-per-token form (lookup_gather_quad.hip; needs a workspace for its record stream): 128-byte
-// slices, 256*np tokens per workgroup, one round costs T/2 pairs x np passes x a measured cost per
-// (pair, pass) plus the packing kernel.  fp32 rows and an even number of tables only.
+// slices, 256*np tokens per workgroup, one round of 256 workgroups costs T/2 pairs x the measured cost of a
+// pair at np passes; plus the packing kernel.  fp32 rows, 256-row tables and an even number of them only.
 template <bool BF16>
 GatherPlan plan_quad(int64_t B, int64_t T, int64_t S, int64_t Do) {
     GatherPlan best{0, 0, 1e300};
-    if (BF16 || S != MAX_S || T < 8 || T % 2 != 0 || Do % 32 != 0 || B * T >= (int64_t(1) << 31) ||
+    if (BF16 || S != MAX_S || T < 8 || T % 2 != 0 || T > (1 << 20) || Do % 32 != 0 || B * T >= (int64_t(1) << 31) ||
         2 * S * Do * 4 >= (int64_t(1) << 32))
         return best;
     const int64_t nslices = Do / 32;
     if (((B + 1023) / 1024) * nslices < 192 || B * nslices > (int64_t(1) << 30)) return best;
-    const bool big = double(T) * double(S) * double(Do) * 4 > 200e6;
     for (int np : {4, 6, 7, 8}) {
         const int64_t tiles = (B + 256 * np - 1) / (256 * np);
         const int64_t rounds = (tiles * nslices + 255) / 256;
-        const double per = big ? QUAD_US_PER_PAIR_PASS_BIG : QUAD_US_PER_PAIR_PASS;
-        const double us = double(rounds) * double(T / 2) * np * per +
+        const double us = double(rounds) * double(T / 2) * (QUAD_US_PER_PAIR + np * QUAD_US_PER_PAIR_PASS) +
                           double(B) * double(T) * 14.0 / 3e6 + 4.0;      // packing: 8 bytes read, 6 written per (token, table)
         if (us < best.us) best = GatherPlan{3, np, us};
     }
@@ -503,12 +503,32 @@ int64_t gather_pieces(int64_t B, int64_t T, int64_t S, int64_t Do) {
     return best_each;
 }
 
+// The four-lanes-per-token form over the whole batch (one launch, however many tokens: its tables come
+// through the touch by turns, so it has no use for pieces), if it promises to beat what the other forms
+// get for the batch by QUAD_MARGIN: pieces, the one-launch LDS forms, the table split.  kind 0 otherwise.
+template <bool BF16>
+GatherPlan choose_quad(int64_t B, int64_t T, int64_t S, int64_t Do) {
+    const GatherPlan none{0, 0, 1e300};
+    const GatherPlan qp = plan_quad<BF16>(B, T, S, Do);
+    if (qp.kind != 3) return none;
+    double other;
+    const int64_t each = gather_pieces<BF16>(B, T, S, Do);
+    if (each < B) {
+        other = double((B + each - 1) / each) * (plan_gather<BF16>(each, T, S, Do).us + 4.0);
+    } else {
+        other = plan_gather<BF16>(B, T, S, Do).us;
+        const SplitPlan sp = plan_split<BF16>(B, T, S, Do);
+        if (sp.nparts > 1 && sp.us < other) other = sp.us;
+    }
+    return qp.us < QUAD_MARGIN * other ? qp : none;
+}
+
 template <bool BF16>
 bool plan_is_valid(const GatherPlan &p, int64_t B, int64_t T, int64_t S, int64_t Do) {
     if (p.kind == 0) return true;
     if (p.kind == 3)        // four lanes per token: fp32 rows, an even number of tables, 32-bit offsets inside a table pair
         return !BF16 && (p.np == 4 || p.np == 6 || p.np == 7 || p.np == 8) && S == MAX_S && T >= 2 && T % 2 == 0 &&
-               Do % 32 == 0 && B * T < (int64_t(1) << 31) && 2 * S * Do * 4 < (int64_t(1) << 32) &&
+               T <= (1 << 20) && Do % 32 == 0 && B * T < (int64_t(1) << 31) && 2 * S * Do * 4 < (int64_t(1) << 32) &&
                B * (Do / 32) <= (int64_t(1) << 30);
     if (p.kind != 1 && p.kind != 2) return false;
     const bool np_ok = BF16 ? (p.np == 4 || p.np == 8) : (p.np == 4 || p.np == 8 || p.np == 13 || p.np == 16);
@@ -531,6 +551,15 @@ int lookup_gather_entry(const int32_t *code, const float *score, const void *tab
     LFFN_REQUIRE(lffn_aligned16(tables) && lffn_aligned16(out) && (!bias || lffn_aligned16(bias)) &&
                      (!residual || lffn_aligned16(residual)), LFFN_ERR_BAD_ARG);
     if (B == 0) return LFFN_OK;
+    if (kind_req < 0 && workspace) {
+        // (the packing kernel reads a table pair's codes and scores as 8-byte vectors)
+        const GatherPlan qp = choose_quad<BF16>(B, T, S, Do);
+        if (qp.kind == 3 && workspace_bytes >= lffn_internal_quad_stream_bytes(B, T) && (uintptr_t)code % 8 == 0 &&
+            (uintptr_t)score % 8 == 0) {
+            LFFN_REQUIRE(lffn_aligned16(workspace), LFFN_ERR_BAD_ARG);
+            return lffn_internal_lookup_gather_quad(code, score, tables, bias, residual, out, B, T, S, Do, qp.np, workspace, stream);
+        }
+    }
     // Many tokens, tables that fit the 256 MB Infinity Cache: take the tokens in pieces, one launch
     // after the other (gather_pieces).
     const int64_t each = kind_req < 0 ? gather_pieces<BF16>(B, T, S, Do) : B;
@@ -550,14 +579,6 @@ int lookup_gather_entry(const int32_t *code, const float *score, const void *tab
     if (kind_req < 0) {
         plan = plan_gather<BF16>(B, T, S, Do);
         if (workspace) {
-            const GatherPlan qp = plan_quad<BF16>(B, T, S, Do);
-            if (qp.kind == 3 && qp.us < QUAD_MARGIN * plan.us && workspace_bytes >= lffn_internal_quad_stream_bytes(B, T)) {
-                LFFN_REQUIRE(lffn_aligned16(workspace), LFFN_ERR_BAD_ARG);
-                plan = qp;
-                quad_ws = workspace;
-            }
-        }
-        if (workspace && plan.kind != 3) {
             const SplitPlan sp = plan_split<BF16>(B, T, S, Do);
             if (sp.nparts > 1 && sp.us < 0.85 * plan.us && workspace_bytes >= int64_t(sp.nparts) * B * Do * 4) {
                 LFFN_REQUIRE(lffn_aligned16(workspace), LFFN_ERR_BAD_ARG);
@@ -589,6 +610,11 @@ int lookup_gather_entry(const int32_t *code, const float *score, const void *tab
         plan.np = kind_req == 0 ? 0 : tokens_req / per_np;
         LFFN_REQUIRE(kind_req == 0 || (tokens_req > 0 && tokens_req % per_np == 0), LFFN_ERR_BAD_ARG);
         LFFN_REQUIRE(plan_is_valid<BF16>(plan, B, T, S, Do), LFFN_ERR_UNSUPPORTED);
+        if (plan.kind == 3) {       // needs the record stream's workspace
+            LFFN_REQUIRE(workspace && workspace_bytes >= lffn_internal_quad_stream_bytes(B, T), LFFN_ERR_UNSUPPORTED);
+            LFFN_REQUIRE(lffn_aligned16(workspace) && (uintptr_t)code % 8 == 0 && (uintptr_t)score % 8 == 0, LFFN_ERR_BAD_ARG);
+            quad_ws = workspace;
+        }
     }
     if (plan.kind == 0)
         return lffn_internal_lookup_gather_token_major(code, score, tables, bias, residual, out, B, T, S, Do, BF16, stream);
@@ -649,22 +675,13 @@ extern "C" int lffn_lookup_gather_workspace_bytes(int64_t B, int64_t T, int64_t 
     LFFN_REQUIRE(bytes, LFFN_ERR_BAD_ARG);
     *bytes = 0;
     if (B < 1 || T < 1 || Do < 1 || !lffn_is_pow2(S) || Do % 64 != 0 || B * T >= (int64_t(1) << 31)) return LFFN_OK;
-    const int64_t each = bf16 ? gather_pieces<true>(B, T, S, Do) : gather_pieces<false>(B, T, S, Do);
-    if (each < B) {                                            // taken in pieces, none of which is split
-        if (!bf16) {
-            const GatherPlan pp = plan_gather<false>(each, T, S, Do), pq = plan_quad<false>(each, T, S, Do);
-            if (pq.kind == 3 && pq.us < QUAD_MARGIN * pp.us) *bytes = lffn_internal_quad_stream_bytes(each, T);
-        }
+    if (!bf16 && choose_quad<false>(B, T, S, Do).kind == 3) {
+        *bytes = lffn_internal_quad_stream_bytes(B, T);
         return LFFN_OK;
     }
+    const int64_t each = bf16 ? gather_pieces<true>(B, T, S, Do) : gather_pieces<false>(B, T, S, Do);
+    if (each < B) return LFFN_OK;                              // taken in pieces, none of which is split
     const GatherPlan plan = bf16 ? plan_gather<true>(B, T, S, Do) : plan_gather<false>(B, T, S, Do);
-    if (!bf16) {
-        const GatherPlan pq = plan_quad<false>(B, T, S, Do);
-        if (pq.kind == 3 && pq.us < QUAD_MARGIN * plan.us) {
-            *bytes = lffn_internal_quad_stream_bytes(B, T);
-            return LFFN_OK;
-        }
-    }
     const SplitPlan sp = bf16 ? plan_split<true>(B, T, S, Do) : plan_split<false>(B, T, S, Do);
     if (sp.nparts > 1 && sp.us < 0.85 * plan.us) *bytes = int64_t(sp.nparts) * B * Do * 4;
     return LFFN_OK;
@@ -695,6 +712,16 @@ extern "C" int lffn_lookup_gather_planned_f32(const int32_t *code, const float *
     LFFN_REQUIRE(tables_per_buffer >= 0, LFFN_ERR_BAD_ARG);
     return lookup_gather_entry<false>(code, score, tables, bias, nullptr, out, B, T, S, Do, tables_per_buffer,
                                       tokens_per_workgroup, stream);
+}
+
+extern "C" int lffn_lookup_gather_ws_planned_f32(const int32_t *code, const float *score, const float *tables,
+                                                 const float *bias, const float *residual, float *out, void *workspace,
+                                                 int64_t workspace_bytes, int64_t B, int64_t T, int64_t S, int64_t Do,
+                                                 int32_t tables_per_buffer, int32_t tokens_per_workgroup, void *stream) {
+    LFFN_REQUIRE(tables_per_buffer >= 0, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(workspace_bytes >= 0 && (workspace || workspace_bytes == 0), LFFN_ERR_BAD_ARG);
+    return lookup_gather_entry<false>(code, score, tables, bias, residual, out, B, T, S, Do, tables_per_buffer,
+                                      tokens_per_workgroup, stream, workspace, workspace_bytes);
 }
 
 extern "C" int lffn_lookup_gather_planned_bf16(const int32_t *code, const float *score, const uint16_t *tables,

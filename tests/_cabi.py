@@ -271,6 +271,23 @@ def lookup_gather_ws(code, score, tables, bias=None, bf16=False, residual=None, 
     return host(out)
 
 
+def lookup_gather_ws_planned(code, score, tables, plan, bias=None, residual=None, ws_bytes=None):
+    """Exactly the kernel `plan` = (tables_per_buffer, tokens_per_workgroup), with a workspace (fp32 rows);
+    ws_bytes None = room for the record stream of form 3.  Returns (status, output)."""
+    cd, sd, td, bd = dev(code), dev(score), dev(tables), dev(bias)
+    rd = None if residual is None else dev(residual)
+    B, T = code.shape
+    _, S, Do = tables.shape
+    if ws_bytes is None:
+        ws_bytes = 6 * T * (B + 2048)
+    ws = torch.full((max(ws_bytes, 16) // 4,), float("nan"), dtype=torch.float32, device=DEV)
+    out = torch.full((B, Do), float("nan"), dtype=torch.float32, device=DEV)
+    rc = _lib.load().lffn_lookup_gather_ws_planned_f32(p(cd), p(sd), p(td), p(bd), p(rd), p(out), p(ws) if ws_bytes else None,
+                                                       ws_bytes, B, T, S, Do, plan[0], plan[1], None)
+    torch.cuda.synchronize()
+    return rc, host(out)
+
+
 def lookup_gather_plan(B, T, S, Do, bf16=False):
     kind = ctypes.c_int32(-1)
     tokens = _lib.load().lffn_lookup_gather_plan(B, T, S, Do, int(bf16), ctypes.byref(kind))

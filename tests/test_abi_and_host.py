@@ -175,16 +175,17 @@ def test_workspace_queries_are_host_side_plans():
     assert gather_ws(1024, 128, 256, 768) == 8 * 1024 * 768 * 4
     assert gather_ws(4096, 128, 256, 768) == 4 * 4096 * 768 * 4
     # enough tokens to fill the chip without a split, too few tokens or tables for it to pay, bad shapes
-    for shape in ((16384, 512, 256, 1024), (256, 32, 256, 256), (4096, 16, 256, 768),
+    for shape in ((16384, 128, 128, 768), (256, 32, 256, 256), (4096, 16, 256, 768),
                   (2048, 128, 512, 768), (2048, 128, 256, 100), (0, 128, 256, 768)):
         assert gather_ws(*shape) == 0, shape
     assert gather_ws(16384, 128, 256, 768, 1) == 0 and gather_ws(65536, 128, 256, 768, 1) == 0      # bf16 rows
     # many tokens, fp32 rows, 256-row tables, an even number of them: the four-lanes-per-token kernel, which
-    # wants 12 bytes per (token, table pair) for its record stream (whole chunks of 8 tables)
-    assert gather_ws(16384, 128, 256, 768) == 16 * 16384 * 48
-    assert gather_ws(8192, 128, 256, 768) == 16 * 8192 * 48
-    assert gather_ws(32768, 128, 256, 512) == 16 * 32768 * 48
-    assert 0 < gather_ws(65536, 128, 256, 768) < 16 * 65536 * 48                                    # taken in pieces
+    # wants 12 bytes per (token, table pair) for its record stream (whole token tiles: up to 2048 tokens more)
+    assert gather_ws(16384, 128, 256, 768) == 64 * (16384 + 2048) * 12
+    assert gather_ws(8192, 128, 256, 768) == 64 * (8192 + 2048) * 12
+    assert gather_ws(32768, 128, 256, 512) == 64 * (32768 + 2048) * 12
+    assert gather_ws(65536, 128, 256, 768) == 64 * (65536 + 2048) * 12                              # one launch, no pieces
+    assert gather_ws(16384, 512, 256, 1024) == 256 * (16384 + 2048) * 12                            # 537 MB of tables
     # which gather kernel a shape gets is a host-side decision as well: (tables per LDS buffer, tokens per workgroup)
     def plan(B, T, S, Do, bf16=0):
         kind = ctypes.c_int32(-1)

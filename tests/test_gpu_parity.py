@@ -775,16 +775,16 @@ def test_lookup_gather_table_split_matches_oracle(B, T, S, Do, bf16):
 
 
 def test_lookup_gather_workspace_query_is_zero_where_the_plain_form_is_as_fast():
-    for shape in ((16384, 512, 256, 1024), (8, 128, 256, 768), (4096, 16, 256, 768), (0, 4, 16, 64),
+    for shape in ((16384, 32, 256, 768), (8, 128, 256, 768), (4096, 16, 256, 768), (0, 4, 16, 64),
                   (16384, 128, 128, 768), (16384, 127, 256, 768)):
         assert cabi.lookup_gather_workspace_bytes(*shape) == 0, shape
     for shape in ((16384, 128, 256, 768), (65536, 128, 256, 768), (16384, 512, 256, 1024)):
         assert cabi.lookup_gather_workspace_bytes(*shape, bf16=True) == 0, shape
 
 
-# The four-lanes-per-token kernel (form 3), every tile size that is built, reading code and score
-# itself (the planned entry point passes no workspace).  (B, T, 256, Do): token counts that end inside
-# a tile, a wavefront and a quad; table counts that leave a chunk of 8 short (2, 4 and 6 tables).
+# The four-lanes-per-token kernel (form 3), every tile size that is built, forced onto shapes it would not
+# be chosen for.  (B, T, 256, Do): token counts that end inside a tile, a wavefront and a quad; 1 to 17
+# table pairs; one column slice and several.
 QUAD_PLANS = [(3, 1024), (3, 1536), (3, 1792), (3, 2048)]
 QUAD_SHAPES = [(3000, 20, 256, 256), (4133, 6, 256, 384), (1793, 34, 256, 128), (1, 2, 256, 64), (2050, 8, 256, 192)]
 
@@ -795,31 +795,41 @@ def test_lookup_gather_quad_kernels_match_oracle(B, T, S, Do, plan):
     rng = np.random.RandomState(B + T + S + Do + plan[1])
     tables, code, idx, w = _rand_gather(rng, B, T, S, Do)
     bias = (0.001 * rng.randn(Do)).astype(np.float32)
+    res = rng.randn(B, Do).astype(np.float32)
     flat = tables.reshape(T * S, Do)
-    got = cabi.lookup_gather(code, w, tables, bias, plan=plan)
-    assert not np.isnan(got).any()
+    rc, got = cabi.lookup_gather_ws_planned(code, w, tables, plan, bias=bias)
+    assert rc == 0 and not np.isnan(got).any()
     want = oracle.gather_add(idx, flat.astype(np.float64), w.astype(np.float64)) + bias
     assert relmax(got, want) <= 1e-5
     dirty = (code + S * rng.randint(0, 5, size=code.shape)).astype(np.int32)      # bits above log2(S) are ignored
-    assert np.array_equal(cabi.lookup_gather(dirty, w, tables, bias, plan=plan), got)
-    assert relmax(cabi.lookup_gather(code, w, tables, None, plan=plan), want - bias) <= 1e-5
+    assert np.array_equal(cabi.lookup_gather_ws_planned(dirty, w, tables, plan, bias=bias)[1], got)
+    rc, got_r = cabi.lookup_gather_ws_planned(code, w, tables, plan, residual=res)
+    assert rc == 0 and relmax(got_r, want - bias + res) <= 1e-5
 
 
 def test_lookup_gather_quad_refusals():
     from lookupffn_amd import _lib
+    rng = np.random.RandomState(3)
+    tables, code, idx, w = _rand_gather(rng, 300, 20, 256, 64)
+    assert cabi.lookup_gather_ws_planned(code, w, tables, (3, 1280))[0] == _lib.LFFN_ERR_UNSUPPORTED      # 5 passes: not built
+    assert cabi.lookup_gather_ws_planned(code, w, tables, (3, 1000))[0] == _lib.LFFN_ERR_BAD_ARG
+    assert cabi.lookup_gather_ws_planned(code, w, tables, (3, 1024), ws_bytes=0)[0] == _lib.LFFN_ERR_UNSUPPORTED   # no room for the records
+    assert cabi.lookup_gather_ws_planned(code, w, tables, (3, 1024), ws_bytes=6 * 20 * 300)[0] == _lib.LFFN_ERR_UNSUPPORTED
+    assert cabi.lookup_gather_ws_planned(code[:, :19].copy(), w[:, :19].copy(), tables[:19].copy(), (3, 1024))[0] == _lib.LFFN_ERR_UNSUPPORTED   # odd T
+    t128 = np.ascontiguousarray(tables[:, :128])
+    assert cabi.lookup_gather_ws_planned(code % 128, w, t128, (3, 1024))[0] == _lib.LFFN_ERR_UNSUPPORTED          # S != 256
+    # the forms that need no workspace run through this entry point as well
+    rc, got = cabi.lookup_gather_ws_planned(code, w, tables, (1, 256))
+    assert rc == 0 and np.array_equal(got, cabi.lookup_gather(code, w, tables, plan=(1, 256)))
+    # without a workspace argument the planned entry point refuses form 3
     lib = _lib.load()
-    # (code, score, tables, bias, out, B, T, S, Do): refused before any launch, so the pointers are never used
-    assert lib.lffn_lookup_gather_planned_f32(256, 256, 256, None, 256, 3000, 21, 256, 256, 3, 1024, None) == _lib.LFFN_ERR_UNSUPPORTED   # odd T
-    assert lib.lffn_lookup_gather_planned_f32(256, 256, 256, None, 256, 3000, 20, 128, 256, 3, 1024, None) == _lib.LFFN_ERR_UNSUPPORTED   # S != 256
-    assert lib.lffn_lookup_gather_planned_f32(256, 256, 256, None, 256, 3000, 20, 256, 256, 3, 1280, None) == _lib.LFFN_ERR_UNSUPPORTED   # 5 passes: not built
-    assert lib.lffn_lookup_gather_planned_f32(256, 256, 256, None, 256, 3000, 20, 256, 256, 3, 1000, None) == _lib.LFFN_ERR_BAD_ARG
-    assert lib.lffn_lookup_gather_planned_bf16(256, 256, 256, None, 256, 3000, 20, 256, 256, 3, 1024, None) == _lib.LFFN_ERR_UNSUPPORTED  # fp32 only
+    assert lib.lffn_lookup_gather_planned_f32(256, 256, 256, None, 256, 3000, 20, 256, 256, 3, 1024, None) == _lib.LFFN_ERR_UNSUPPORTED
 
 
 # (B, T, S, Do): shapes for which the workspace query asks for the record stream of form 3: config 2,
-# a token count that ends inside a tile and a quad, a table count that leaves the last chunk of 8 short,
-# and enough tokens that the entry point takes them in pieces (one workspace serves every piece)
-QUAD_WS_SHAPES = [(16384, 128, 256, 768), (16001, 32, 256, 768), (20000, 30, 256, 512), (70001, 16, 256, 768)]
+# a token count that ends inside a tile and a quad, an odd number of table pairs, and several rounds of
+# workgroups in one launch
+QUAD_WS_SHAPES = [(16384, 128, 256, 768), (16001, 64, 256, 768), (20000, 30, 256, 512), (70001, 16, 256, 768)]
 
 
 @pytest.mark.parametrize("B,T,S,Do", QUAD_WS_SHAPES)
@@ -830,7 +840,7 @@ def test_lookup_gather_record_stream_form_matches_oracle(B, T, S, Do):
     res = rng.randn(B, Do).astype(np.float32)
     flat = tables.reshape(T * S, Do)
     nbytes = cabi.lookup_gather_workspace_bytes(B, T, S, Do)
-    assert nbytes > 0 and nbytes % 48 == 0 and nbytes < B * Do * 4           # the record stream, not the table split
+    assert nbytes > 0 and nbytes % 12 == 0 and nbytes < B * Do * 4           # the record stream, not the table split
     got = cabi.lookup_gather_ws(code, w, tables, bias, residual=res)
     assert not np.isnan(got).any()
     sub = np.unique(np.concatenate([rng.choice(B, 128, replace=False), np.arange(B - 70, B), np.arange(0, 8)]))
@@ -841,9 +851,11 @@ def test_lookup_gather_record_stream_form_matches_oracle(B, T, S, Do):
     assert relmax(got, plain) <= 2e-6
     # reproducible; a second call may reuse the workspace
     assert np.array_equal(got, cabi.lookup_gather_ws(code, w, tables, bias, residual=res))
-    # without a workspace, or with one that is too small, the entry point is the plain one
+    # without a workspace the entry point is the plain one; one that is too small for the batch is used for
+    # what it can hold (pieces of a large batch) or not at all
     assert np.array_equal(cabi.lookup_gather_ws(code, w, tables, bias, residual=res, ws_bytes=0), plain)
-    assert np.array_equal(cabi.lookup_gather_ws(code, w, tables, bias, residual=res, ws_bytes=nbytes - 48), plain)
+    assert relmax(cabi.lookup_gather_ws(code, w, tables, bias, residual=res, ws_bytes=nbytes - 16), plain) <= 2e-6
+    assert np.array_equal(cabi.lookup_gather_ws(code, w, tables, bias, residual=res, ws_bytes=1024), plain)
     # no bias, no residual
     assert relmax(cabi.lookup_gather_ws(code, w, tables, None)[sub], want) <= 1e-5
 
