@@ -81,7 +81,7 @@ L2_READ_PEAK_GBS = 16 * 128 * 8 * 2.4
 # measured on; the summaries are kept under profiles/.  Reported only while the library still runs
 # that form for the workload (a figure for another kernel would be stale).
 MEASURED_TRAFFIC = {
-    "cfg2": {"bytes": 281335769, "form": "record stream (four lanes per token)"},
+    
 }
 
 
@@ -96,12 +96,18 @@ def gather_form(B, T, S, Do, bf16):
 
     from lookupffn_amd import _lib
     lib = _lib.load()
+    if not bf16:
+        tok, stride, nbytes = ctypes.c_int32(0), ctypes.c_int64(0), ctypes.c_int64(0)
+        _lib.check(lib.lffn_lookup_gather_records_plan(B, T, S, Do, ctypes.byref(tok), ctypes.byref(stride), ctypes.byref(nbytes)),
+                   "records plan")
+        if nbytes.value > 0:
+            return f"record stream (four lanes per token), {tok.value} tokens per workgroup"
     ws = ctypes.c_int64(0)
     _lib.check(lib.lffn_lookup_gather_workspace_bytes(B, T, S, Do, int(bf16), ctypes.byref(ws)), "workspace query")
     kind = ctypes.c_int32(-1)
     tokens = lib.lffn_lookup_gather_plan(B, T, S, Do, int(bf16), ctypes.byref(kind))
     if ws.value > 0:
-        return "record stream (four lanes per token)" if ws.value < B * Do * 4 else "table split"
+        return "table split"
     return "token-major" if kind.value == 0 else f"{kind.value} table(s) per LDS buffer, {tokens} tokens per workgroup"
 
 
@@ -401,8 +407,8 @@ def main_encoder(args):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--graph", action="store_true",
@@ -449,6 +455,11 @@ def main():
         type(layer).FUSED_LAYER_MAX_TOKENS = 0
     with torch.no_grad():
         fused_layer = layer.can_fuse_layer(x)      # few tokens: the layer is one launch, gather included
+    # many tokens, diagonal BH4, fp32 tables: the projection kernel writes the gather's record stream itself
+    st = layer._inference_state()
+    rec_plan = None
+    if not fused_layer and not block and not wl["bf16"] and T % 2 == 0 and st is not None and st["form"] == "diag":
+        rec_plan = ops.lookup_gather_records_plan(B, T, S, Do)
 
     def step(events=None):
         # exactly what LookupFFN.forward runs in eval mode (checked below), with an
@@ -458,6 +469,15 @@ def main():
                 if events is not None:
                     events[0].record()
                 out = layer._forward(x)
+                if events is not None:
+                    events[1].record()
+                return out
+            if rec_plan is not None:
+                records = ops.ln_project_hash_records_direct(x, st["ln_w"], st["ln_b"], st["eps"], st["diag"], st["pbias"],
+                                                             T, st["decay"], st["res_coef"], rec_plan)
+                if events is not None:
+                    events[0].record()
+                out = ops.lookup_gather_records_direct(records, rec_plan, st["tables"], st["obias"], None, B)
                 if events is not None:
                     events[1].record()
                 return out
@@ -544,8 +564,13 @@ def main():
             fn()
         b.record(); torch.cuda.synchronize()
         return a.elapsed_time(b) / n
+    def front():
+        if rec_plan is not None:
+            return ops.ln_project_hash_records_direct(x, st["ln_w"], st["ln_b"], st["eps"], st["diag"], st["pbias"],
+                                                      T, st["decay"], st["res_coef"], rec_plan)
+        return hash_front()
     with torch.no_grad():
-        hash_ms = None if fused_layer else timed(hash_front)
+        hash_ms = None if fused_layer else timed(front)
 
     # Warm and cold medians of single launches (outside the timed region).  Warm: back to
     # back, the tables still in the caches from the launch before.  Cold: a 1 GiB fill
@@ -564,8 +589,12 @@ def main():
         if fused_layer:
             gather_only = step
         else:
-            code, score = hash_front()
-            gather_only = lambda: ops.lookup_gather(code, score, layer.tables, layer.bias)
+            if rec_plan is not None:
+                records = front()
+                gather_only = lambda: ops.lookup_gather_records_direct(records, rec_plan, st["tables"], st["obias"], None, B)
+            else:
+                code, score = hash_front()
+                gather_only = lambda: ops.lookup_gather(code, score, layer.tables, layer.bias)
         warm_gather, warm_step = single(gather_only, 25), single(step, 25)
         flush = torch.zeros(1 << 28, dtype=torch.float32, device=dev)
         cold_gather, cold_step = single(gather_only, 15, flush), single(step, 15, flush)
@@ -590,6 +619,8 @@ def main():
                    "step": ("one kernel: LayerNorm + BH4(block 64)x4 on fp32 MFMA + mix + hash (weights folded once, "
                             "outside the step); one kernel: gather-add + bias") if block else
                            ("one kernel: LayerNorm + BH4(block 1)x4 + mix + hash + gather-add + bias" if fused_layer else
+                            ("one kernel: LayerNorm + BH4(block 1)x4 + mix + hash, written as the gather's record stream; "
+                             "one kernel: gather-add + bias") if rec_plan is not None else
                             "one kernel: LayerNorm + BH4(block 1)x4 + mix + hash; one kernel: gather-add + bias")},
         "roofline": roofline,
         "stages_ms": ({"whole_layer": gather_ms} if fused_layer else

@@ -313,6 +313,44 @@ int lffn_ln_project_hash_f32(const float *x, const float *ln_weight, const float
                              int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
                              float decay, float residual, void *stream);
 
+/*
+ * The layer's inference path at many tokens without the [B, T] codes and scores in between: the
+ * projection kernel writes the record stream that the four-lanes-per-token gather reads (the form
+ * lffn_lookup_gather_ws_f32 packs for itself), and the gather runs from it.  Three calls:
+ *
+ * lffn_lookup_gather_records_plan: host-side query.  When this form is the one to use for a shape
+ * (fp32 rows, S = 256, an even number of tables, enough tokens: the conditions under which
+ * lffn_lookup_gather_workspace_bytes asks for a record stream) it sets *tokens_per_workgroup (1024,
+ * 1536, 1792 or 2048), *record_stride (B rounded up to whole workgroup tiles) and *bytes (the size of
+ * the stream: 6 * T * record_stride); otherwise all three are 0 and the caller uses the other entry
+ * points.
+ *
+ * lffn_ln_project_hash_records_f32: lffn_ln_project_hash_f32 (ln_weight and ln_bias both NULL: no
+ * LayerNorm, as lffn_project_hash_f32) with its codes and scores written as records: 4-byte aligned
+ * device memory of `bytes`, three planes of record_stride words per table pair k:
+ *   word 0: score of the pair's first table, word 1: score of its second, word 2: row of the first |
+ *   row of the second << 8, where token b takes the tables in the order (2k, 2k+1) when bit 1 of b is
+ *   clear and (2k+1, 2k) when it is set (the order its lanes read them in the gather kernel).
+ * Words of tokens from B up to record_stride are left as they are: the gather ignores them.  T even,
+ * D >= 16.  The layout is private to these entry points: write it with this call only.
+ *
+ * lffn_lookup_gather_records_f32: out[b,:] = residual[b,:] + bias + sum_t score[b,t] * tables[t, code[b,t], :]
+ * from such a stream, with the tokens_per_workgroup and record_stride the plan gave.  Results are
+ * bit-identical to lffn_lookup_gather_ws_f32's for the same shape.  bias and residual may be NULL.
+ *
+ * Replaces the same reference code as lffn_ln_project_hash_f32 followed by lffn_lookup_gather_f32
+ * (PL/lookup.py:29-39,64-77,99 and 120-130,108).
+ */
+int lffn_lookup_gather_records_plan(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t *tokens_per_workgroup,
+                                    int64_t *record_stride, int64_t *bytes);
+int lffn_ln_project_hash_records_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
+                                     const float *diag, const float *proj_bias, uint32_t *records,
+                                     int64_t record_stride, int64_t B, int64_t H, int64_t D, int64_t R,
+                                     int64_t J, int64_t T, float decay, float residual, void *stream);
+int lffn_lookup_gather_records_f32(const uint32_t *records, int64_t record_stride, const float *tables,
+                                   const float *bias, const float *residual, float *out, int64_t B, int64_t T,
+                                   int64_t S, int64_t Do, int32_t tokens_per_workgroup, void *stream);
+
 /* ---------------------------------------------------------------- code + score */
 
 /*

@@ -143,6 +143,13 @@ struct ProjectArgs {
     float *out;           // [B, out_stride] or null
     int32_t *codes;       // [B, T] (HASH only)
     float *scores;        // [B, T] (HASH only)
+    // HASH only, instead of codes and scores: the record stream of the four-lanes-per-token gather
+    // (lookup_gather_quad.hip), three planes of rec_stride words per table pair: score of the pair's first
+    // table, score of its second, row of the first | row of the second << 8, where a token whose index has
+    // bit 1 set takes the pair's tables in the order (2k+1, 2k).  T even, 8-bit codes.
+    uint32_t *records;    // [T/2][3][rec_stride] or null
+    int64_t rec_stride;   // >= B
+    int blocks_per_xcd;   // records: workgroup b takes rows from the range of XCD b % 8 (see project_kernel)
     int64_t B;
     int H;                // valid input columns (<= D)
     int R, J;
@@ -251,7 +258,13 @@ __global__ __launch_bounds__(256) void project_kernel(ProjectArgs a) {
     const int lr = lane % LPR;
     // GATHER: one token per workgroup; its four wavefronts each compute the token's codes (no
     // hand-over needed) and then share the gather, a quarter of the tables each
-    const int64_t row = GATHER ? int64_t(blockIdx.x) : (int64_t(blockIdx.x) * 4 + wave) * RPW + lane / LPR;
+    // Records are written a word at a time into planes indexed by token: a 128-byte line holds 32
+    // consecutive tokens' words, and consecutive workgroups run on different XCDs, whose L2s would each
+    // write back a sliver of every line.  So with records every XCD takes a contiguous range of rows
+    // (workgroup b runs on XCD b % 8 and is that XCD's workgroup number b / 8).
+    const int64_t blk = (HASH && !GATHER && a.records)
+                            ? int64_t(blockIdx.x % 8) * a.blocks_per_xcd + blockIdx.x / 8 : int64_t(blockIdx.x);
+    const int64_t row = GATHER ? int64_t(blockIdx.x) : (blk * 4 + wave) * RPW + lane / LPR;
     const bool live = row < a.B;
 
     float orig[NJ][4];
@@ -405,6 +418,22 @@ __global__ __launch_bounds__(256) void project_kernel(ProjectArgs a) {
                             }
                         }
                     }
+                } else if (a.records) {
+                    // Tables t - 1 (even) and t sit in lanes 4m + 1 and 4m + 3: the latter fetches the
+                    // former's code and score (quad_perm [1,1,1,1]) and writes the pair's record.
+                    const int code_here = (nib_hi << 4) | nib;
+                    const float score_here = s_run / p_run;
+                    const int code_even = __builtin_amdgcn_update_dpp(0, code_here, 0x55, 0xF, 0xF, true);
+                    const float score_even = __int_as_float(
+                        __builtin_amdgcn_update_dpp(0, __float_as_int(score_here), 0x55, 0xF, 0xF, true));
+                    if (live && (lr & 3) == 3 && t < a.T) {
+                        const bool second_first = (row & 2) != 0;
+                        uint32_t *dst = a.records + (size_t)(t >> 1) * 3 * a.rec_stride + row;
+                        dst[0] = __float_as_uint(second_first ? score_here : score_even);
+                        dst[a.rec_stride] = __float_as_uint(second_first ? score_even : score_here);
+                        dst[2 * a.rec_stride] = second_first ? (unsigned)(code_here | (code_even << 8))
+                                                             : (unsigned)(code_even | (code_here << 8));
+                    }
                 } else if (live && (lr & 1) && t < a.T) {
                     a.codes[row * a.T + t] = (nib_hi << 4) | nib;
                     a.scores[row * a.T + t] = s_run / p_run;
@@ -420,8 +449,13 @@ int launch_project(const ProjectArgs &a, int logd, hipStream_t stream) {
     auto go = [&](auto tag) {
         constexpr int L = decltype(tag)::value;
         const int64_t rows_per_block = 4 * FhtCfg<L>::RPW;
-        const int64_t blocks = (a.B + rows_per_block - 1) / rows_per_block;
-        hipLaunchKernelGGL((project_kernel<L, HASH>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+        int64_t blocks = (a.B + rows_per_block - 1) / rows_per_block;
+        ProjectArgs b = a;
+        if (HASH && a.records) {        // whole rounds of eight workgroups, one per XCD
+            b.blocks_per_xcd = (int)((blocks + 7) / 8);
+            blocks = int64_t(b.blocks_per_xcd) * 8;
+        }
+        hipLaunchKernelGGL((project_kernel<L, HASH>), dim3((unsigned)blocks), dim3(256), 0, stream, b);
     };
     switch (logd) {
         case 2: if constexpr (!HASH) { go(std::integral_constant<int, 2>{}); break; } else return LFFN_ERR_UNSUPPORTED;
@@ -773,7 +807,8 @@ static int project_hash_impl(const float *x, const float *ln_w, const float *ln_
                              const float *diag, const float *proj_bias,
                              float *z_out, int32_t *codes, float *scores,
                              int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
-                             float decay, float residual, void *stream);
+                             float decay, float residual, void *stream, uint32_t *records = nullptr,
+                             int64_t record_stride = 0);
 
 extern "C" int lffn_ln_project_hash_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
                                         const float *diag, const float *proj_bias,
@@ -783,6 +818,17 @@ extern "C" int lffn_ln_project_hash_f32(const float *x, const float *ln_weight, 
     LFFN_REQUIRE(ln_weight && ln_bias && ln_eps >= 0.f, LFFN_ERR_BAD_ARG);
     return project_hash_impl(x, ln_weight, ln_bias, ln_eps, diag, proj_bias, z_out, codes, scores,
                              B, H, D, R, J, T, decay, residual, stream);
+}
+
+extern "C" int lffn_ln_project_hash_records_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
+                                                const float *diag, const float *proj_bias, uint32_t *records,
+                                                int64_t record_stride, int64_t B, int64_t H, int64_t D, int64_t R,
+                                                int64_t J, int64_t T, float decay, float residual, void *stream) {
+    LFFN_REQUIRE(ln_eps >= 0.f && ((ln_weight && ln_bias) || (!ln_weight && !ln_bias)), LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(records && record_stride >= B && T % 2 == 0, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(D >= 16, LFFN_ERR_UNSUPPORTED);           // a table pair's 16 values within an aligned lane quad
+    return project_hash_impl(x, ln_weight, ln_bias, ln_eps, diag, proj_bias, nullptr, nullptr, nullptr,
+                             B, H, D, R, J, T, decay, residual, stream, records, record_stride);
 }
 
 extern "C" int lffn_project_hash_f32(const float *x, const float *diag, const float *proj_bias,
@@ -797,8 +843,8 @@ static int project_hash_impl(const float *x, const float *ln_w, const float *ln_
                              const float *diag, const float *proj_bias,
                              float *z_out, int32_t *codes, float *scores,
                              int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
-                             float decay, float residual, void *stream) {
-    LFFN_REQUIRE(x && diag && codes && scores, LFFN_ERR_BAD_ARG);
+                             float decay, float residual, void *stream, uint32_t *records, int64_t record_stride) {
+    LFFN_REQUIRE(x && diag && ((codes && scores) || records), LFFN_ERR_BAD_ARG);
     int rc = check_dims(B, H, D, R, J);
     if (rc != LFFN_OK) return rc;
     LFFN_REQUIRE(D >= 8, LFFN_ERR_UNSUPPORTED);
@@ -808,6 +854,7 @@ static int project_hash_impl(const float *x, const float *ln_w, const float *ln_
                  LFFN_ERR_BAD_ARG);
     ProjectArgs a{};
     a.x = x; a.diag = diag; a.pbias = proj_bias; a.out = z_out; a.codes = codes; a.scores = scores;
+    a.records = records; a.rec_stride = record_stride;
     a.ln_w = ln_w; a.ln_b = ln_b; a.ln_eps = ln_eps;
     a.B = B; a.H = (int)H; a.R = (int)R; a.J = (int)J;
     a.out_stride = (int)(T * 8); a.out_cols = (int)(T * 8); a.T = (int)T;

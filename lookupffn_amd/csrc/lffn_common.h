@@ -85,6 +85,12 @@ int lffn_internal_lookup_gather_quad(const int32_t *code, const float *score, co
                                      int64_t S, int64_t Do, int np, void *workspace, void *stream);
 __attribute__((visibility("hidden")))
 int64_t lffn_internal_quad_stream_bytes(int64_t B, int64_t T);
+__attribute__((visibility("hidden")))
+int64_t lffn_internal_quad_record_stride(int64_t B, int np);
+__attribute__((visibility("hidden")))
+int lffn_internal_lookup_gather_quad_records(const uint32_t *records, int64_t record_stride, const void *tables,
+                                             const float *bias, const float *residual, float *out, int64_t B,
+                                             int64_t T, int64_t S, int64_t Do, int np, void *stream);
 
 static inline int lffn_launch_status() {
     return hipGetLastError() == hipSuccess ? LFFN_OK : LFFN_ERR_LAUNCH;

@@ -740,3 +740,32 @@ extern "C" int lffn_lookup_gather_plan(int64_t B, int64_t T, int64_t S, int64_t 
     if (tables_per_buffer) *tables_per_buffer = plan.kind;
     return plan.kind == 0 ? 0 : (plan.kind == 1 ? 64 : (plan.kind == 3 ? 256 : 128)) * plan.np;
 }
+
+// ---------------------------------------------------------------- gather from a record stream
+
+extern "C" int lffn_lookup_gather_records_plan(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t *tokens_per_workgroup,
+                                               int64_t *record_stride, int64_t *bytes) {
+    LFFN_REQUIRE(tokens_per_workgroup && record_stride && bytes, LFFN_ERR_BAD_ARG);
+    *tokens_per_workgroup = 0; *record_stride = 0; *bytes = 0;
+    if (B < 1 || T < 1 || Do < 1 || !lffn_is_pow2(S) || Do % 64 != 0 || B * T >= (int64_t(1) << 31)) return LFFN_OK;
+    const GatherPlan qp = choose_quad<false>(B, T, S, Do);
+    if (qp.kind != 3) return LFFN_OK;
+    *tokens_per_workgroup = 256 * qp.np;
+    *record_stride = lffn_internal_quad_record_stride(B, qp.np);
+    *bytes = (T / 2) * 3 * *record_stride * 4;
+    return LFFN_OK;
+}
+
+extern "C" int lffn_lookup_gather_records_f32(const uint32_t *records, int64_t record_stride, const float *tables,
+                                              const float *bias, const float *residual, float *out, int64_t B, int64_t T,
+                                              int64_t S, int64_t Do, int32_t tokens_per_workgroup, void *stream) {
+    LFFN_REQUIRE(B >= 0 && T >= 0 && Do >= 1 && tokens_per_workgroup > 0, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(tokens_per_workgroup % 256 == 0, LFFN_ERR_BAD_ARG);
+    const GatherPlan plan{3, tokens_per_workgroup / 256, 0.0};
+    LFFN_REQUIRE(lffn_is_pow2(S) && Do % 64 == 0 && plan_is_valid<false>(plan, B, T, S, Do), LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(tables && out && (records || B == 0), LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_aligned16(tables) && lffn_aligned16(out) && (!bias || lffn_aligned16(bias)) &&
+                     (!residual || lffn_aligned16(residual)) && (uintptr_t)records % 4 == 0, LFFN_ERR_BAD_ARG);
+    if (B == 0) return LFFN_OK;
+    return lffn_internal_lookup_gather_quad_records(records, record_stride, tables, bias, residual, out, B, T, S, Do, plan.np, stream);
+}

@@ -392,11 +392,6 @@ int launch_quad(QuadArgs a, hipStream_t stream) {
     return lffn_launch_status();
 }
 
-template <int NP>
-int launch_quad_touch(const QuadArgs &a, bool touch, hipStream_t st) {
-    return touch ? launch_quad<NP, true>(a, st) : launch_quad<NP, false>(a, st);
-}
-
 }  // namespace
 
 // Bytes of the record stream for a shape: T/2 table pairs x the tokens rounded up to whole tiles
@@ -405,35 +400,52 @@ int64_t lffn_internal_quad_stream_bytes(int64_t B, int64_t T) {
     return (T / 2) * (B + 2048) * (int64_t)(REC_WORDS * 4);
 }
 
-// Pack the (code, score) pairs into the record stream in `workspace` (at least
-// lffn_internal_quad_stream_bytes(B, T) bytes, 16-byte aligned) and run the gather from it with 256*np
-// tokens per workgroup.  The caller has checked that the shape qualifies: fp32 rows, S = 256 (a table
-// pair fills an LDS buffer), T even, Do a multiple of 32, B*T < 2^31, 2*S*Do*4 < 2^32 (32-bit lane
-// offsets from a table pair's base), np one of {4, 6, 7, 8}.
-int lffn_internal_lookup_gather_quad(const int32_t *code, const float *score, const void *tables,
-                                     const float *bias, const float *residual, float *out, int64_t B, int64_t T,
-                                     int64_t S, int64_t Do, int np, void *workspace, void *stream) {
-    if (!workspace || S != MAX_S || T % 2 != 0 || !(np == 4 || np == 6 || np == 7 || np == 8)) return LFFN_ERR_BAD_ARG;
+// Run the gather from a record stream [T/2][3][record_stride] (pack_pairs_kernel's layout; the projection
+// kernel of fht.hip writes the same) with 256*np tokens per workgroup.  The caller has checked that the
+// shape qualifies: fp32 rows, S = 256 (a table pair fills an LDS buffer), T even, Do a multiple of 32,
+// 2*S*Do*4 < 2^32 (32-bit lane offsets from a table pair's base), np one of {4, 6, 7, 8}.  record_stride:
+// whole tiles of 256*np tokens, at least B; what the records of tokens from B on hold does not matter
+// (their row numbers are bytes, always inside the LDS buffer, and their sums are not stored).
+int lffn_internal_lookup_gather_quad_records(const uint32_t *records, int64_t record_stride, const void *tables,
+                                             const float *bias, const float *residual, float *out, int64_t B,
+                                             int64_t T, int64_t S, int64_t Do, int np, void *stream) {
+    if (!records || S != MAX_S || T % 2 != 0 || !(np == 4 || np == 6 || np == 7 || np == 8)) return LFFN_ERR_BAD_ARG;
+    const int64_t tile_tokens = 256 * int64_t(np);
+    if (record_stride % tile_tokens != 0 || record_stride < B) return LFFN_ERR_BAD_ARG;
     QuadArgs a{};
     a.tables = static_cast<const char *>(tables); a.bias = bias; a.residual = residual; a.out = out;
     a.B = B; a.T = (int)T; a.S = (int)S; a.Do = (int)Do;
     a.nslices = (int)(Do / SLICE_COLS);
     a.row_bytes = (int)(Do * 4);
+    a.Bpad = record_stride;
+    a.stream = records;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    uint32_t *recs = static_cast<uint32_t *>(workspace);
-    const int64_t tile_tokens = 256 * int64_t(np);
-    a.Bpad = (B + tile_tokens - 1) / tile_tokens * tile_tokens;
-    a.stream = recs;
-    const dim3 grid((unsigned)((a.Bpad + 63) / 64), (unsigned)((T / 2 + 31) / 32));
-    hipLaunchKernelGGL(pack_pairs_kernel, grid, dim3(256), 0, st, code, score, recs, B, a.Bpad, (int)T, (int)S);
-    if (hipGetLastError() != hipSuccess) return LFFN_ERR_LAUNCH;
     // the touch by turns, always: tables beyond the 256 MB memory-side cache need it most (984 -> 736 us
     // at 512 tables x 256 x 1024 and 1024 tokens per workgroup)
-    const bool touch = true;
     switch (np) {
-        case 8: return launch_quad_touch<8>(a, touch, st);
-        case 7: return launch_quad_touch<7>(a, touch, st);
-        case 6: return launch_quad_touch<6>(a, touch, st);
-        default: return launch_quad_touch<4>(a, touch, st);
+        case 8: return launch_quad<8, true>(a, st);
+        case 7: return launch_quad<7, true>(a, st);
+        case 6: return launch_quad<6, true>(a, st);
+        default: return launch_quad<4, true>(a, st);
     }
+}
+
+int64_t lffn_internal_quad_record_stride(int64_t B, int np) {
+    const int64_t tile_tokens = 256 * int64_t(np);
+    return (B + tile_tokens - 1) / tile_tokens * tile_tokens;
+}
+
+// Pack the (code, score) pairs into the record stream in `workspace` (at least
+// lffn_internal_quad_stream_bytes(B, T) bytes, 16-byte aligned) and run the gather from it.
+int lffn_internal_lookup_gather_quad(const int32_t *code, const float *score, const void *tables,
+                                     const float *bias, const float *residual, float *out, int64_t B, int64_t T,
+                                     int64_t S, int64_t Do, int np, void *workspace, void *stream) {
+    if (!workspace || S != MAX_S || T % 2 != 0 || !(np == 4 || np == 6 || np == 7 || np == 8)) return LFFN_ERR_BAD_ARG;
+    uint32_t *recs = static_cast<uint32_t *>(workspace);
+    const int64_t stride = lffn_internal_quad_record_stride(B, np);
+    const dim3 grid((unsigned)((stride + 63) / 64), (unsigned)((T / 2 + 31) / 32));
+    hipLaunchKernelGGL(pack_pairs_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), code, score, recs, B,
+                       stride, (int)T, (int)S);
+    if (hipGetLastError() != hipSuccess) return LFFN_ERR_LAUNCH;
+    return lffn_internal_lookup_gather_quad_records(recs, stride, tables, bias, residual, out, B, T, S, Do, np, stream);
 }

@@ -719,6 +719,61 @@ def _(indexes, source, weights):
     return weights.new_empty(indexes.shape[0], source.shape[1])
 
 
+# The inference path of the layer at many tokens: the projection kernel writes the gather kernel's record
+# stream itself (no [B, T] codes and scores, no packing kernel).  Plain functions, no operator: the
+# records are a private hand-over between the two kernels.
+_RECORDS_PLANS = {}
+
+
+def lookup_gather_records_plan(B, T, S, Do):
+    """(tokens per workgroup, record stride in tokens, bytes of the stream) when the record-stream form of
+    the gather is the one to use for this shape (fp32 rows), else None.  Host-side query, cached."""
+    key = (B, T, S, Do)
+    hit = _RECORDS_PLANS.get(key, False)
+    if hit is not False:
+        return hit
+    tokens, stride, nbytes = ctypes.c_int32(0), ctypes.c_int64(0), ctypes.c_int64(0)
+    _lib.check(_lib.load().lffn_lookup_gather_records_plan(B, T, S, Do, ctypes.byref(tokens), ctypes.byref(stride),
+                                                           ctypes.byref(nbytes)), "lffn_lookup_gather_records_plan")
+    plan = (tokens.value, stride.value, nbytes.value) if nbytes.value > 0 else None
+    if len(_RECORDS_PLANS) < 4096:
+        _RECORDS_PLANS[key] = plan
+    return plan
+
+
+def ln_project_hash_records_direct(x, ln_w, ln_b, eps, diag, pbias, T, decay, residual, plan):
+    """LayerNorm + diagonal BH4 + mix + 8-bit hash of x [B, H], written as the record stream of `plan`
+    (from lookup_gather_records_plan) instead of codes and scores.  The caller has checked the parameters
+    (fp32, contiguous, on x's device)."""
+    assert x.dtype == torch.float32 and x.is_cuda and x.is_contiguous() and x.dim() == 2
+    B, H = x.shape
+    R, J, D = diag.shape
+    assert H == ln_w.numel() and T * 8 <= R * D and T % 2 == 0 and plan[1] >= B
+    records = torch.empty(plan[2] // 4, dtype=torch.int32, device=x.device)
+    with _dev_guard(x):
+        rc = _lib.load().lffn_ln_project_hash_records_f32(
+            x.data_ptr(), ln_w.data_ptr(), ln_b.data_ptr(), eps, diag.data_ptr(), None if pbias is None else pbias.data_ptr(),
+            records.data_ptr(), plan[1], B, H, D, R, J, T, decay, residual, _lib.stream_of(x))
+    if rc != 0:
+        _lib.check(rc, f"lffn_ln_project_hash_records_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T})")
+    return records
+
+
+def lookup_gather_records_direct(records, plan, tables, bias, residual, B):
+    """out[b] = residual[b] + bias + sum_t score * row, from the record stream written for `plan`."""
+    T, S, Do = tables.shape
+    assert tables.dtype == torch.float32 and tables.is_contiguous() and records.numel() * 4 >= plan[2]
+    assert residual is None or (residual.dtype == torch.float32 and residual.is_contiguous() and tuple(residual.shape) == (B, Do))
+    out = torch.empty(B, Do, dtype=torch.float32, device=tables.device)
+    with _dev_guard(tables):
+        rc = _lib.load().lffn_lookup_gather_records_f32(
+            records.data_ptr(), plan[1], tables.data_ptr(), None if bias is None else bias.data_ptr(),
+            None if residual is None else residual.data_ptr(), out.data_ptr(), B, T, S, Do, plan[0], _lib.stream_of(tables))
+    if rc != 0:
+        _lib.check(rc, f"lffn_lookup_gather_records_f32(B={B}, T={T}, S={S}, Do={Do})")
+    return out
+
+
 _L.define("lookup_gather(Tensor code, Tensor score, Tensor tables, Tensor? bias, Tensor? residual=None) -> Tensor")
 
 

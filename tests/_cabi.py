@@ -288,6 +288,30 @@ def lookup_gather_ws_planned(code, score, tables, plan, bias=None, residual=None
     return rc, host(out)
 
 
+def lookup_gather_records_plan(B, T, S, Do):
+    tokens, stride, nbytes = ctypes.c_int32(-1), ctypes.c_int64(-1), ctypes.c_int64(-1)
+    assert _lib.load().lffn_lookup_gather_records_plan(B, T, S, Do, ctypes.byref(tokens), ctypes.byref(stride),
+                                                       ctypes.byref(nbytes)) == 0
+    return tokens.value, stride.value, nbytes.value
+
+
+def layer_through_records(x, ln_w, ln_b, eps, diag, pbias, tables, obias, residual=None, decay=0.7, plan=None):
+    """lffn_ln_project_hash_records_f32 followed by lffn_lookup_gather_records_f32; returns (output, records)."""
+    B, H = x.shape
+    R, J, D = diag.shape
+    T, S, Do = tables.shape
+    tokens, stride, nbytes = plan if plan is not None else lookup_gather_records_plan(B, T, S, Do)
+    assert nbytes > 0
+    xd, wd, bd, dd, pd, td, od = dev(x), dev(ln_w), dev(ln_b), dev(diag), dev(pbias), dev(tables), dev(obias)
+    rd = None if residual is None else dev(residual)
+    rec = torch.full((nbytes // 4,), -1, dtype=torch.int32, device=DEV)
+    out = torch.full((B, Do), float("nan"), dtype=torch.float32, device=DEV)
+    _call("lffn_ln_project_hash_records_f32", p(xd), p(wd), p(bd), eps, p(dd), p(pd), p(rec), stride, B, H, D, R, J, T,
+          decay, 1.0 - decay)
+    _call("lffn_lookup_gather_records_f32", p(rec), stride, p(td), p(od), p(rd), p(out), B, T, S, Do, tokens)
+    return host(out), rec.cpu().numpy().view(np.uint32)
+
+
 def lookup_gather_plan(B, T, S, Do, bf16=False):
     kind = ctypes.c_int32(-1)
     tokens = _lib.load().lffn_lookup_gather_plan(B, T, S, Do, int(bf16), ctypes.byref(kind))

@@ -477,6 +477,75 @@ def test_ln_project_hash_matches_oracle(H, D, R, T):
     assert np.abs(z - z2).max() <= 1e-5 * scale
 
 
+# (B, H, D, R, T, Do, forced plan or None): config 2's layer shape; a token count that ends inside a tile, a
+# workgroup of the projection kernel and a quad; two repeats of a short transform (rows shared by four
+# tokens per wavefront); an odd number of table pairs
+RECORD_LAYERS = [(16384, 768, 1024, 1, 128, 768, None), (4099, 768, 1024, 1, 128, 768, (1024, 5120)),
+                 (5000, 100, 128, 2, 30, 128, (1536, 6144)), (2050, 64, 64, 1, 6, 64, (2048, 4096))]
+
+
+@pytest.mark.parametrize("B,H,D,R,T,Do,plan", RECORD_LAYERS)
+def test_layer_through_the_record_stream_matches_the_two_kernel_form(B, H, D, R, T, Do, plan):
+    """lffn_ln_project_hash_records_f32 + lffn_lookup_gather_records_f32: the records hold exactly the codes
+    and scores lffn_ln_project_hash_f32 writes, in the layout the gather kernel reads, and the output is
+    that of the gather on those codes and scores (bit for bit against the workspace entry point where both
+    run the same tile size; against the float64 sum on a sample)."""
+    rng = np.random.RandomState(B + H + T)
+    S, J = 256, 4
+    x = (rng.randn(B, H) * 1.5 + 0.3).astype(np.float32)
+    ln_w = (1 + 0.1 * rng.randn(H)).astype(np.float32)
+    ln_b = (0.1 * rng.randn(H)).astype(np.float32)
+    diag = ((2 * rng.randint(0, 2, size=(R, J, D)) - 1) / math.sqrt(D)).astype(np.float32)
+    pbias = (0.05 * rng.randn(T * 8)).astype(np.float32)
+    tables = (0.02 * rng.randn(T, S, Do)).astype(np.float32)
+    obias = (0.001 * rng.randn(Do)).astype(np.float32)
+    res = rng.randn(B, Do).astype(np.float32)
+    if plan is None:
+        plan = cabi.lookup_gather_records_plan(B, T, S, Do)[:2]
+        assert plan == (1792, 17920)                                            # config 2: 10 tiles x 24 slices
+    tokens, stride = plan
+    full_plan = (tokens, stride, 6 * T * stride)
+    got, rec = cabi.layer_through_records(x, ln_w, ln_b, 1e-5, diag, pbias, tables, obias, residual=res, plan=full_plan)
+    assert not np.isnan(got).any()
+    codes, scores, _ = cabi.ln_project_hash(x, ln_w, ln_b, 1e-5, diag, pbias, T)
+    # the records, word for word
+    rec = rec.reshape(T // 2, 3, stride)[:, :, :B]
+    swap = ((np.arange(B) & 2) != 0)[None, :]
+    c0, c1 = codes[:, 0::2].T, codes[:, 1::2].T                                  # [T/2, B]
+    s0, s1 = scores[:, 0::2].T, scores[:, 1::2].T
+    assert np.array_equal(rec[:, 0].view(np.float32), np.where(swap, s1, s0))
+    assert np.array_equal(rec[:, 1].view(np.float32), np.where(swap, s0, s1))
+    assert np.array_equal(rec[:, 2], np.where(swap, c1 | (c0 << 8), c0 | (c1 << 8)).astype(np.uint32))
+    # the output: the same kernel at the same tile size through the workspace entry point, bit for bit
+    rc, want_same = cabi.lookup_gather_ws_planned(codes, scores, tables, (3, tokens), bias=obias, residual=res)
+    assert rc == 0 and np.array_equal(got, want_same)
+    # and the float64 sum over the kernel's own codes and scores, on a sample
+    sub = np.unique(np.concatenate([rng.choice(B, 96, replace=False), np.arange(B - 40, B), np.arange(0, 8)]))
+    idx = codes[sub] + (np.arange(T, dtype=np.int32) * S)[None]
+    want = oracle.gather_add(idx, tables.reshape(T * S, Do).astype(np.float64), scores[sub].astype(np.float64))
+    assert relmax(got[sub], want + obias + res[sub]) <= 1e-5
+
+
+def test_record_stream_plan_and_refusals():
+    from lookupffn_amd import _lib
+    lib = _lib.load()
+    assert cabi.lookup_gather_records_plan(16384, 128, 256, 768) == (1792, 17920, 6 * 128 * 17920)
+    assert cabi.lookup_gather_records_plan(16384, 512, 256, 1024) == (2048, 16384, 6 * 512 * 16384)
+    for shape in ((256, 32, 256, 256), (16384, 128, 128, 768), (16384, 127, 256, 768), (0, 128, 256, 768)):
+        assert cabi.lookup_gather_records_plan(*shape) == (0, 0, 0), shape
+    # (records, stride, tables, bias, residual, out, B, T, S, Do, tokens): refused before any launch
+    bad = lambda *a: lib.lffn_lookup_gather_records_f32(256, *a, None)
+    assert bad(4096, 256, None, None, 256, 3000, 20, 256, 256, 1000) == _lib.LFFN_ERR_BAD_ARG            # not whole passes
+    assert bad(4096, 256, None, None, 256, 3000, 20, 256, 256, 1280) == _lib.LFFN_ERR_UNSUPPORTED        # 5 passes: not built
+    assert bad(4096, 256, None, None, 256, 3000, 21, 256, 256, 1024) == _lib.LFFN_ERR_UNSUPPORTED        # odd T
+    assert bad(4000, 256, None, None, 256, 3000, 20, 256, 256, 1024) == _lib.LFFN_ERR_BAD_ARG            # stride not whole tiles
+    assert bad(2048, 256, None, None, 256, 3000, 20, 256, 256, 1024) == _lib.LFFN_ERR_BAD_ARG            # stride < B
+    assert lib.lffn_ln_project_hash_records_f32(256, 256, 256, 1e-5, 256, None, 256, 100, 300, 64, 64, 1, 4, 6, 0.7, 0.3, None) \
+        == _lib.LFFN_ERR_BAD_ARG                                                                         # stride < B
+    assert lib.lffn_ln_project_hash_records_f32(256, 256, 256, 1e-5, 256, None, 256, 1024, 300, 64, 64, 1, 4, 5, 0.7, 0.3, None) \
+        == _lib.LFFN_ERR_BAD_ARG                                                                         # odd T
+
+
 @pytest.mark.parametrize("P,na,nb", [(1, 4, 0), (7, 64, 100), (512, 768, 768), (512, 4096, 1024), (1000, 260, 4),
                                       (129, 0, 72), (16, 8, 0)])
 def test_sum_partials_matches_float64(P, na, nb):
