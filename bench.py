@@ -458,8 +458,15 @@ def main():
     # many tokens, diagonal BH4, fp32 tables: the projection kernel writes the gather's record stream itself
     st = layer._inference_state()
     rec_plan = None
-    if not fused_layer and not block and not wl["bf16"] and T % 2 == 0 and st is not None and st["form"] == "diag":
+    if not fused_layer and not wl["bf16"] and T % 2 == 0 and st is not None:
         rec_plan = ops.lookup_gather_records_plan(B, T, S, Do)
+
+    def records_front():
+        if block:
+            return ops.ln_bh4_block_hash_records_direct(x, st["ln_w"], st["ln_b"], st["eps"], layer.hash.folded_weight(),
+                                                        st["pbias"], T, st["decay"], st["res_coef"], rec_plan)
+        return ops.ln_project_hash_records_direct(x, st["ln_w"], st["ln_b"], st["eps"], st["diag"], st["pbias"],
+                                                  T, st["decay"], st["res_coef"], rec_plan)
 
     def step(events=None):
         # exactly what LookupFFN.forward runs in eval mode (checked below), with an
@@ -473,8 +480,7 @@ def main():
                     events[1].record()
                 return out
             if rec_plan is not None:
-                records = ops.ln_project_hash_records_direct(x, st["ln_w"], st["ln_b"], st["eps"], st["diag"], st["pbias"],
-                                                             T, st["decay"], st["res_coef"], rec_plan)
+                records = records_front()
                 if events is not None:
                     events[0].record()
                 out = ops.lookup_gather_records_direct(records, rec_plan, st["tables"], st["obias"], None, B)
@@ -566,8 +572,7 @@ def main():
         return a.elapsed_time(b) / n
     def front():
         if rec_plan is not None:
-            return ops.ln_project_hash_records_direct(x, st["ln_w"], st["ln_b"], st["eps"], st["diag"], st["pbias"],
-                                                      T, st["decay"], st["res_coef"], rec_plan)
+            return records_front()
         return hash_front()
     with torch.no_grad():
         hash_ms = None if fused_layer else timed(front)
@@ -617,7 +622,8 @@ def main():
         "config": {"workload": wl["desc"], "tokens": B, "d_model": H, "fht_dim": layer.hash.projection.padded_in_dim,
                    "tables": T, "table_size": S, "d_out": Do,
                    "step": ("one kernel: LayerNorm + BH4(block 64)x4 on fp32 MFMA + mix + hash (weights folded once, "
-                            "outside the step); one kernel: gather-add + bias") if block else
+                            "outside the step)" + (", written as the gather's record stream" if rec_plan is not None else "") +
+                            "; one kernel: gather-add + bias") if block else
                            ("one kernel: LayerNorm + BH4(block 1)x4 + mix + hash + gather-add + bias" if fused_layer else
                             ("one kernel: LayerNorm + BH4(block 1)x4 + mix + hash, written as the gather's record stream; "
                              "one kernel: gather-add + bias") if rec_plan is not None else

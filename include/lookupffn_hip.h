@@ -347,6 +347,12 @@ int lffn_ln_project_hash_records_f32(const float *x, const float *ln_weight, con
                                      const float *diag, const float *proj_bias, uint32_t *records,
                                      int64_t record_stride, int64_t B, int64_t H, int64_t D, int64_t R,
                                      int64_t J, int64_t T, float decay, float residual, void *stream);
+/* lffn_ln_bh4_block_hash_f32 (below) with its codes and scores written as records in the same way. */
+int lffn_ln_bh4_block_hash_records_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
+                                       const float *w_folded, const float *proj_bias, uint32_t *records,
+                                       int64_t record_stride, int64_t B, int64_t H, int64_t D, int64_t R,
+                                       int64_t J, int64_t T, int64_t block_size, float decay, float residual,
+                                       void *stream);
 int lffn_lookup_gather_records_f32(const uint32_t *records, int64_t record_stride, const float *tables,
                                    const float *bias, const float *residual, float *out, int64_t B, int64_t T,
                                    int64_t S, int64_t Do, int32_t tokens_per_workgroup, void *stream);

@@ -74,6 +74,7 @@ SIGNATURES = {
     "lffn_lookup_gather_ws_bf16": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp],
     "lffn_lookup_gather_ws_planned_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, ctypes.c_int32, ctypes.c_int32, _vp],
     "lffn_ln_project_hash_records_f32": [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _vp],
+    "lffn_ln_bh4_block_hash_records_f32": [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _vp],
     "lffn_lookup_gather_records_plan": [_i64, _i64, _i64, _i64, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64)],
     "lffn_lookup_gather_records_f32": [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, ctypes.c_int32, _vp],
     "lffn_lookup_gather_plan": [_i64, _i64, _i64, _i64, ctypes.c_int32, ctypes.POINTER(ctypes.c_int32)],

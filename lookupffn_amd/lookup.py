@@ -392,12 +392,17 @@ class LookupFFN(nn.Module):
             # small batches: the whole layer in one launch
             return ops.lookup_ffn_fused_direct(x, st["ln_w"], st["ln_b"], st["eps"], st["diag"], st["pbias"],
                                                st["tables"], st["obias"], residual, st["decay"], st["res_coef"])
-        if st["form"] == "diag" and st["tables"].dtype == torch.float32 and self.num_table % 2 == 0:
+        if st["tables"].dtype == torch.float32 and self.num_table % 2 == 0:
             # many tokens: the projection kernel writes the gather kernel's record stream directly
             plan = ops.lookup_gather_records_plan(x.shape[0], self.num_table, self.table_size, self.output_size)
-            if plan is not None and st["diag"].shape[2] >= 16:
+            records = None
+            if plan is not None and st["form"] == "diag" and st["diag"].shape[2] >= 16:
                 records = ops.ln_project_hash_records_direct(x, st["ln_w"], st["ln_b"], st["eps"], st["diag"], st["pbias"],
                                                              self.num_table, st["decay"], st["res_coef"], plan)
+            elif plan is not None and st["form"] == "block":
+                records = ops.ln_bh4_block_hash_records_direct(x, st["ln_w"], st["ln_b"], st["eps"], self.hash.folded_weight(),
+                                                               st["pbias"], self.num_table, st["decay"], st["res_coef"], plan)
+            if records is not None:
                 return ops.lookup_gather_records_direct(records, plan, st["tables"], st["obias"], residual, x.shape[0])
         if st["form"] == "diag":
             code, score, _ = ops.ln_project_hash_direct(x, st["ln_w"], st["ln_b"], st["eps"], st["diag"], st["pbias"],

@@ -759,6 +759,23 @@ def ln_project_hash_records_direct(x, ln_w, ln_b, eps, diag, pbias, T, decay, re
     return records
 
 
+def ln_bh4_block_hash_records_direct(x, ln_w, ln_b, eps, w_folded, pbias, T, decay, residual, plan):
+    """The same for BH4 with 64 x 64 blocks (folded weights [R, J, D/64, 64, 64]) on the matrix cores."""
+    assert x.dtype == torch.float32 and x.is_cuda and x.is_contiguous() and x.dim() == 2
+    B, H = x.shape
+    R, J, NB, bs, _ = w_folded.shape
+    D = NB * bs
+    assert H == ln_w.numel() and T * 8 <= R * D and T % 2 == 0 and plan[1] >= B
+    records = torch.empty(plan[2] // 4, dtype=torch.int32, device=x.device)
+    with _dev_guard(x):
+        rc = _lib.load().lffn_ln_bh4_block_hash_records_f32(
+            x.data_ptr(), ln_w.data_ptr(), ln_b.data_ptr(), eps, w_folded.data_ptr(), None if pbias is None else pbias.data_ptr(),
+            records.data_ptr(), plan[1], B, H, D, R, J, T, bs, decay, residual, _lib.stream_of(x))
+    if rc != 0:
+        _lib.check(rc, f"lffn_ln_bh4_block_hash_records_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T})")
+    return records
+
+
 def lookup_gather_records_direct(records, plan, tables, bias, residual, B):
     """out[b] = residual[b] + bias + sum_t score * row, from the record stream written for `plan`."""
     T, S, Do = tables.shape

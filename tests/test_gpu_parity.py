@@ -526,6 +526,41 @@ def test_layer_through_the_record_stream_matches_the_two_kernel_form(B, H, D, R,
     assert relmax(got[sub], want + obias + res[sub]) <= 1e-5
 
 
+@pytest.mark.parametrize("B,H,D,R,T,Do,tokens", [(4099, 768, 1024, 1, 128, 768, 1024), (2050, 256, 256, 2, 60, 128, 2048),
+                                                   (3000, 64, 64, 1, 8, 64, 1536)])
+def test_block_layer_through_the_record_stream(B, H, D, R, T, Do, tokens):
+    """lffn_ln_bh4_block_hash_records_f32: the records hold the codes and scores lffn_ln_bh4_block_hash_f32
+    writes, and the gather from them equals the gather kernel run on those codes and scores."""
+    rng = np.random.RandomState(B + H + T + 1)
+    S, J, bs = 256, 4, 64
+    x = (rng.randn(B, H) * 1.5 + 0.3).astype(np.float32)
+    ln_w = (1 + 0.1 * rng.randn(H)).astype(np.float32)
+    ln_b = (0.1 * rng.randn(H)).astype(np.float32)
+    w = (rng.randn(R, J, D // bs, bs, bs) / math.sqrt(bs * D)).astype(np.float32)
+    pbias = (0.05 * rng.randn(T * 8)).astype(np.float32)
+    tables = (0.02 * rng.randn(T, S, Do)).astype(np.float32)
+    obias = (0.001 * rng.randn(Do)).astype(np.float32)
+    wf = cabi.bh4_fold_mode(w, 0).reshape(w.shape)           # the forward fold (what lffn_bh4_fold_f32 writes)
+    codes, scores = cabi.ln_bh4_block_hash(x, ln_w, ln_b, 1e-5, w, pbias, T)
+    stride = -(-B // tokens) * tokens
+    rec = torch.full((3 * (T // 2) * stride,), -1, dtype=torch.int32, device="cuda:0")
+    out = torch.full((B, Do), float("nan"), dtype=torch.float32, device="cuda:0")
+    d = cabi.dev
+    xd, lw, lb, wd, pd, td, od = d(x), d(ln_w), d(ln_b), d(wf), d(pbias), d(tables), d(obias)
+    cabi._call("lffn_ln_bh4_block_hash_records_f32", cabi.p(xd), cabi.p(lw), cabi.p(lb), float(np.float32(1e-5)), cabi.p(wd),
+               cabi.p(pd), cabi.p(rec), stride, B, H, D, R, J, T, bs, float(np.float32(0.7)), float(np.float32(1 - 0.7)))
+    cabi._call("lffn_lookup_gather_records_f32", cabi.p(rec), stride, cabi.p(td), cabi.p(od), None, cabi.p(out), B, T, S, Do, tokens)
+    r = rec.cpu().numpy().view(np.uint32).reshape(T // 2, 3, stride)[:, :, :B]
+    swap = ((np.arange(B) & 2) != 0)[None, :]
+    c0, c1 = codes[:, 0::2].T, codes[:, 1::2].T
+    s0, s1 = scores[:, 0::2].T, scores[:, 1::2].T
+    assert np.array_equal(r[:, 0].view(np.float32), np.where(swap, s1, s0))
+    assert np.array_equal(r[:, 1].view(np.float32), np.where(swap, s0, s1))
+    assert np.array_equal(r[:, 2], np.where(swap, c1 | (c0 << 8), c0 | (c1 << 8)).astype(np.uint32))
+    rc, want = cabi.lookup_gather_ws_planned(codes, scores, tables, (3, tokens), bias=obias)
+    assert rc == 0 and np.array_equal(cabi.host(out), want)
+
+
 def test_record_stream_plan_and_refusals():
     from lookupffn_amd import _lib
     lib = _lib.load()
