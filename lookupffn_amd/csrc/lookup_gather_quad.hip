@@ -285,21 +285,6 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
         // order the quad takes the pair's tables
         LdsRecord rec0 = read_record<WAVE_RECS>(rec_read0);
         LdsRecord rec1 = read_record<WAVE_RECS>(rec_read1);
-        // Next pair's segments go straight into the other buffer (last read one pair ago, before the
-        // previous barrier); the last step copies the last pair's again.  Issued while the records are
-        // on their way from LDS.
-        const int kn = min(k + 1, npairs - 1);
-        copy_pair_to_lds(slice_base + (size_t)kn * pair_stride, lds0 + (uint32_t)((k + 1) & 1) * BUF_BYTES);
-        // both records have arrived (the compiler waits here) ...
-        asm volatile("" : "+v"(rec0.x), "+v"(rec0.y), "+v"(rec0.z), "+v"(rec1.x), "+v"(rec1.y), "+v"(rec1.z));
-        // ... so the next pair's records may overwrite them in LDS
-        copy_records_to_lds(kn);
-        if constexpr (TOUCH) {
-            const bool mine = turn == tile;                              // uniform
-            const int kt = mine ? min(k + QUAD_TOUCH_AHEAD, npairs - 1) : k;
-            l2_touch(slice_base + (size_t)kt * pair_stride, mine ? touch_off_on : 0u, touch_dst);
-            turn = turn + 1 == a.ntiles ? 0 : turn + 1;
-        }
 
         // Software pipeline over the passes: a pass's four rows are requested while the pass before
         // is still being added (its first table's two rows are consumed, their registers take the
@@ -321,12 +306,29 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
             return __uint_as_float(quad_broadcast<P % 4>(P < 4 ? (W ? rec0.y : rec0.x) : (W ? rec1.y : rec1.x)));
         };
         using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
+        // the first pass's rows are asked for before anything else ...
         u32x4 r[4];
         unsigned pk = rows_of(I0{});
         r[0] = *(lds_vec_ptr)(uintptr_t)with_row<0>(base[0], pk);
         r[1] = *(lds_vec_ptr)(uintptr_t)with_row<0>(base[1], pk);
         r[2] = *(lds_vec_ptr)(uintptr_t)with_row<1>(base[2], pk);
         r[3] = *(lds_vec_ptr)(uintptr_t)with_row<1>(base[3], pk);
+        __builtin_amdgcn_sched_barrier(0);
+        // ... and the copies are issued while they are on their way.  The records have been read (the row
+        // numbers above came from them), so the next pair's may overwrite them in LDS; the next pair's
+        // segments go straight into the other buffer (last read one pair ago, before the previous
+        // barrier); the last step copies the last pair's again.
+        asm volatile("" : "+v"(rec0.x), "+v"(rec0.y), "+v"(rec0.z), "+v"(rec1.x), "+v"(rec1.y), "+v"(rec1.z));
+        const int kn = min(k + 1, npairs - 1);
+        copy_records_to_lds(kn);
+        copy_pair_to_lds(slice_base + (size_t)kn * pair_stride, lds0 + (uint32_t)((k + 1) & 1) * BUF_BYTES);
+        if constexpr (TOUCH) {
+            const bool mine = turn == tile;                              // uniform
+            const int kt = mine ? min(k + QUAD_TOUCH_AHEAD, npairs - 1) : k;
+            l2_touch(slice_base + (size_t)kt * pair_stride, mine ? touch_off_on : 0u, touch_dst);
+            turn = turn + 1 == a.ntiles ? 0 : turn + 1;
+        }
+        __builtin_amdgcn_sched_barrier(0);
         static_for<NP>([&](auto p_c) {
             constexpr int P = decltype(p_c)::value;
             constexpr bool MORE = P + 1 < NP;
