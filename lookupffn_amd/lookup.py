@@ -184,7 +184,11 @@ class Hashing(nn.Module):
 
     def folded_weight(self):
         """The BH4 weights with the 64-point transform applied (what ops.bh4_block takes), kept
-        until the parameter is modified or moved."""
+        until the parameter is modified or moved.  Modifications are seen through the tensor's
+        version counter, which in-place writes through ``.data`` (``w.data.add_(...)``, some
+        hand-written optimizers) do not advance: after such a write call
+        ``invalidate_folded_weight()``; switching the module between train() and eval() drops
+        the cached copy as well."""
         w = self.projection.weight
         key = (w._version, w.data_ptr(), w.device)
         cached = getattr(self, "_folded", None)
@@ -192,6 +196,15 @@ class Hashing(nn.Module):
             cached = (key, ops.bh4_fold(w.detach().contiguous()))
             self._folded = cached
         return cached[1]
+
+    def invalidate_folded_weight(self):
+        """Forget the folded copy of the BH4 weights: the next block-64 inference call folds again."""
+        self._folded = None
+
+    def train(self, mode=True):
+        if mode != self.training:
+            self._folded = None           # weights usually change between an eval and the next one
+        return super().train(mode)
 
     def forward_block(self, x, layer_norm=None):
         """8-bit codes: one kernel, (LayerNorm ->) BH4 on the matrix cores -> mix -> bias ->

@@ -401,7 +401,16 @@ def test_checkpoint_round_trip_and_folded_weight_cache(tmp_path):
         assert torch.equal(b(x), out_a)           # not the stale folded weights
         # an in-place update (an optimizer step) is seen as well
         b.hash.projection.weight.mul_(0.5)
-        assert not torch.equal(b(x), out_a)
+        out_half = b(x)
+        assert not torch.equal(out_half, out_a)
+        # a write through .data does not advance the version counter: the folded copy stays until it is
+        # invalidated by hand, or by a switch between train() and eval()
+        b.hash.projection.weight.data.mul_(2.0)
+        b.hash.invalidate_folded_weight()
+        assert torch.equal(b(x), out_a)
+        b.hash.projection.weight.data.mul_(0.5)
+        b.train(); b.eval()
+        assert torch.equal(b(x), out_half)
 
 
 @pytest.mark.parametrize("bs", [1, 64])
