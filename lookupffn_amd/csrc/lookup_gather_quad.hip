@@ -278,13 +278,15 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
     copy_records_to_lds(0);
     copy_pair_to_lds(slice_base, lds0);
     __builtin_amdgcn_s_waitcnt(WAIT_VMCNT_0);
+    // A pair's records: x, y = the scores and z = the row numbers (first | second << 8), in the order the
+    // quad takes the pair's tables.  They sit in this wavefront's own corner of LDS and it has just waited
+    // for its own copies, so they are read BEFORE the barrier: their latency is out of the way when the
+    // barrier opens and the first row reads go out at once.
+    LdsRecord rec0 = read_record<WAVE_RECS>(rec_read0);
+    LdsRecord rec1 = read_record<WAVE_RECS>(rec_read1);
     __syncthreads();
 
     for (int k = 0; k < npairs; ++k) {
-        // this pair's records: x, y = the scores and z = the row numbers (first | second << 8), in the
-        // order the quad takes the pair's tables
-        LdsRecord rec0 = read_record<WAVE_RECS>(rec_read0);
-        LdsRecord rec1 = read_record<WAVE_RECS>(rec_read1);
 
         // Software pipeline over the passes: a pass's four rows are requested while the pass before
         // is still being added (its first table's two rows are consumed, their registers take the
@@ -358,6 +360,9 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
         for (int i = 0; i < 4; ++i) base[i] ^= (unsigned)BUF_BYTES;
         // the copies issued above have landed (records and segments); the touch, issued after them, may still be out
         __builtin_amdgcn_s_waitcnt(TOUCH ? WAIT_VMCNT_1 : WAIT_VMCNT_0);
+        // the next pair's records (this wavefront's own, just landed), then the barrier for the segments
+        rec0 = read_record<WAVE_RECS>(rec_read0);
+        rec1 = read_record<WAVE_RECS>(rec_read1);
         __syncthreads();
     }
     __builtin_amdgcn_s_waitcnt(WAIT_VMCNT_0);         // nothing may still be writing this workgroup's LDS when it ends
