@@ -1044,6 +1044,52 @@ def test_every_gather_form_and_the_inner_product_on_random_shapes():
             assert np.abs(got_i - want_i).max() <= 1e-5 * np.abs(want_i).max(), (it, B, T, S, Do)
 
 
+def test_four_lane_gather_and_record_layer_on_random_shapes():
+    """Seeded sweep: the four-lanes-per-token gather at every tile size on ragged shapes (1 to 39 table
+    pairs, token counts around the quad, wavefront, pass and tile boundaries, bias and residual on and
+    off), the workspace entry point's own choice, and the layer through the record stream, all against
+    float64 sums."""
+    rng = np.random.RandomState(4242)
+    S = 256
+    for it in range(20):
+        T = 2 * int(rng.randint(1, 40))
+        Do = int(rng.choice([64, 128, 192, 256, 512, 768]))
+        B = int(rng.choice([1, 2, 3, 5, 15, 17, 255, 257, 1023, 1025, 1791, 1793, 2047, 2049, 3000]))
+        tables = (0.1 * rng.randn(T, S, Do)).astype(np.float32)
+        code = rng.randint(0, S, size=(B, T)).astype(np.int32)
+        score = rng.rand(B, T).astype(np.float32)
+        bias = (0.01 * rng.randn(Do)).astype(np.float32) if rng.rand() < 0.7 else None
+        res = rng.randn(B, Do).astype(np.float32) if rng.rand() < 0.5 else None
+        want = np.einsum("bt,btd->bd", score.astype(np.float64), tables[np.arange(T)[None, :], code].astype(np.float64))
+        want = want + (0 if bias is None else bias) + (0 if res is None else res)
+        scale = np.abs(want).max()
+        for tok in (1024, 1536, 1792, 2048):
+            rc, got = cabi.lookup_gather_ws_planned(code, score, tables, (3, tok), bias=bias, residual=res)
+            assert rc == 0 and np.abs(got - want).max() <= 1e-5 * scale, (it, B, T, Do, tok)
+        got = cabi.lookup_gather_ws(code, score, tables, bias, residual=res)
+        assert np.abs(got - want).max() <= 1e-5 * scale, (it, B, T, Do)
+    for it in range(8):
+        D = int(rng.choice([64, 128, 256, 512, 1024]))
+        R = int(rng.choice([1, 2])) if D <= 256 else 1
+        H = int(rng.choice([D, D - 4, D // 2 + 4]))
+        T = 2 * int(rng.randint(1, R * D // 16 + 1))
+        Do = int(rng.choice([64, 128, 256]))
+        B = int(rng.choice([1, 3, 5, 31, 33, 257, 1000, 2049]))
+        tok = int(rng.choice([1024, 1536, 1792, 2048]))
+        stride = -(-B // tok) * tok
+        x = (rng.randn(B, H) * 1.5 + 0.3).astype(np.float32)
+        ln_w = (1 + 0.1 * rng.randn(H)).astype(np.float32)
+        ln_b = (0.1 * rng.randn(H)).astype(np.float32)
+        diag = ((2 * rng.randint(0, 2, size=(R, 4, D)) - 1) / math.sqrt(D)).astype(np.float32)
+        pbias = (0.05 * rng.randn(T * 8)).astype(np.float32)
+        tables = (0.1 * rng.randn(T, S, Do)).astype(np.float32)
+        obias = (0.01 * rng.randn(Do)).astype(np.float32)
+        got, _ = cabi.layer_through_records(x, ln_w, ln_b, 1e-5, diag, pbias, tables, obias, plan=(tok, stride, 6 * T * stride))
+        codes, scores, _ = cabi.ln_project_hash(x, ln_w, ln_b, 1e-5, diag, pbias, T)
+        want = obias + np.einsum("bt,btd->bd", scores.astype(np.float64), tables[np.arange(T)[None, :], codes].astype(np.float64))
+        assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max(), (it, B, H, D, R, T, Do, tok)
+
+
 def test_gather_special_cases():
     rng = np.random.RandomState(30)
     tables, code, idx, w = _rand_gather(rng, 16, 8, 16, 128)
