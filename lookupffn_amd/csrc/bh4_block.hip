@@ -621,10 +621,14 @@ int dispatch_block_bwd(const BlockArgs &a, int64_t D, hipStream_t st) {
 template <bool HASH>
 int dispatch_block(const BlockArgs &a, int64_t D, hipStream_t st) {
     switch (D / BS) {
-        case 1: return launch_block<1, HASH, 2>(a, st);
-        case 2: return launch_block<2, HASH, 2>(a, st);
+        // The hash form as 16-token workgroups of 4 wavefronts where that measured faster (more workgroups
+        // per compute unit: the vector work of one hides behind the products of the others): 32768 tokens,
+        // D = 512, two repeats 268 -> 212 us; D = 128 74 -> 70 us; D = 64 44 -> 41 us; D = 256 65 -> 69 us
+        // (kept on 32 tokens); the plain form is as fast or faster with 32 tokens everywhere.
+        case 1: return HASH ? launch_block<1, HASH, 1, false, 1>(a, st) : launch_block<1, HASH, 2>(a, st);
+        case 2: return HASH ? launch_block<2, HASH, 1, false, 1>(a, st) : launch_block<2, HASH, 2>(a, st);
         case 4: return launch_block<4, HASH, 2>(a, st);
-        case 8: return launch_block<8, HASH, 2>(a, st);
+        case 8: return HASH ? launch_block<8, HASH, 1, false, 1>(a, st) : launch_block<8, HASH, 2>(a, st);
         // measured at 16384 x 1024: the plain form 110 us with 4 wavefronts, 118 us with 8 (the
         // second fetch of the weight fragments costs more than the other phases gain); the hash
         // form 141 us with 4, 133 us with 8 (LayerNorm and the hash are vector-ALU work), 118 us
