@@ -15,7 +15,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_NAME = "liblookupffn_hip.so"
 LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
-SOURCES = ["fht.hip", "code_score.hip", "gather.hip", "lookup_gather.hip", "lookup_gather_pair.hip", "lookup_gather_quad.hip", "lookup_scatter.hip", "lookup_scatter_sorted.hip", "lookup_inner.hip", "bh4_block.hip", "bh4_wgrad.hip", "layer_norm.hip"]
+SOURCES = ["fht.hip", "code_score.hip", "gather.hip", "lookup_gather.hip", "lookup_gather_pair.hip", "lookup_gather_quad.hip", "lookup_scatter.hip", "lookup_scatter_sorted.hip", "lookup_inner.hip", "lookup_inner_quad.hip", "bh4_block.hip", "bh4_wgrad.hip", "layer_norm.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

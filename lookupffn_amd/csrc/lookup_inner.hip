@@ -254,6 +254,15 @@ extern "C" int lffn_lookup_inner_f32(const int32_t *code, const float *g, const 
     if (B * T == 0) return LFFN_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int64_t nslices = Do / 64;
+    // Four lanes per token, one owner per (token, table) (lookup_inner_quad.hip): tiles of 1024 tokens x
+    // chunks of 4 or 2 table pairs; 4 when that still gives the chip a round of workgroups (the g values are
+    // fetched once per chunk and slice), and the form below when even 2 leaves most of it idle.
+    if (S == MAX_S && T % 2 == 0 && reinterpret_cast<uintptr_t>(code) % 8 == 0 && 2 * S * Do * 4 < (int64_t(1) << 32)) {
+        const int64_t tiles = (B + 1023) / 1024, pairs = T / 2;
+        const int c = tiles * ((pairs + 3) / 4) >= 200 ? 4 : (tiles * ((pairs + 1) / 2) >= 96 ? 2 : 0);
+        if (c) return lffn_internal_lookup_inner_quad(code, g, Do, 32, tables, grad_score, B, T, S, Do, 4, c, stream);
+    }
+
     // LDS form: table fits the buffers, and enough (token tile, slice) units to fill most CUs
     const bool lds_ok = S <= MAX_S && T >= 4 && B * T < (int64_t(1) << 30) &&
                         ((B + 255) / 256) * nslices >= 192 && B * nslices <= (int64_t(1) << 30);

@@ -1271,11 +1271,16 @@ def test_lookup_scatter_full_size_zipf_properties():
 
 # (B, T, S, Do): the LDS kernel needs ceil(B/256) * Do/64 >= 192 units, T >= 4 and S <= 256; the
 # first rows take it with each token tile (832, 512, 256 tokens), ragged token counts, table counts
-# that are no multiple of the 16-table chunk and tables smaller than the LDS slice; the rest fall
-# back to the token-major kernel
+# that are no multiple of the 16-table chunk and tables smaller than the LDS slice; the next rows
+# fall back to the token-major kernel.  The last rows take the four-lanes-per-token kernel (S = 256,
+# T even, ceil(B/1024) * ceil(T/8) >= 200 workgroups with chunks of 4 table pairs, or
+# ceil(B/1024) * ceil(T/4) >= 96 with chunks of 2): last chunks of 1, 3 and 2 pairs, a last tile of one
+# token, a last chunk of 1 pair with chunks of 2.
 INNER_CASES = [(16384, 20, 256, 768), (4100, 17, 256, 768), (3000, 5, 64, 1024), (12289, 33, 16, 768),
                (8191, 16, 256, 1536), (8191, 9, 128, 768), (256, 32, 256, 256), (1, 2, 4, 64), (65, 5, 256, 192),
-               (500, 4, 512, 128), (2000, 3, 256, 1024), (0, 4, 16, 64)]
+               (500, 4, 512, 128), (2000, 3, 256, 1024), (0, 4, 16, 64),
+               (20000, 82, 256, 64), (20481, 86, 256, 64), (24000, 76, 256, 128), (6000, 66, 256, 64),
+               (4096, 128, 256, 192)]
 
 
 @pytest.mark.parametrize("B,T,S,Do", INNER_CASES)
