@@ -260,7 +260,7 @@ extern "C" int lffn_lookup_inner_f32(const int32_t *code, const float *g, const 
     if (S == MAX_S && T % 2 == 0 && reinterpret_cast<uintptr_t>(code) % 8 == 0 && 2 * S * Do * 4 < (int64_t(1) << 32)) {
         const int64_t tiles = (B + 1023) / 1024, pairs = T / 2;
         const int c = tiles * ((pairs + 3) / 4) >= 200 ? 4 : (tiles * ((pairs + 1) / 2) >= 96 ? 2 : 0);
-        if (c) return lffn_internal_lookup_inner_quad(code, g, Do, 32, tables, grad_score, B, T, S, Do, 4, c, stream);
+        if (c && tiles * ((pairs + c - 1) / c) <= (int64_t(1) << 30)) return lffn_internal_lookup_inner_quad(code, g, Do, 32, tables, grad_score, B, T, S, Do, 4, c, stream);
     }
 
     // LDS form: table fits the buffers, and enough (token tile, slice) units to fill most CUs

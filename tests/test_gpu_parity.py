@@ -1302,6 +1302,23 @@ def test_lookup_inner_matches_oracle(B, T, S, Do):
     assert relmax(cabi.lookup_inner(dirty, g, tables), want) <= 1e-5
 
 
+def test_lookup_inner_is_reproducible_where_every_sum_has_one_owner():
+    # the four-lanes-per-token kernel adds a (token, table)'s 24 slice sums in a fixed order in one
+    # lane: two runs agree bit for bit (the form with atomics does not promise that)
+    rng = np.random.RandomState(77)
+    B, T, S, Do = 16384, 128, 256, 768
+    tables, code, _, _ = _rand_gather(rng, B, T, S, Do)
+    g = rng.randn(B, Do).astype(np.float32)
+    first = cabi.lookup_inner(code, g, tables)
+    second = cabi.lookup_inner(code, g, tables)
+    assert np.array_equal(first, second)
+    # where a token sits in the batch (tile, pass, quad) only changes the order in which its quad adds the
+    # two halves of a 32-column slice
+    perm = rng.permutation(B)
+    moved = cabi.lookup_inner(np.ascontiguousarray(code[perm]), np.ascontiguousarray(g[perm]), tables)
+    assert relmax(moved, first[perm].astype(np.float64)) <= 1e-6
+
+
 def test_lookup_inner_full_size_duality():
     # BASELINE.json config 2 shape: <G(w), g> = sum_bt w[b,t] * grad_score[b,t], and linearity in g
     rng = np.random.RandomState(43)
