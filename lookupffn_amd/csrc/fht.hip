@@ -3,8 +3,11 @@
 // fused projection -> mix -> bias -> 8-bit code + score front-end.
 //
 // One row (or, for D < 256, 256/D rows) lives in the registers of one 64-lane
-// wavefront for the whole computation: nothing is staged in LDS and nothing
-// round-trips through memory between the transforms.
+// wavefront for the whole computation: nothing round-trips through memory between
+// the transforms.  The forward kernel's 512- and 1024-point transforms turn the row
+// round through the wavefront's own 4 KB of LDS twice per transform, so that the
+// upper lane bits become register bits for a while (fht_rows_xl below: 16 % faster
+// than six cross-lane stages at D = 1024); everything else stays in registers.
 //
 // Register layout.  A lane holds NJ float4; value c of float4 j of row-lane lr is
 // element  e = 256*j + 4*lr + c.  So bits 0-1 of e are in-register (c), bits 2..
@@ -122,6 +125,86 @@ __device__ __forceinline__ void fht_rows(float (&v)[FhtCfg<LOGD>::NJ][4], int lr
     lane_stage<2, C::LPR, NJ, SWAP>(v, lr);
     lane_stage<1, C::LPR, NJ, SWAP>(v, lr);
     // strides 2 and 1: inside a float4
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        float a0 = v[j][0], a1 = v[j][1], a2 = v[j][2], a3 = v[j][3];
+        float b0 = a0 + a2, b2 = a0 - a2, b1 = a1 + a3, b3 = a1 - a3;
+        v[j][0] = b0 + b1;
+        v[j][1] = b0 - b1;
+        v[j][2] = b2 + b3;
+        v[j][3] = b2 - b3;
+    }
+}
+
+// The 512- and 1024-point transforms with two trips through LDS instead of cross-lane moves for the
+// upper lane bits.  A lane holds NV = 4*NJ values (8 or 16).  Strides >= 256 are register pairs in the
+// load layout, as in fht_rows; then the row is written to the wavefront's own LDS region and read back
+// with the top log2(NV) lane bits of the element index in registers (element bits 8-KB .. 7; the lane
+// is the low 8-KB bits and bits 8-9), strides 128 .. 2^(8-KB) are plain adds, the row goes back the
+// same way, the remaining lane strides (lanes 2 and 1 apart at D = 1024; 4, 2, 1 at 512) are DPP
+// butterflies and strides 2 and 1 are inside a float4.  Same additions in the same order as fht_rows:
+// results are bit-identical.  Each block of 256 floats starts PAD floats after the one before, so that
+// the 64 lanes of a transposed access fall on 64 different banks.
+template <int LOGD>
+struct XlCfg {
+    static constexpr int NJ = FhtCfg<LOGD>::NJ, NV = 4 * NJ;
+    static constexpr int KB = LOGD - 6;              // element bits 8-KB .. 7 in registers after the first trip
+    static constexpr int STEP = 1 << (8 - KB);       // floats between a lane's values in the transposed layout
+    static constexpr int BLOCK = 256 + STEP;         // floats from one block of 256 to the next
+    static constexpr int ROW = NJ * BLOCK;           // floats per wavefront region
+    static_assert(LOGD == 9 || LOGD == 10, "two-trip form: 512 and 1024 points");
+};
+
+template <int LOGD>
+__device__ __forceinline__ void fht_rows_xl(float (&v)[FhtCfg<LOGD>::NJ][4], int lr, float *wl) {
+    using X = XlCfg<LOGD>;
+    constexpr int NJ = X::NJ, NV = X::NV, STEP = X::STEP, BLOCK = X::BLOCK;
+    if constexpr (NJ == 4) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                float a = v[j][c], b = v[j + 2][c];
+                v[j][c] = a + b;
+                v[j + 2][c] = a - b;
+            }
+    }
+#pragma unroll
+    for (int j = 0; j < NJ; j += 2)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            float a = v[j][c], b = v[j + 1][c];
+            v[j][c] = a + b;
+            v[j + 1][c] = a - b;
+        }
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+        *reinterpret_cast<float4 *>(wl + BLOCK * j + 4 * lr) = make_float4(v[j][0], v[j][1], v[j][2], v[j][3]);
+    // transposed: lane = (element bits 0 .. 7-KB) | (bits 8-9) << (8-KB); value k = element bits 8-KB .. 7
+    float *col = wl + BLOCK * (lr / STEP) + (lr % STEP);
+    float w[NV];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) w[k] = col[STEP * k];
+#pragma unroll
+    for (int bit = NV / 2; bit >= 1; bit >>= 1)
+#pragma unroll
+        for (int k = 0; k < NV; ++k)
+            if (!(k & bit)) {
+                float a = w[k], b = w[k | bit];
+                w[k] = a + b;
+                w[k | bit] = a - b;
+            }
+#pragma unroll
+    for (int k = 0; k < NV; ++k) col[STEP * k] = w[k];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        const float4 t = *reinterpret_cast<const float4 *>(wl + BLOCK * j + 4 * lr);
+        v[j][0] = t.x; v[j][1] = t.y; v[j][2] = t.z; v[j][3] = t.w;
+    }
+    // lane strides STEP/8 .. 1 (element strides STEP/2 .. 4)
+    if constexpr (STEP / 8 >= 4) lane_stage<4, 64, NJ, false>(v, lr);
+    lane_stage<2, 64, NJ, false>(v, lr);
+    lane_stage<1, 64, NJ, false>(v, lr);
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
         float a0 = v[j][0], a1 = v[j][1], a2 = v[j][2], a3 = v[j][3];
@@ -347,7 +430,12 @@ __global__ __launch_bounds__(256) void project_kernel(ProjectArgs a) {
                     v[j][3] = v[j][3] * w.w;
                 }
             }
-            fht_rows<LOGD>(v, lr);
+            if constexpr ((LOGD == 10 || LOGD == 9) && !GATHER) {
+                __shared__ float xl[4 * XlCfg<LOGD>::ROW];
+                fht_rows_xl<LOGD>(v, lr, xl + wave * XlCfg<LOGD>::ROW);
+            } else {
+                fht_rows<LOGD>(v, lr);
+            }
         }
 
 #pragma unroll
@@ -519,6 +607,9 @@ __global__ __launch_bounds__(256) void project_hash_bwd_kernel(ProjectBwdArgs a)
     const int wave = threadIdx.x >> 6;
     const int lr = lane;
     const int r = blockIdx.y;
+    // Cross-lane swaps, not the two-trip form of the forward kernel: with two wavefronts per SIMD every
+    // LDS round trip is waited for (165 us against 117 us at 16384 x 1024, four stages).
+    auto transform = [&](float (&t)[NJ][4]) { fht_rows<LOGD, true>(t, lr); };
     const int ncols = a.T * 8;
     const int64_t nwaves = int64_t(gridDim.x) * 4;
 
@@ -586,7 +677,7 @@ __global__ __launch_bounds__(256) void project_hash_bwd_kernel(ProjectBwdArgs a)
                     for (int c = 0; c < 4; ++c) u[s][j][c] = t[j][c];
                     t[j][0] = t[j][0] * w.x; t[j][1] = t[j][1] * w.y; t[j][2] = t[j][2] * w.z; t[j][3] = t[j][3] * w.w;
                 }
-                if (s + 1 < a.J) fht_rows<LOGD, true>(t, lr);      // the last transform's output is not needed
+                if (s + 1 < a.J) transform(t);                     // the last transform's output is not needed
             }
         }
 
@@ -640,7 +731,7 @@ __global__ __launch_bounds__(256) void project_hash_bwd_kernel(ProjectBwdArgs a)
 #pragma unroll
         for (int s = MAXJ - 1; s >= 0; --s) {
             if (s < a.J) {
-                fht_rows<LOGD, true>(t, lr);
+                transform(t);
                 const float *dg = a.diag + (int64_t(r) * a.J + s) * D;
 #pragma unroll
                 for (int j = 0; j < NJ; ++j) {
