@@ -823,7 +823,12 @@ __global__ __launch_bounds__(256) void fht16_kernel(const uint16_t *__restrict__
         v[j][2] = widen16<BF16>(t.y & 0xffffu);
         v[j][3] = widen16<BF16>(t.y >> 16);
     }
-    fht_rows<LOGD>(v, lr);
+    if constexpr (LOGD == 10 || LOGD == 9) {
+        __shared__ float xl[4 * XlCfg<LOGD>::ROW];
+        fht_rows_xl<LOGD>(v, lr, xl + wave * XlCfg<LOGD>::ROW);
+    } else {
+        fht_rows<LOGD>(v, lr);
+    }
     if (live) {
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
