@@ -1090,6 +1090,31 @@ def test_four_lane_gather_and_record_layer_on_random_shapes():
         assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max(), (it, B, H, D, R, T, Do, tok)
 
 
+def test_inner_product_four_lane_kernel_on_random_shapes():
+    """Seeded sweep of lffn_lookup_inner_f32 over shapes that take the four-lanes-per-token kernel (S = 256,
+    32 to 69 table pairs, 6 to 21 tiles of 1024 tokens: chunks of 2 or 4 pairs, last chunks of 1 to 3,
+    ragged last tiles) against the token-major kernel on every entry and float64 sums on a sample."""
+    rng = np.random.RandomState(777)
+    S = 256
+    for it in range(8):
+        T = 2 * int(rng.randint(32, 70))
+        Do = int(rng.choice([64, 128, 192]))
+        B = int(rng.choice([6000, 7169, 8193, 12000, 16385, 20481]))
+        tables = (0.1 * rng.randn(T, S, Do)).astype(np.float32)
+        code = rng.randint(0, S, size=(B, T)).astype(np.int32)
+        g = rng.randn(B, Do).astype(np.float32)
+        got = cabi.lookup_inner(code, g, tables)
+        assert not np.isnan(got).any(), (it, B, T, Do)
+        idx = code + (np.arange(T, dtype=np.int32) * S)[None]
+        flat = tables.reshape(T * S, Do)
+        other = cabi.indexed_inner_product(idx, g, flat)
+        scale = np.abs(other).max()
+        assert np.abs(got.astype(np.float64) - other).max() <= 2e-6 * scale, (it, B, T, Do)
+        sub = np.unique(np.concatenate([rng.choice(B, 64, replace=False), np.arange(B - 20, B), np.arange(1020, 1030)]))
+        want = oracle.indexed_inner_product(idx[sub], g[sub].astype(np.float64), flat.astype(np.float64))
+        assert np.abs(got[sub] - want).max() <= 1e-5 * np.abs(want).max(), (it, B, T, Do)
+
+
 def test_gather_special_cases():
     rng = np.random.RandomState(30)
     tables, code, idx, w = _rand_gather(rng, 16, 8, 16, 128)
