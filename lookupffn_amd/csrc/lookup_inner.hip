@@ -2,6 +2,10 @@
 //
 //   grad_score[b,t] = < g[b,:], tables[t, code[b,t] & (S-1), :] >
 //
+// This file: the entry point, and the form with atomics that serves the shapes the
+// four-lanes-per-token kernel of lookup_inner_quad.hip does not take (S < 256, an odd
+// number of tables, too few tokens to fill the chip with 1024-token tiles).
+//
 // The mirror image of lookup_gather.hip.  A 1024-lane workgroup owns a 256-byte
 // column slice (64 fp32 columns) and a tile of 64*NP tokens whose slice of g stays
 // in registers for the whole kernel (16 lanes side by side hold a token's 64
