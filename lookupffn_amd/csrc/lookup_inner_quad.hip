@@ -60,6 +60,7 @@ struct InnerQuadArgs {
     int64_t B;
     int T, S, Do;          // T even, S = 256
     int ntiles, nchunks, nslices, per_xcd;
+    int group_tiles;       // tiles per tile group (see the unit order in the kernel)
     int row_bytes;         // Do * 4
 };
 
@@ -122,9 +123,17 @@ __global__ __launch_bounds__(WG) void lookup_inner_quad_kernel(InnerQuadArgs a) 
 
     const int xcd = blockIdx.x % XCDS;
     const int unit = xcd * a.per_xcd + blockIdx.x / XCDS;
-    if (unit >= a.ntiles * a.nchunks) return;     // uniform over the workgroup
-    const int chunk = unit / a.ntiles;            // the workgroups of a chunk sit side by side on one XCD
-    const int tile = unit % a.ntiles;
+    // Units in the order (tile group, chunk, tile of the group), consecutive units on one XCD: an XCD then
+    // works on group_tiles tiles x a few chunks, and what it pulls through the fabric is those chunks'
+    // tables once and those tiles' rows of g once per chunk group (every tile's workgroups of a chunk run in
+    // step and share the copies in L2).  The launch picks group_tiles to make the sum smallest.
+    const int group_units = a.nchunks * a.group_tiles;
+    const int group = unit / group_units, in_group = unit % group_units;
+    const int chunk = in_group / a.group_tiles;
+    const int tile_in_group = in_group % a.group_tiles;
+    const int tile = group * a.group_tiles + tile_in_group;
+    if (tile >= a.ntiles) return;                 // uniform over the workgroup (ragged last group; also past the last group)
+    const int team = min(a.group_tiles, a.ntiles - group * a.group_tiles);     // workgroups that share this chunk's copies
     const int npairs = a.T / 2;
     const int k0 = chunk * C;
     const int nk = min(C, npairs - k0);           // table pairs in this chunk
@@ -178,7 +187,7 @@ __global__ __launch_bounds__(WG) void lookup_inner_quad_kernel(InnerQuadArgs a) 
     };
 
     // Touch by turns (see lookup_gather_quad.hip): the workgroups of a chunk run in step; in step n the one
-    // whose tile number is n mod ntiles pulls all 2*S lines of the step TOUCH_AHEAD further on into the
+    // whose number among the chunk's workgroups on this XCD is n mod their count pulls all 2*S lines of the step TOUCH_AHEAD further on into the
     // XCD's L2, the others touch a line of the step they are on.
     const int my_line = tid < 2 * a.S ? tid : 0;
     const bool line_second = my_line >= a.S;
@@ -255,7 +264,7 @@ __global__ __launch_bounds__(WG) void lookup_inner_quad_kernel(InnerQuadArgs a) 
             const int nkk = LAST_OF_SLICE ? (more_slices ? 0 : KK) : KK + 1;
             copy_pair_to_lds(uniform_ptr(step_base(nslice, nkk)), lds0 + (uint32_t)(parity ^ 1) * BUF_BYTES);
             // touch by turns: the step TOUCH_AHEAD further on (the last step, beyond it)
-            const bool mine = turn == tile;                              // uniform
+            const bool mine = turn == tile_in_group;                     // uniform
             int ts = slice, tk = KK + TOUCH_AHEAD;
 #pragma unroll
             for (int i = 0; i < TOUCH_AHEAD; ++i) {
@@ -263,7 +272,7 @@ __global__ __launch_bounds__(WG) void lookup_inner_quad_kernel(InnerQuadArgs a) 
             }
             if (ts >= a.nslices) { ts = a.nslices - 1; tk = NK - 1; }
             l2_touch(uniform_ptr(mine ? step_base(ts, tk) : step_base(slice, KK)), mine ? touch_off_on : 0u, touch_dst);
-            turn = turn + 1 == a.ntiles ? 0 : turn + 1;
+            turn = turn + 1 == team ? 0 : turn + 1;
         }
         __builtin_amdgcn_sched_barrier(0);
         static_for<NP>([&](auto p_c) {
@@ -349,7 +358,23 @@ template <int NP, int C>
 int launch_inner_quad(InnerQuadArgs a, hipStream_t stream) {
     a.ntiles = (int)((a.B + 256 * NP - 1) / (256 * NP));
     a.nchunks = (a.T / 2 + C - 1) / C;
-    const int units = a.ntiles * a.nchunks;
+    // tile groups: with per_xcd units on an XCD, group_tiles tiles and per_xcd / group_tiles chunks meet there;
+    // bytes through the fabric per XCD = chunks x (C pairs of tables) + tiles x (1024 rows of g)
+    {
+        const int per_xcd0 = (a.ntiles * a.nchunks + XCDS - 1) / XCDS;
+        const double chunk_bytes = double(C) * 2 * a.S * a.row_bytes, tile_bytes = 256.0 * NP * a.row_bytes;
+        int best = a.ntiles;
+        double best_bytes = 1e300;
+        for (int gt = a.ntiles; gt >= 1; gt = (gt + 1) / 2) {
+            const double bytes = double((per_xcd0 + gt - 1) / gt) * chunk_bytes + double(gt) * tile_bytes;
+            const int idle_tiles = (a.ntiles + gt - 1) / gt * gt - a.ntiles;          // of a ragged last group
+            if (bytes < best_bytes && idle_tiles * 8 <= a.ntiles) { best_bytes = bytes; best = gt; }
+            if (gt == 1) break;
+        }
+        a.group_tiles = best;
+    }
+    const int groups = (a.ntiles + a.group_tiles - 1) / a.group_tiles;
+    const int units = groups * a.nchunks * a.group_tiles;       // the last group's missing tiles included
     a.per_xcd = (units + XCDS - 1) / XCDS;
     const size_t lds_bytes = size_t(2) * BUF_BYTES + TOUCH_SINK_BYTES;
     auto kern = lookup_inner_quad_kernel<NP, C>;
