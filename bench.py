@@ -85,7 +85,7 @@ MEASURED_TRAFFIC = {
     "cfg2b64": {"bytes": 268655264, "form": "record stream (four lanes per token), 1792 tokens per workgroup"},
     "cfg3": {"bytes": 1092682313, "form": "record stream (four lanes per token), 2048 tokens per workgroup"},
     "cfg3bf16": {"bytes": 1393399611, "form": "1 table(s) per LDS buffer, 512 tokens per workgroup"},
-    "cfg5": {"bytes": 944883952, "form": "sorted"},
+    "cfg5": {"bytes": 944068093, "form": "sorted"},
 }
 
 
