@@ -1335,8 +1335,8 @@ def test_lookup_inner_is_reproducible_where_every_sum_has_one_owner():
     tables, code, _, _ = _rand_gather(rng, B, T, S, Do)
     g = rng.randn(B, Do).astype(np.float32)
     first = cabi.lookup_inner(code, g, tables)
-    second = cabi.lookup_inner(code, g, tables)
-    assert np.array_equal(first, second)
+    for _ in range(12):
+        assert np.array_equal(cabi.lookup_inner(code, g, tables), first)
     # where a token sits in the batch (tile, pass, quad) only changes the order in which its quad adds the
     # two halves of a 32-column slice
     perm = rng.permutation(B)
