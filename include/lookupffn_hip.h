@@ -220,8 +220,10 @@ int lffn_layer_norm_bwd_f32(const float *x, const float *ln_weight, float ln_eps
  *   g_x [B, H] as lffn_layer_norm_bwd_f32;  g_weight [H] = sum_b g * x^;  g_bias [H] = sum_b g
  * with min(512, max(1, ceil(B / 4))) partials, added up by lffn_sum_partials_f32 (chunks = 1): the
  * results are bit-identical to those two calls with that many partials.  No hipMalloc, hipFree or
- * other allocating call is made.  Shapes whose partials exceed the buffer (H > 1024) return
- * LFFN_ERR_SCRATCH.  The buffer keeps the last call's contents; every call overwrites all it reads, so
+ * other allocating call is made.  Rows wider than the buffer is sized for (H > 1024) return
+ * LFFN_ERR_SCRATCH, whatever B, before anything is launched.  The first call on a device looks up the
+ * buffer's device address (hipGetSymbolAddress, once per device): a caller that captures HIP graphs makes
+ * one call per device outside any capture first (an empty batch, B = 0, is enough).  The buffer keeps the last call's contents; every call overwrites all it reads, so
  * nothing needs clearing.  All calls on one GPU share the one buffer: calls that overlap on a GPU
  * (two streams, two threads) race.  ln_weight may be null (no affine; g_weight is still written).
  * No counterpart in the reference (it has no entry point of this kind; the operator is the LayerNorm
@@ -563,9 +565,12 @@ int lffn_lookup_scatter_sorted_f32(const int32_t *code, const float *score, cons
  *   grad_score[b, t] = < g[b, :], tables[t, code[b,t] & (S-1), :] >
  * code: [B, T] int32; g: [B, Do]; tables: [T, S, Do] fp32; grad_score: [B, T],
  * overwritten (it needs no zero-fill).  For S <= 256 the table slices are staged
- * in LDS and the partial sums of the 64-column slices of a row are combined with
- * global atomics, in no fixed order (as the partial sums of the reference's
- * kernel are, PL/gather/cuda/extension/gather_kernel_fp32.cu:141).
+ * in LDS.  At the layer's shapes (S = 256, T even, Do a multiple of 32, a few thousand
+ * tokens or more) every (token, table) sum has one owner that walks the column slices
+ * itself: no atomics, a fixed order of additions, results bit-identical from run to
+ * run.  The other shapes (S < 256, odd T, small batches) combine the partial sums of
+ * the 64-column slices of a row with global atomics, in no fixed order (as the partial
+ * sums of the reference's kernel are, PL/gather/cuda/extension/gather_kernel_fp32.cu:141).
  * Replaces WeightedVectorGatherAdd.backward's indexed_inner_product call
  * (PL/gather/cuda/kernel.py:199) together with the index offset of PL/lookup.py:126.
  */

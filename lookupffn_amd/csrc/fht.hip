@@ -155,6 +155,16 @@ struct XlCfg {
     static_assert(LOGD == 9 || LOGD == 10, "two-trip form: 512 and 1024 points");
 };
 
+// Between a phase in which the lanes of a wavefront store to the wavefront's own LDS region and the phase in
+// which they load what other lanes stored: the hardware executes a wavefront's LDS operations in order, so
+// no instruction is needed, but the compiler must not move or forward accesses across the hand-over.  A
+// release/acquire pair at wavefront scope and a wave barrier say so and emit nothing.
+__device__ __forceinline__ void wave_lds_handover() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 template <int LOGD>
 __device__ __forceinline__ void fht_rows_xl(float (&v)[FhtCfg<LOGD>::NJ][4], int lr, float *wl) {
     using X = XlCfg<LOGD>;
@@ -180,6 +190,7 @@ __device__ __forceinline__ void fht_rows_xl(float (&v)[FhtCfg<LOGD>::NJ][4], int
 #pragma unroll
     for (int j = 0; j < NJ; ++j)
         *reinterpret_cast<float4 *>(wl + BLOCK * j + 4 * lr) = make_float4(v[j][0], v[j][1], v[j][2], v[j][3]);
+    wave_lds_handover();
     // transposed: lane = (element bits 0 .. 7-KB) | (bits 8-9) << (8-KB); value k = element bits 8-KB .. 7
     float *col = wl + BLOCK * (lr / STEP) + (lr % STEP);
     float w[NV];
@@ -196,6 +207,7 @@ __device__ __forceinline__ void fht_rows_xl(float (&v)[FhtCfg<LOGD>::NJ][4], int
             }
 #pragma unroll
     for (int k = 0; k < NV; ++k) col[STEP * k] = w[k];
+    wave_lds_handover();
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
         const float4 t = *reinterpret_cast<const float4 *>(wl + BLOCK * j + 4 * lr);

@@ -242,6 +242,8 @@ extern "C" int lffn_layer_norm_bwd_noalloc_f32(const float *x, const float *ln_w
                                                float *g_x, float *g_weight, float *g_bias, int64_t B, int64_t H,
                                                int64_t R, void *stream) {
     LFFN_REQUIRE(B >= 0 && H >= 1, LFFN_ERR_BAD_ARG);
+    // the array is sized for rows of up to 256 * NJ_MAX columns, whatever the number of rows
+    LFFN_REQUIRE(H <= 256 * NJ_MAX, LFFN_ERR_SCRATCH);
     // as many partials as workgroups that have a row, at most LN_NOALLOC_PARTIALS
     const int64_t want = (B + 3) / 4;
     const int64_t num_partials = want < 1 ? 1 : (want > LN_NOALLOC_PARTIALS ? LN_NOALLOC_PARTIALS : want);

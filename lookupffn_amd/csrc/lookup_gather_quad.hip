@@ -281,7 +281,10 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
     // A pair's records: x, y = the scores and z = the row numbers (first | second << 8), in the order the
     // quad takes the pair's tables.  They sit in this wavefront's own corner of LDS and it has just waited
     // for its own copies, so they are read BEFORE the barrier: their latency is out of the way when the
-    // barrier opens and the first row reads go out at once.
+    // barrier opens and the first row reads go out at once.  (The copies are inline assembly: the compiler
+    // does not know that they write LDS nor that the wait is what completes them, so an ordering point it
+    // does honour keeps the reads below the wait.)
+    asm volatile("" ::: "memory");
     LdsRecord rec0 = read_record<WAVE_RECS>(rec_read0);
     LdsRecord rec1 = read_record<WAVE_RECS>(rec_read1);
     __syncthreads();
@@ -360,7 +363,9 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
         for (int i = 0; i < 4; ++i) base[i] ^= (unsigned)BUF_BYTES;
         // the copies issued above have landed (records and segments); the touch, issued after them, may still be out
         __builtin_amdgcn_s_waitcnt(TOUCH ? WAIT_VMCNT_1 : WAIT_VMCNT_0);
-        // the next pair's records (this wavefront's own, just landed), then the barrier for the segments
+        // the next pair's records (this wavefront's own, just landed; kept below the wait by the ordering
+        // point), then the barrier for the segments
+        asm volatile("" ::: "memory");
         rec0 = read_record<WAVE_RECS>(rec_read0);
         rec1 = read_record<WAVE_RECS>(rec_read1);
         __syncthreads();

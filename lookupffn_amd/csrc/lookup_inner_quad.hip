@@ -116,6 +116,7 @@ __device__ __forceinline__ float dot4(const float4 &g, const u32x4 &v, float acc
 template <int NP, int C>
 __global__ __launch_bounds__(WG) void lookup_inner_quad_kernel(InnerQuadArgs a) {
     static_assert(NP >= 4 && NP <= 8, "lane l of a quad holds the row numbers of passes l and l + 4");
+    static_assert(1 + 2 * NP <= 15, "the wait before the barrier names 1 + 2*NP operations in the 4-bit vmcnt field");
     // (NP = 4 is what is built: 6 and 8 passes need more than the 128 registers of a 16-wavefront workgroup)
     static_assert(C >= 1 && C <= 4, "row numbers of a chunk: two registers per lane");
     constexpr int W = (C + 1) / 2;                // words of row numbers per pass: two pairs (4 bytes) a word
@@ -311,7 +312,9 @@ __global__ __launch_bounds__(WG) void lookup_inner_quad_kernel(InnerQuadArgs a) 
             // The copies and the touch came first, then the 2*NP loads of g, in that order: loads cannot move
             // below a statement that may write memory, and none of them can be merged or dropped.  With at
             // most 2*NP + 1 operations still out, the copies have landed (more operations than that, such as
-            // a register spill, only make the wait stricter).
+            // a register spill, only make the wait stricter; FEWER than 2*NP loads after the copies would
+            // leave a copy in flight at the barrier, which is why load_g issues exactly two loads per pass
+            // and this kernel must not spill: the test suite checks the compiler's resource report).
             asm volatile("" ::: "memory");
             __builtin_amdgcn_s_waitcnt(WAIT_VMCNT_0 | (1 + 2 * NP));
         } else {

@@ -400,6 +400,10 @@ class LookupFFN(nn.Module):
         are called without the operator dispatcher or autograd (same kernels, same results)."""
         x = x.contiguous()
         if residual is not None:
+            # forward() hands over fp32 of shape [tokens, output_size]; anything else is a caller's mistake
+            if (residual.dtype != torch.float32 or residual.device != x.device
+                    or tuple(residual.shape) != (x.shape[0], self.output_size)):
+                raise ValueError("residual: fp32 [tokens, output_size] on the input's device")
             residual = residual.contiguous()
         if st["one_launch"] and x.shape[0] <= self.FUSED_LAYER_MAX_TOKENS:
             # small batches: the whole layer in one launch

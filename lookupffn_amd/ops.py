@@ -741,14 +741,21 @@ def lookup_gather_records_plan(B, T, S, Do):
     return plan
 
 
+def _require(cond, what):
+    """Argument checks of the *_direct helpers (no operator dispatcher in front of them): a real exception,
+    also under ``python -O``."""
+    if not cond:
+        raise ValueError(what)
+
+
 def ln_project_hash_records_direct(x, ln_w, ln_b, eps, diag, pbias, T, decay, residual, plan):
     """LayerNorm + diagonal BH4 + mix + 8-bit hash of x [B, H], written as the record stream of `plan`
     (from lookup_gather_records_plan) instead of codes and scores.  The caller has checked the parameters
     (fp32, contiguous, on x's device)."""
-    assert x.dtype == torch.float32 and x.is_cuda and x.is_contiguous() and x.dim() == 2
+    _require(x.dtype == torch.float32 and x.is_cuda and x.is_contiguous() and x.dim() == 2, "x: contiguous fp32 [B, H] on the GPU")
     B, H = x.shape
     R, J, D = diag.shape
-    assert H == ln_w.numel() and T * 8 <= R * D and T % 2 == 0 and plan[1] >= B
+    _require(H == ln_w.numel() and T * 8 <= R * D and T % 2 == 0 and plan[1] >= B, "shapes do not fit the record plan")
     records = torch.empty(plan[2] // 4, dtype=torch.int32, device=x.device)
     with _dev_guard(x):
         rc = _lib.load().lffn_ln_project_hash_records_f32(
@@ -761,11 +768,11 @@ def ln_project_hash_records_direct(x, ln_w, ln_b, eps, diag, pbias, T, decay, re
 
 def ln_bh4_block_hash_records_direct(x, ln_w, ln_b, eps, w_folded, pbias, T, decay, residual, plan):
     """The same for BH4 with 64 x 64 blocks (folded weights [R, J, D/64, 64, 64]) on the matrix cores."""
-    assert x.dtype == torch.float32 and x.is_cuda and x.is_contiguous() and x.dim() == 2
+    _require(x.dtype == torch.float32 and x.is_cuda and x.is_contiguous() and x.dim() == 2, "x: contiguous fp32 [B, H] on the GPU")
     B, H = x.shape
     R, J, NB, bs, _ = w_folded.shape
     D = NB * bs
-    assert H == ln_w.numel() and T * 8 <= R * D and T % 2 == 0 and plan[1] >= B
+    _require(H == ln_w.numel() and T * 8 <= R * D and T % 2 == 0 and plan[1] >= B, "shapes do not fit the record plan")
     records = torch.empty(plan[2] // 4, dtype=torch.int32, device=x.device)
     with _dev_guard(x):
         rc = _lib.load().lffn_ln_bh4_block_hash_records_f32(
@@ -779,8 +786,11 @@ def ln_bh4_block_hash_records_direct(x, ln_w, ln_b, eps, w_folded, pbias, T, dec
 def lookup_gather_records_direct(records, plan, tables, bias, residual, B):
     """out[b] = residual[b] + bias + sum_t score * row, from the record stream written for `plan`."""
     T, S, Do = tables.shape
-    assert tables.dtype == torch.float32 and tables.is_contiguous() and records.numel() * 4 >= plan[2]
-    assert residual is None or (residual.dtype == torch.float32 and residual.is_contiguous() and tuple(residual.shape) == (B, Do))
+    _require(tables.dtype == torch.float32 and tables.is_contiguous() and records.numel() * 4 >= plan[2],
+             "tables: contiguous fp32; records: at least the plan's bytes")
+    _require(residual is None or (residual.dtype == torch.float32 and residual.is_contiguous()
+                                  and residual.device == tables.device and tuple(residual.shape) == (B, Do)),
+             "residual: contiguous fp32 [B, Do] on the tables' device")
     out = torch.empty(B, Do, dtype=torch.float32, device=tables.device)
     with _dev_guard(tables):
         rc = _lib.load().lffn_lookup_gather_records_f32(

@@ -85,6 +85,65 @@ def test_layer_forward_eval_matches_oracle(H, T, Do, bs):
         assert (err <= 2e-5).all()
 
 
+# (tokens as batch x sequence, hidden, tables, columns, block size): BASELINE.json configs 2 and 3, and config 2 with the
+# reference's shipped block size; all take the many-token path (projection kernel writing the record stream,
+# four-lanes-per-token gather)
+MANY_TOKEN_LAYERS = [((32, 512), 768, 128, 768, 1), ((32, 512), 1024, 512, 1024, 1), ((32, 512), 768, 128, 768, 64)]
+
+
+@pytest.mark.parametrize("shape,H,T,Do,bs", MANY_TOKEN_LAYERS)
+def test_layer_forward_eval_many_tokens_matches_oracle(shape, H, T, Do, bs):
+    """LookupFFN.eval() at 16384 tokens: the record-stream path of LookupFFN._forward_inference, on a sample of
+    tokens against the oracle."""
+    from lookupffn_amd import ops
+    torch.manual_seed(H + T + bs)
+    S = 256
+    layer = lookupffn_amd.LookupFFN(_config(hidden_size=H, ffn_num_table=T, block_size=bs), Do).eval().to(DEV)
+    with torch.no_grad():
+        layer.hash.projection.bias.normal_(0, 0.05)
+    B = shape[0] * shape[1]
+    assert ops.lookup_gather_records_plan(B, T, S, Do) is not None         # this shape takes the record stream
+    x = torch.randn(*shape, H, device=DEV) * 1.5 + 0.3
+    with torch.no_grad():
+        out = layer(x)
+        again = layer(x)
+    assert out.shape == (*shape, Do) and torch.equal(out, again)
+    out = npf(out).reshape(B, Do)
+    assert not np.isnan(out).any()
+    rng = np.random.RandomState(5)
+    sub = np.unique(np.concatenate([rng.choice(B, 150, replace=False), np.arange(B - 40, B), np.arange(0, 8)]))
+    xs = x.reshape(B, H)[torch.as_tensor(sub, device=DEV)].contiguous()
+    with torch.no_grad():
+        h = layer.LayerNorm(xs)
+        # the front-end kernel's own codes and scores for these rows (a row's result does not depend on the batch)
+        if bs == 1:
+            code_k, score_k = layer.hash.forward_fused(xs, layer_norm=layer.LayerNorm)
+        else:
+            code_k, score_k = layer.hash.forward_block(xs, layer_norm=layer.LayerNorm)
+    code_k, score_k = npf(code_k).astype(np.int32), npf(score_k)
+    # the oracle from torch's LayerNorm output: codes agree except where z is within LayerNorm's rounding of zero
+    p = layer.hash.projection
+    z = oracle.projection(npf(h), npf(p.weight), npf(p.bias), T * 8, np.float32(p.decay_coeff))
+    code_o, score_o = oracle.code_score(z.reshape(-1, T, 8))
+    same = code_k == code_o
+    assert same.mean() > 0.999
+    np.testing.assert_allclose(score_k[same], score_o[same], rtol=2e-4)
+    # the layer's output = bias + the float64 sum over the kernel's own codes and scores ...
+    tables = npf(layer.tables).reshape(T * S, Do)
+
+    def gathered(code, score):
+        idx = code + (np.arange(T, dtype=np.int32) * S)[None]
+        uniq, inv = np.unique(idx, return_inverse=True)
+        return oracle.gather_add(inv.reshape(idx.shape).astype(np.int32), tables[uniq].astype(np.float64),
+                                 score.astype(np.float64)) + npf(layer.bias)
+    assert relmax(out[sub], gathered(code_k, score_k)) <= 1e-5
+    # ... and, for the tokens whose codes all agree, the oracle's own layer output
+    agree = same.all(axis=1)
+    assert agree.mean() > 0.5
+    want = gathered(code_o, score_o)
+    assert relmax(out[sub][agree], want[agree]) <= (2e-5 if bs == 1 else 1e-4)
+
+
 def test_training_path_matches_eval_path():
     torch.manual_seed(3)
     layer = lookupffn_amd.LookupFFN(_config(), 128).to(DEV)

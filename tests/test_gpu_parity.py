@@ -480,8 +480,13 @@ def test_ln_project_hash_matches_oracle(H, D, R, T):
 # (B, H, D, R, T, Do, forced plan or None): config 2's layer shape; a token count that ends inside a tile, a
 # workgroup of the projection kernel and a quad; two repeats of a short transform (rows shared by four
 # tokens per wavefront); an odd number of table pairs
+# what lffn_lookup_gather_records_plan picks at configs 2 and 3: (tokens per workgroup, record stride, bytes)
+CONFIG2_RECORD_PLAN = (1792, 17920, 6 * 128 * 17920)        # 10 tiles x 24 slices
+CONFIG3_RECORD_PLAN = (2048, 16384, 6 * 512 * 16384)        # 8 tiles x 32 slices
 RECORD_LAYERS = [(16384, 768, 1024, 1, 128, 768, None), (4099, 768, 1024, 1, 128, 768, (1024, 5120)),
-                 (5000, 100, 128, 2, 30, 128, (1536, 6144)), (2050, 64, 64, 1, 6, 64, (2048, 4096))]
+                 (5000, 100, 128, 2, 30, 128, (1536, 6144)), (2050, 64, 64, 1, 6, 64, (2048, 4096)),
+                 # config 3's layer shape (four repeats of the transform, 512 tables, 4 KB rows, 2048-token tiles)
+                 (4099, 1024, 1024, 4, 512, 1024, (2048, 6144))]
 
 
 @pytest.mark.parametrize("B,H,D,R,T,Do,plan", RECORD_LAYERS)
@@ -502,7 +507,7 @@ def test_layer_through_the_record_stream_matches_the_two_kernel_form(B, H, D, R,
     res = rng.randn(B, Do).astype(np.float32)
     if plan is None:
         plan = cabi.lookup_gather_records_plan(B, T, S, Do)[:2]
-        assert plan == (1792, 17920)                                            # config 2: 10 tiles x 24 slices
+        assert plan == CONFIG2_RECORD_PLAN[:2]
     tokens, stride = plan
     full_plan = (tokens, stride, 6 * T * stride)
     got, rec = cabi.layer_through_records(x, ln_w, ln_b, 1e-5, diag, pbias, tables, obias, residual=res, plan=full_plan)
@@ -564,8 +569,8 @@ def test_block_layer_through_the_record_stream(B, H, D, R, T, Do, tokens):
 def test_record_stream_plan_and_refusals():
     from lookupffn_amd import _lib
     lib = _lib.load()
-    assert cabi.lookup_gather_records_plan(16384, 128, 256, 768) == (1792, 17920, 6 * 128 * 17920)
-    assert cabi.lookup_gather_records_plan(16384, 512, 256, 1024) == (2048, 16384, 6 * 512 * 16384)
+    assert cabi.lookup_gather_records_plan(16384, 128, 256, 768) == CONFIG2_RECORD_PLAN
+    assert cabi.lookup_gather_records_plan(16384, 512, 256, 1024) == CONFIG3_RECORD_PLAN
     for shape in ((256, 32, 256, 256), (16384, 128, 128, 768), (16384, 127, 256, 768), (0, 128, 256, 768)):
         assert cabi.lookup_gather_records_plan(*shape) == (0, 0, 0), shape
     # (records, stride, tables, bias, residual, out, B, T, S, Do, tokens): refused before any launch
@@ -1431,6 +1436,38 @@ def test_config3_gather_full_size(config3, bf16):
     assert relmax(got.astype(np.float64).sum(0), want_sum) <= 1e-5
     # a second launch gives the same bits (fixed order of additions)
     assert np.array_equal(got, cabi.lookup_gather(c["code"], c["w"], src.reshape(T, S, Do), c["bias"], bf16=bf16))
+
+
+def test_config3_gather_record_stream_full_size(config3):
+    """Config 3 through the form the layer and bench.py run there: lffn_lookup_gather_ws_f32 packs the record
+    stream and launches the four-lanes-per-token kernel (2048-token tiles, 256 table pairs, 4 KB rows)."""
+    c = config3
+    B, T, S, Do = c["B"], c["T"], c["S"], c["Do"]
+    nbytes = cabi.lookup_gather_workspace_bytes(B, T, S, Do)
+    assert nbytes > 0 and nbytes % 12 == 0 and nbytes < B * Do * 4            # the record stream, not the table split
+    assert cabi.lookup_gather_records_plan(B, T, S, Do) == CONFIG3_RECORD_PLAN
+    flat = c["tables"].reshape(T * S, Do)
+    got = cabi.lookup_gather_ws(c["code"], c["w"], c["tables"], c["bias"])
+    assert not np.isnan(got).any()
+    sub = c["sub"]
+    rows, ridx = _rows64(flat, c["idx"][sub])
+    want = oracle.gather_add(ridx, rows, c["w"][sub].astype(np.float64)) + c["bias"]
+    assert relmax(got[sub], want) <= 1e-5
+    # every token against the plain entry point (same rows; the two tables of a pair added in either order)
+    assert relmax(got, cabi.lookup_gather(c["code"], c["w"], c["tables"], c["bias"])) <= 2e-6
+    # checksum over all tokens: sum_b out[b] = B * bias + sum_{t,s} cnt[t,s] * tables[t,s]
+    want_sum = B * c["bias"].astype(np.float64)
+    for t0 in range(0, T, 64):
+        want_sum = want_sum + np.einsum("ts,tsd->d", c["cnt"][t0:t0 + 64], flat[t0 * S:(t0 + 64) * S].reshape(64, S, Do).astype(np.float64))
+    assert relmax(got.astype(np.float64).sum(0), want_sum) <= 1e-5
+    # a second launch gives the same bits; so does the same tile size named explicitly
+    assert np.array_equal(got, cabi.lookup_gather_ws(c["code"], c["w"], c["tables"], c["bias"]))
+    rc, forced = cabi.lookup_gather_ws_planned(c["code"], c["w"], c["tables"], (3, CONFIG3_RECORD_PLAN[0]), bias=c["bias"])
+    assert rc == 0 and np.array_equal(got, forced)
+    # the residual goes into the store: the same sums plus the residual, rounded once more
+    res = np.random.default_rng(36).standard_normal((B, Do), dtype=np.float32)
+    got_r = cabi.lookup_gather_ws(c["code"], c["w"], c["tables"], c["bias"], residual=res)
+    assert np.array_equal(got_r, got + res)
 
 
 def test_config3_inner_product_full_size(config3):

@@ -72,6 +72,10 @@ def test_layer_norm_bwd_noalloc_rejects_what_the_buffer_cannot_hold():
                                              2048, 2048, 1, None)
     assert rc == _lib.LFFN_ERR_SCRATCH
     assert b"scratch" in lib.lffn_error_string(rc)
+    # ... also with so few rows that their partial sums alone would fit
+    rc = lib.lffn_layer_norm_bwd_noalloc_f32(t.data_ptr(), None, 1e-5, t.data_ptr(), t.data_ptr(), o.data_ptr(), o.data_ptr(),
+                                             8, 2048, 1, None)
+    assert rc == _lib.LFFN_ERR_SCRATCH
     # an empty batch: zeros for the parameter gradients
     gw = torch.full((64,), float("nan"), device=DEV)
     gb = torch.full((64,), float("nan"), device=DEV)
