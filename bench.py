@@ -49,6 +49,10 @@ WORKLOADS = {
                  desc="config 3: 16384 tokens, d=1024, 512 tables x 256 x 1024 fp32"),
     "cfg3bf16": dict(B=16384, H=1024, T=512, S=256, Do=1024, bf16=True,
                      desc="config 3: 16384 tokens, d=1024, 512 tables x 256 x 1024 bf16 rows, fp32 accumulate"),
+    # config 3 with half rows: the row format of the reference's own reduced-precision gather
+    # (PL/gather/cuda/extension/gather_kernel_fp16.cu), fp32 accumulate here
+    "cfg3f16": dict(B=16384, H=1024, T=512, S=256, Do=1024, bf16=False, f16=True,
+                    desc="config 3: 16384 tokens, d=1024, 512 tables x 256 x 1024 half (fp16) rows, fp32 accumulate"),
     # config 2 with the 64 x 64 block-diagonal BH4 the reference's training configs use
     # (cfgs/roberta/small-512/lookup-t128-s8-bh4.py:25-26) instead of the sign diagonal
     "cfg2b64": dict(B=16384, H=768, T=128, S=256, Do=768, bf16=False, bs=64,
@@ -95,25 +99,31 @@ def measured_traffic(workload, form):
     return rec["bytes"] if rec and rec["form"] == form else None
 
 
-def gather_form(B, T, S, Do, bf16):
-    """Which gather kernel the library runs for a shape, as a short string (host-side queries only)."""
+def row_format(wl):
+    """The C ABI's row_format of a workload's tables: 0 fp32, 1 bfloat16, 2 half."""
+    return 1 if wl["bf16"] else (2 if wl.get("f16") else 0)
+
+
+def gather_form(B, T, S, Do, fmt):
+    """Which gather kernel the layer runs for a shape and row format, as a short string (host-side queries only)."""
     import ctypes
 
     from lookupffn_amd import _lib
     lib = _lib.load()
-    if not bf16:
-        tok, stride, nbytes = ctypes.c_int32(0), ctypes.c_int64(0), ctypes.c_int64(0)
-        _lib.check(lib.lffn_lookup_gather_records_plan(B, T, S, Do, ctypes.byref(tok), ctypes.byref(stride), ctypes.byref(nbytes)),
-                   "records plan")
-        if nbytes.value > 0:
-            return f"record stream (four lanes per token), {tok.value} tokens per workgroup"
+    tok, stride, nbytes = ctypes.c_int32(0), ctypes.c_int64(0), ctypes.c_int64(0)
+    _lib.check(lib.lffn_lookup_gather_records_plan_rows(B, T, S, Do, fmt, ctypes.byref(tok), ctypes.byref(stride),
+                                                        ctypes.byref(nbytes)), "records plan")
+    if nbytes.value > 0:
+        return f"record stream (four lanes per token), {tok.value} tokens per workgroup"
     ws = ctypes.c_int64(0)
-    _lib.check(lib.lffn_lookup_gather_workspace_bytes(B, T, S, Do, int(bf16), ctypes.byref(ws)), "workspace query")
-    kind = ctypes.c_int32(-1)
-    tokens = lib.lffn_lookup_gather_plan(B, T, S, Do, int(bf16), ctypes.byref(kind))
-    if ws.value > 0:
+    _lib.check(lib.lffn_lookup_gather_workspace_bytes(B, T, S, Do, fmt, ctypes.byref(ws)), "workspace query")
+    form = ctypes.c_int32(-1)
+    tokens = lib.lffn_lookup_gather_ws_plan(B, T, S, Do, fmt, ws.value, ctypes.byref(form))
+    if form.value == 4:
         return "table split"
-    return "token-major" if kind.value == 0 else f"{kind.value} table(s) per LDS buffer, {tokens} tokens per workgroup"
+    if form.value == 3:
+        return f"record stream (four lanes per token), {tokens} tokens per workgroup"
+    return "token-major" if form.value == 0 else f"{form.value} table(s) per LDS buffer, {tokens} tokens per workgroup"
 
 
 def build_layer(wl, device):
@@ -141,6 +151,8 @@ def build_layer(wl, device):
     layer = layer.to(device)
     if wl["bf16"]:
         layer.tables.data = layer.tables.data.to(torch.bfloat16)
+    elif wl.get("f16"):
+        layer.tables.data = layer.tables.data.to(torch.float16)
     return layer, x
 
 
@@ -172,7 +184,7 @@ def cpu_baseline(layer, x, wl, budget_s=12.0):
     out = {"value": n * reps / t_total, "unit": "tokens/s", "cores": oracle.num_threads(), "kind": "port",
            "cpu_model": cpu_model,
            "sample": f"first {n} of {wl['B']} tokens, full tables, {reps} passes of the OpenMP C oracle "
-                     f"(whole layer, fp32{' on bf16-rounded tables' if wl['bf16'] else ''}), {t_total:.1f} s"}
+                     f"(whole layer, fp32{' on the 16-bit-rounded tables' if row_format(wl) else ''}), {t_total:.1f} s"}
     # the reference's own x86 kernels (compiled from its sources), gather + code/score legs only
     try:
         import torch
@@ -480,7 +492,8 @@ def main():
     B, H, T, S, Do = wl["B"], wl["H"], wl["T"], wl["S"], wl["Do"]
     layer, x_cpu = build_layer(wl, dev)
     x = x_cpu.to(dev)
-    esz = 2 if wl["bf16"] else 4
+    fmt = row_format(wl)
+    esz = 2 if fmt else 4
     gather_bytes = B * T * Do * esz + B * T * 8 + B * Do * 4
 
     block = layer.hash.projection.block_size != 1
@@ -497,8 +510,8 @@ def main():
     # many tokens, diagonal BH4, fp32 tables: the projection kernel writes the gather's record stream itself
     st = layer._inference_state()
     rec_plan = None
-    if not fused_layer and not wl["bf16"] and T % 2 == 0 and st is not None:
-        rec_plan = ops.lookup_gather_records_plan(B, T, S, Do)
+    if not fused_layer and T % 2 == 0 and st is not None:
+        rec_plan = ops.lookup_gather_records_plan(B, T, S, Do, fmt)
 
     def records_front():
         if block:
@@ -584,7 +597,7 @@ def main():
     logical_gbps = gather_bytes / (gather_ms * 1e-3) / 1e9
     row_bytes = B * T * Do * esz                                          # one row per (token, table)
     compulsory = T * S * Do * esz + B * T * 8 + B * Do * 4                # tables, codes + scores, output: each once
-    form = "whole layer in one launch (rows from L2)" if fused_layer else gather_form(B, T, S, Do, wl["bf16"])
+    form = "whole layer in one launch (rows from L2)" if fused_layer else gather_form(B, T, S, Do, fmt)
     lds_bound = not fused_layer and form != "token-major"
     traffic = measured_traffic(args.workload, form)
     hbm = {"compulsory_bytes": compulsory, "frac_of_peak": compulsory / (gather_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
@@ -659,7 +672,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16 rows, f32 accumulate" if wl["bf16"] else "f32",
+        "dtype": ("f32", "bf16 rows, f32 accumulate", "f16 rows, f32 accumulate")[fmt],
         "data": ("synthetic (seeded N(0,1) tokens, N(0,1)/sqrt(64 D) block weights, N(0,0.02) tables)" if block else
                  "synthetic (seeded N(0,1) tokens, seeded +-1/sqrt(D) sign diagonals, N(0,0.02) tables)"),
         "config": {"workload": wl["desc"], "tokens": B, "d_model": H, "fht_dim": layer.hash.projection.padded_in_dim,

@@ -41,7 +41,7 @@ extern "C" {
 #define LFFN_ERR_LAUNCH      -3   /* hipGetLastError() after the launch was not hipSuccess */
 #define LFFN_ERR_SCRATCH     -4   /* an entry point that allocates nothing: the shape exceeds its static scratch */
 
-#define LFFN_ABI_VERSION 5
+#define LFFN_ABI_VERSION 6
 
 /* ABI version of the loaded library (LFFN_ABI_VERSION at build time). */
 int lffn_version(void);
@@ -340,8 +340,13 @@ int lffn_ln_project_hash_f32(const float *x, const float *ln_weight, const float
  * from such a stream, with the tokens_per_workgroup and record_stride the plan gave.  Results are
  * bit-identical to lffn_lookup_gather_ws_f32's for the same shape.  bias and residual may be NULL.
  *
+ * lffn_lookup_gather_records_plan_rows / lffn_lookup_gather_records_rows: the same two calls for any
+ * row format (row_format 0 fp32, 1 bfloat16, 2 half; tables typed accordingly).  16-bit rows run 1024
+ * tokens per workgroup over 64-column slices, fp32 sums.  The records do not depend on the row format.
+ *
  * Replaces the same reference code as lffn_ln_project_hash_f32 followed by lffn_lookup_gather_f32
- * (PL/lookup.py:29-39,64-77,99 and 120-130,108).
+ * (PL/lookup.py:29-39,64-77,99 and 120-130,108); with half rows, the gather of
+ * PL/gather/cuda/extension/gather_kernel_fp16.cu:6-62 (fp32 sums instead of its half sums).
  */
 int lffn_lookup_gather_records_plan(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t *tokens_per_workgroup,
                                     int64_t *record_stride, int64_t *bytes);
@@ -358,6 +363,12 @@ int lffn_ln_bh4_block_hash_records_f32(const float *x, const float *ln_weight, c
 int lffn_lookup_gather_records_f32(const uint32_t *records, int64_t record_stride, const float *tables,
                                    const float *bias, const float *residual, float *out, int64_t B, int64_t T,
                                    int64_t S, int64_t Do, int32_t tokens_per_workgroup, void *stream);
+int lffn_lookup_gather_records_plan_rows(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t row_format,
+                                         int32_t *tokens_per_workgroup, int64_t *record_stride, int64_t *bytes);
+int lffn_lookup_gather_records_rows(const uint32_t *records, int64_t record_stride, const void *tables,
+                                    const float *bias, const float *residual, float *out, int64_t B, int64_t T,
+                                    int64_t S, int64_t Do, int32_t row_format, int32_t tokens_per_workgroup,
+                                    void *stream);
 
 /* ---------------------------------------------------------------- code + score */
 
@@ -401,6 +412,15 @@ int lffn_gather_add_bf16(const int32_t *idx, const uint16_t *src, const float *w
                          int64_t B, int64_t I, int64_t source_size, int64_t Dv, void *stream);
 
 /*
+ * The same with half rows (IEEE binary16), fp32 sums.  Replaces
+ * gather_add.weighted_vector_gather_add_fp16 (PL/gather/cuda/extension/gather_kernel_fp16.cu:6-62),
+ * which multiplies and accumulates in half (__hfma2, :56-57): the results here are the fp32 sums of
+ * the same products, i.e. closer to the exact sum than the reference's, not bit-identical to it.
+ */
+int lffn_gather_add_f16(const int32_t *idx, const uint16_t *src, const float *w, float *out,
+                        int64_t B, int64_t I, int64_t source_size, int64_t Dv, void *stream);
+
+/*
  * The gather as LookupFFN.gather issues it (PL/lookup.py:120-130): one index per
  * table, idx[b,t] = code[b,t] + t*S folded in, optional bias (PL/lookup.py:108):
  *   out[b,:] = bias + sum_t score[b,t] * tables[t, code[b,t] & (S-1), :]
@@ -434,8 +454,9 @@ int lffn_lookup_gather_residual_bf16(const int32_t *code, const float *score, co
 
 /*
  * The same gather with a caller-provided workspace, which two forms use:
- *  - many tokens, fp32 rows, S = 256, an even number of tables (16384 tokens at the RoBERTa-base
- *    tables): the four-lanes-per-token kernel.  A small kernel first packs the (code, score) pairs
+ *  - many tokens, S = 256, an even number of tables (16384 tokens at the RoBERTa-base tables): the
+ *    four-lanes-per-token kernel (fp32, bfloat16 and half rows; 128-byte column slices = 32 fp32 or
+ *    64 16-bit columns).  A small kernel first packs the (code, score) pairs
  *    into a stream of 12-byte records in the workspace (6 bytes per (token, table)), one row of
  *    records per table pair, which the gather kernel copies into LDS a pair ahead; the gather
  *    kernel walks 128-byte column slices, two tables per LDS buffer, 1024 to 2048 tokens per
@@ -448,20 +469,32 @@ int lffn_lookup_gather_residual_bf16(const int32_t *code, const float *score, co
  *    the partials, in table order, with bias and residual (reproducible, and equal to the one-part
  *    kernel's up to the association of the fp32 sums).
  * lffn_lookup_gather_workspace_bytes sets *bytes to the workspace that pays for a shape, or to 0
- * when the plain entry points are as fast (very few tokens, bf16 rows at 16384 tokens and more,
- * tables beyond the 256 MB memory-side cache); with a null or too small workspace the _ws entry
- * points behave exactly like lffn_lookup_gather_residual_*.  The workspace is scratch: 16-byte
+ * when the plain entry points are as fast (very few tokens); row_format is 0 (fp32 rows), 1
+ * (bfloat16) or 2 (half).  With a null or too small workspace the _ws entry points behave exactly
+ * like lffn_lookup_gather_residual_* (half rows: the token-major kernel).  lffn_lookup_gather_ws_plan
+ * reports which kernel the _ws entry points run for a shape and a workspace size: the return value
+ * is the tokens per workgroup (0: token-major) and *form (may be NULL) receives 0 (token-major), 1 or
+ * 2 (tables per LDS buffer, as lffn_lookup_gather_plan), 3 (four lanes per token, record stream in
+ * the workspace) or 4 (table split, partial outputs in the workspace); a batch taken in pieces
+ * reports the form of a piece.  Pure host functions.
+ * lffn_lookup_gather_ws_f16: half rows (the row format of the reference's reduced-precision gather,
+ * gather_kernel_fp16.cu:6-62, with fp32 sums instead of its half sums): form 3 or token-major.  The workspace is scratch: 16-byte
  * aligned device memory, contents undefined afterwards; calls that share one must be ordered on
  * the stream.  residual may be null.
  * Same replacement as lffn_lookup_gather_f32 (PL/lookup.py:120-130, 108).
  */
-int lffn_lookup_gather_workspace_bytes(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t bf16, int64_t *bytes);
+int lffn_lookup_gather_workspace_bytes(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t row_format, int64_t *bytes);
 int lffn_lookup_gather_ws_f32(const int32_t *code, const float *score, const float *tables, const float *bias,
                               const float *residual, float *out, void *workspace, int64_t workspace_bytes,
                               int64_t B, int64_t T, int64_t S, int64_t Do, void *stream);
 int lffn_lookup_gather_ws_bf16(const int32_t *code, const float *score, const uint16_t *tables, const float *bias,
                                const float *residual, float *out, void *workspace, int64_t workspace_bytes,
                                int64_t B, int64_t T, int64_t S, int64_t Do, void *stream);
+int lffn_lookup_gather_ws_f16(const int32_t *code, const float *score, const uint16_t *tables, const float *bias,
+                              const float *residual, float *out, void *workspace, int64_t workspace_bytes,
+                              int64_t B, int64_t T, int64_t S, int64_t Do, void *stream);
+int lffn_lookup_gather_ws_plan(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t row_format,
+                               int64_t workspace_bytes, int32_t *form);
 
 /*
  * Which kernel lffn_lookup_gather_{f32,bf16} runs for a shape.  Returns the number
@@ -469,9 +502,9 @@ int lffn_lookup_gather_ws_bf16(const int32_t *code, const float *score, const ui
  * tables through LDS, or 0 when the token-major kernel is used (small batches,
  * S > 256); *tables_per_buffer (may be NULL) receives 0 (token-major), 1 (256-byte
  * column slices, one table per LDS buffer) or 2 (128-byte slices, two tables per
- * buffer).  (The workspace entry points may run a form this function does not report:
- * 3, the four-lanes-per-token kernel.)  Pure host function, no GPU work; negative on
- * bad arguments.
+ * buffer).  The workspace entry points may run forms this function does not report
+ * (3, the four-lanes-per-token kernel, and the table split): lffn_lookup_gather_ws_plan
+ * reports those.  Pure host function, no GPU work; negative on bad arguments.
  * No counterpart in the reference (its gather has one kernel, gather_fp32.cu:6-36).
  */
 int lffn_lookup_gather_plan(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t bf16,
@@ -489,6 +522,9 @@ int lffn_lookup_gather_plan(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t
  * form 3, the four-lanes-per-token kernel (tokens_per_workgroup 1024, 1536, 1792 or
  * 2048; S = 256, T even, Do a multiple of 32; the workspace must hold the record
  * stream, 6 * T * (B + 2048) bytes, or the call is refused with LFFN_ERR_UNSUPPORTED).
+ * lffn_lookup_gather_ws_planned_rows is the same for any row format (row_format 0 fp32,
+ * 1 bfloat16, 2 half; tables typed accordingly): 16-bit rows take form 3 with 1024
+ * tokens per workgroup and Do a multiple of 64; half rows take forms 0 and 3 only.
  * No counterpart in the reference.
  */
 int lffn_lookup_gather_planned_f32(const int32_t *code, const float *score, const float *tables,
@@ -503,6 +539,11 @@ int lffn_lookup_gather_planned_bf16(const int32_t *code, const float *score, con
                                     const float *bias, float *out,
                                     int64_t B, int64_t T, int64_t S, int64_t Do,
                                     int32_t tables_per_buffer, int32_t tokens_per_workgroup, void *stream);
+int lffn_lookup_gather_ws_planned_rows(const int32_t *code, const float *score, const void *tables,
+                                       const float *bias, const float *residual, float *out, void *workspace,
+                                       int64_t workspace_bytes, int64_t B, int64_t T, int64_t S, int64_t Do,
+                                       int32_t row_format, int32_t tables_per_buffer, int32_t tokens_per_workgroup,
+                                       void *stream);
 
 /*
  * out[b,i] = <g[b,:], src[idx[b,i],:]>   (gradient w.r.t. the weights).

@@ -15,7 +15,7 @@ _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 # LOOKUPFFN_HIP_LIB points at another build of the same ABI (e.g. a tuning build)
 LIB_PATH = os.environ.get("LOOKUPFFN_HIP_LIB") or os.path.join(_PKG_DIR, "liblookupffn_hip.so")
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 LFFN_OK = 0
 LFFN_ERR_BAD_ARG = -1
@@ -61,6 +61,7 @@ SIGNATURES = {
     "lffn_code_score_bwd_f32": [_vp, _vp, _vp, _i64, _i64, _vp],
     "lffn_gather_add_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "lffn_gather_add_bf16": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
+    "lffn_gather_add_f16": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "lffn_lookup_gather_f32": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "lffn_lookup_gather_bf16": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "lffn_lookup_gather_residual_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
@@ -72,11 +73,18 @@ SIGNATURES = {
     "lffn_lookup_gather_workspace_bytes": [_i64, _i64, _i64, _i64, ctypes.c_int32, ctypes.POINTER(ctypes.c_int64)],
     "lffn_lookup_gather_ws_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp],
     "lffn_lookup_gather_ws_bf16": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp],
+    "lffn_lookup_gather_ws_f16": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp],
+    "lffn_lookup_gather_ws_plan": [_i64, _i64, _i64, _i64, ctypes.c_int32, _i64, ctypes.POINTER(ctypes.c_int32)],
+    "lffn_lookup_gather_ws_planned_rows": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, ctypes.c_int32,
+                                           ctypes.c_int32, ctypes.c_int32, _vp],
     "lffn_lookup_gather_ws_planned_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, ctypes.c_int32, ctypes.c_int32, _vp],
     "lffn_ln_project_hash_records_f32": [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _vp],
     "lffn_ln_bh4_block_hash_records_f32": [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _vp],
     "lffn_lookup_gather_records_plan": [_i64, _i64, _i64, _i64, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64)],
     "lffn_lookup_gather_records_f32": [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, ctypes.c_int32, _vp],
+    "lffn_lookup_gather_records_plan_rows": [_i64, _i64, _i64, _i64, ctypes.c_int32, ctypes.POINTER(ctypes.c_int32),
+                                             ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64)],
+    "lffn_lookup_gather_records_rows": [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, ctypes.c_int32, ctypes.c_int32, _vp],
     "lffn_lookup_gather_plan": [_i64, _i64, _i64, _i64, ctypes.c_int32, ctypes.POINTER(ctypes.c_int32)],
     "lffn_indexed_inner_product_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "lffn_scatter_add_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],

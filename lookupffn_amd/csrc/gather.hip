@@ -25,15 +25,27 @@ namespace {
 constexpr int IC = 64;      // (index, weight) pairs staged per token per pass
 constexpr int UNROLL = 8;   // rows in flight per lane group
 
-template <bool BF16>
+// FMT: the row format, LFFN_ROWS_F32 (0), LFFN_ROWS_BF16 (1) or LFFN_ROWS_F16 (2)
+template <int FMT>
 struct Row {
-    static constexpr int EPV = BF16 ? 8 : 4;   // elements per 16-byte vector
-    static constexpr int ESZ = BF16 ? 2 : 4;
+    static constexpr int EPV = FMT != LFFN_ROWS_F32 ? 8 : 4;   // elements per 16-byte vector
+    static constexpr int ESZ = FMT != LFFN_ROWS_F32 ? 2 : 4;
 };
 
-template <bool BF16>
-__device__ __forceinline__ void axpy_vec(float (&acc)[Row<BF16>::EPV], const uint4 &r, float w) {
-    if constexpr (BF16) {
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+template <int FMT>
+__device__ __forceinline__ void axpy_vec(float (&acc)[Row<FMT>::EPV], const uint4 &r, float w) {
+    if constexpr (FMT == LFFN_ROWS_F16) {
+        // (float)half * float + float: one v_fma_mix_f32 per value
+        const unsigned q[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const half2_t h = __builtin_bit_cast(half2_t, q[i]);
+            acc[2 * i] = fmaf((float)h.x, w, acc[2 * i]);
+            acc[2 * i + 1] = fmaf((float)h.y, w, acc[2 * i + 1]);
+        }
+    } else if constexpr (FMT == LFFN_ROWS_BF16) {
         acc[0] = fmaf(bf16_lo(r.x), w, acc[0]);
         acc[1] = fmaf(bf16_hi(r.x), w, acc[1]);
         acc[2] = fmaf(bf16_lo(r.y), w, acc[2]);
@@ -92,10 +104,10 @@ __device__ __forceinline__ void stage_pairs(const GatherArgs &a, int64_t tok0, i
     }
 }
 
-template <bool BF16, int LPT, int NV>
+template <int FMT, int LPT, int NV>
 __global__ __launch_bounds__(256) void gather_add_kernel(GatherArgs a) {
     constexpr int TPB = 256 / LPT;
-    constexpr int EPV = Row<BF16>::EPV;
+    constexpr int EPV = Row<FMT>::EPV;
     __shared__ int s_row[TPB][IC];
     __shared__ float s_w[TPB][IC];
 
@@ -104,7 +116,7 @@ __global__ __launch_bounds__(256) void gather_add_kernel(GatherArgs a) {
     const int64_t tok0 = int64_t(blockIdx.x) * TPB;
     const int64_t tok = tok0 + tl;
     const int vec0 = blockIdx.y * (LPT * NV) + ll;            // first 16-byte vector of this lane
-    const size_t row_bytes = size_t(a.Dv) * Row<BF16>::ESZ;
+    const size_t row_bytes = size_t(a.Dv) * Row<FMT>::ESZ;
     const char *base = static_cast<const char *>(a.src) + size_t(vec0) * 16;
 
     float acc[NV][EPV];
@@ -147,14 +159,14 @@ __global__ __launch_bounds__(256) void gather_add_kernel(GatherArgs a) {
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
-                for (int v = 0; v < NV; ++v) axpy_vec<BF16>(acc[v], r[u][v], wt[u]);
+                for (int v = 0; v < NV; ++v) axpy_vec<FMT>(acc[v], r[u][v], wt[u]);
         }
         for (; ii < n; ++ii) {
             const int row = s_row[tl][ii];
             const float wt = s_w[tl][ii];
             const uint4 *p = reinterpret_cast<const uint4 *>(base + size_t(row) * row_bytes);
 #pragma unroll
-            for (int v = 0; v < NV; ++v) axpy_vec<BF16>(acc[v], p[v * LPT], wt);
+            for (int v = 0; v < NV; ++v) axpy_vec<FMT>(acc[v], p[v * LPT], wt);
         }
     }
 
@@ -317,38 +329,38 @@ Tiling pick_tiling(int nvec) {
 
 enum class Op { Gather, Inner, Scatter };
 
-template <bool BF16, Op OP, int LPT, int NV>
+template <int FMT, Op OP, int LPT, int NV>
 void launch_one(const GatherArgs &a, const Tiling &t, hipStream_t s) {
     constexpr int TPB = 256 / LPT;
     const unsigned gx = (unsigned)((a.B + TPB - 1) / TPB);
     if constexpr (OP == Op::Gather)
-        hipLaunchKernelGGL((gather_add_kernel<BF16, LPT, NV>), dim3(gx, t.chunks), dim3(256), 0, s, a);
+        hipLaunchKernelGGL((gather_add_kernel<FMT, LPT, NV>), dim3(gx, t.chunks), dim3(256), 0, s, a);
     else if constexpr (OP == Op::Inner)
         hipLaunchKernelGGL((inner_product_kernel<LPT, NV>), dim3(gx), dim3(256), 0, s, a, t.chunks);
     else
         hipLaunchKernelGGL((scatter_add_kernel<LPT, NV>), dim3(gx, t.chunks), dim3(256), 0, s, a);
 }
 
-template <bool BF16, Op OP, int LPT>
+template <int FMT, Op OP, int LPT>
 void launch_nv(const GatherArgs &a, const Tiling &t, hipStream_t s) {
     switch (t.nv) {
-        case 1: launch_one<BF16, OP, LPT, 1>(a, t, s); break;
-        case 2: launch_one<BF16, OP, LPT, 2>(a, t, s); break;
-        case 3: launch_one<BF16, OP, LPT, 3>(a, t, s); break;
-        default: launch_one<BF16, OP, LPT, 4>(a, t, s); break;
+        case 1: launch_one<FMT, OP, LPT, 1>(a, t, s); break;
+        case 2: launch_one<FMT, OP, LPT, 2>(a, t, s); break;
+        case 3: launch_one<FMT, OP, LPT, 3>(a, t, s); break;
+        default: launch_one<FMT, OP, LPT, 4>(a, t, s); break;
     }
 }
 
-template <bool BF16, Op OP>
+template <int FMT, Op OP>
 int launch(const GatherArgs &a, hipStream_t s) {
     if (a.B == 0 || (a.I == 0 && OP != Op::Gather)) return LFFN_OK;
-    const Tiling t = pick_tiling(a.Dv / Row<BF16>::EPV);
+    const Tiling t = pick_tiling(a.Dv / Row<FMT>::EPV);
     switch (t.lpt) {
-        case 64: launch_nv<BF16, OP, 64>(a, t, s); break;
-        case 32: launch_nv<BF16, OP, 32>(a, t, s); break;
-        case 16: launch_nv<BF16, OP, 16>(a, t, s); break;
+        case 64: launch_nv<FMT, OP, 64>(a, t, s); break;
+        case 32: launch_nv<FMT, OP, 32>(a, t, s); break;
+        case 16: launch_nv<FMT, OP, 16>(a, t, s); break;
         default:
-            if constexpr (BF16) { launch_nv<BF16, OP, 8>(a, t, s); break; }
+            if constexpr (FMT != LFFN_ROWS_F32) { launch_nv<FMT, OP, 8>(a, t, s); break; }
             else return LFFN_ERR_UNSUPPORTED;
     }
     return lffn_launch_status();
@@ -364,7 +376,7 @@ int check_common(const void *idx, int64_t B, int64_t I, int64_t rows, int64_t Dv
     return LFFN_OK;
 }
 
-template <bool BF16>
+template <int FMT>
 int gather_entry(const int32_t *idx, const void *src, const float *w, const float *bias, const float *residual,
                  float *out,
                  int64_t B, int64_t I, int64_t rows, int64_t Dv, int64_t S, void *stream) {
@@ -375,19 +387,24 @@ int gather_entry(const int32_t *idx, const void *src, const float *w, const floa
     GatherArgs a{};
     a.idx = idx; a.src = src; a.w = w; a.g = nullptr; a.bias = bias; a.residual = residual; a.out = out;
     a.B = B; a.I = (int)I; a.source_size = rows; a.Dv = (int)Dv; a.S = (int)S;
-    return launch<BF16, Op::Gather>(a, static_cast<hipStream_t>(stream));
+    return launch<FMT, Op::Gather>(a, static_cast<hipStream_t>(stream));
 }
 
 }  // namespace
 
 extern "C" int lffn_gather_add_f32(const int32_t *idx, const float *src, const float *w, float *out,
                                    int64_t B, int64_t I, int64_t source_size, int64_t Dv, void *stream) {
-    return gather_entry<false>(idx, src, w, nullptr, nullptr, out, B, I, source_size, Dv, 0, stream);
+    return gather_entry<LFFN_ROWS_F32>(idx, src, w, nullptr, nullptr, out, B, I, source_size, Dv, 0, stream);
 }
 
 extern "C" int lffn_gather_add_bf16(const int32_t *idx, const uint16_t *src, const float *w, float *out,
                                     int64_t B, int64_t I, int64_t source_size, int64_t Dv, void *stream) {
-    return gather_entry<true>(idx, src, w, nullptr, nullptr, out, B, I, source_size, Dv, 0, stream);
+    return gather_entry<LFFN_ROWS_BF16>(idx, src, w, nullptr, nullptr, out, B, I, source_size, Dv, 0, stream);
+}
+
+extern "C" int lffn_gather_add_f16(const int32_t *idx, const uint16_t *src, const float *w, float *out,
+                                   int64_t B, int64_t I, int64_t source_size, int64_t Dv, void *stream) {
+    return gather_entry<LFFN_ROWS_F16>(idx, src, w, nullptr, nullptr, out, B, I, source_size, Dv, 0, stream);
 }
 
 // Token-major kernel on table-local codes (offset i*S and bias folded in): the
@@ -395,10 +412,11 @@ extern "C" int lffn_gather_add_bf16(const int32_t *idx, const uint16_t *src, con
 // built for.
 int lffn_internal_lookup_gather_token_major(const int32_t *code, const float *score, const void *tables,
                                             const float *bias, const float *residual, float *out, int64_t B,
-                                            int64_t T, int64_t S, int64_t Do, bool bf16, void *stream) {
+                                            int64_t T, int64_t S, int64_t Do, int fmt, void *stream) {
     const int64_t rows = T * S > 0 ? T * S : 1;
-    return bf16 ? gather_entry<true>(code, tables, score, bias, residual, out, B, T, rows, Do, S, stream)
-                : gather_entry<false>(code, tables, score, bias, residual, out, B, T, rows, Do, S, stream);
+    if (fmt == LFFN_ROWS_F16) return gather_entry<LFFN_ROWS_F16>(code, tables, score, bias, residual, out, B, T, rows, Do, S, stream);
+    return fmt == LFFN_ROWS_BF16 ? gather_entry<LFFN_ROWS_BF16>(code, tables, score, bias, residual, out, B, T, rows, Do, S, stream)
+                                 : gather_entry<LFFN_ROWS_F32>(code, tables, score, bias, residual, out, B, T, rows, Do, S, stream);
 }
 
 // Atomic scatter-add on table-local codes (row = code & (S-1) + t*S), into a buffer
@@ -408,7 +426,7 @@ int lffn_internal_lookup_scatter_atomic(const int32_t *code, const float *score,
     GatherArgs a{};
     a.idx = code; a.src = nullptr; a.w = score; a.g = g; a.bias = nullptr; a.out = out;
     a.B = B; a.I = (int)T; a.source_size = T * S; a.Dv = (int)Do; a.S = (int)S;
-    return launch<false, Op::Scatter>(a, static_cast<hipStream_t>(stream));
+    return launch<LFFN_ROWS_F32, Op::Scatter>(a, static_cast<hipStream_t>(stream));
 }
 
 // Token-major inner product on table-local codes: the fallback of lookup_inner.hip.
@@ -418,7 +436,7 @@ int lffn_internal_lookup_inner_token_major(const int32_t *code, const float *g, 
     GatherArgs a{};
     a.idx = code; a.src = tables; a.w = nullptr; a.g = g; a.bias = nullptr; a.out = out;
     a.B = B; a.I = (int)T; a.source_size = T * S; a.Dv = (int)Do; a.S = (int)S;
-    return launch<false, Op::Inner>(a, static_cast<hipStream_t>(stream));
+    return launch<LFFN_ROWS_F32, Op::Inner>(a, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int lffn_indexed_inner_product_f32(const int32_t *idx, const float *g, const float *src, float *out,
@@ -430,7 +448,7 @@ extern "C" int lffn_indexed_inner_product_f32(const int32_t *idx, const float *g
     GatherArgs a{};
     a.idx = idx; a.src = src; a.w = nullptr; a.g = g; a.bias = nullptr; a.out = out;
     a.B = B; a.I = (int)I; a.source_size = source_size; a.Dv = (int)Dv; a.S = 0;
-    return launch<false, Op::Inner>(a, static_cast<hipStream_t>(stream));
+    return launch<LFFN_ROWS_F32, Op::Inner>(a, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int lffn_scatter_add_f32(const int32_t *idx, const float *g, const float *w, float *out,
@@ -442,7 +460,7 @@ extern "C" int lffn_scatter_add_f32(const int32_t *idx, const float *g, const fl
     GatherArgs a{};
     a.idx = idx; a.src = nullptr; a.w = w; a.g = g; a.bias = nullptr; a.out = out;
     a.B = B; a.I = (int)I; a.source_size = out_size; a.Dv = (int)Dv; a.S = 0;
-    return launch<false, Op::Scatter>(a, static_cast<hipStream_t>(stream));
+    return launch<LFFN_ROWS_F32, Op::Scatter>(a, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int lffn_version(void) { return LFFN_ABI_VERSION; }

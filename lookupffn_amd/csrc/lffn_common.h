@@ -25,11 +25,14 @@ static inline int lffn_log2(int64_t v) {
     return l;
 }
 
-// gather.hip: token-major gather on table-local codes (not exported)
+// Row formats of the gather's tables: the values of the C ABI's row_format arguments.
+constexpr int LFFN_ROWS_F32 = 0, LFFN_ROWS_BF16 = 1, LFFN_ROWS_F16 = 2;
+
+// gather.hip: token-major gather on table-local codes (not exported); fmt is one of LFFN_ROWS_*
 __attribute__((visibility("hidden")))
 int lffn_internal_lookup_gather_token_major(const int32_t *code, const float *score, const void *tables,
                                             const float *bias, const float *residual, float *out, int64_t B,
-                                            int64_t T, int64_t S, int64_t Do, bool bf16, void *stream);
+                                            int64_t T, int64_t S, int64_t Do, int fmt, void *stream);
 
 // gather.hip: atomic scatter-add on table-local codes (not exported)
 __attribute__((visibility("hidden")))
@@ -78,11 +81,14 @@ static inline bool lffn_grant_dynamic_lds(const void *kernel, size_t lds_bytes, 
     return true;
 }
 
-// lookup_gather_quad.hip: the two-tables-per-buffer LDS gather with four lanes per token, fp32 rows (not exported)
+// lookup_gather_quad.hip: the two-tables-per-buffer LDS gather with four lanes per token (not exported);
+// fmt is one of LFFN_ROWS_*
 __attribute__((visibility("hidden")))
 int lffn_internal_lookup_gather_quad(const int32_t *code, const float *score, const void *tables,
                                      const float *bias, const float *residual, float *out, int64_t B, int64_t T,
-                                     int64_t S, int64_t Do, int np, void *workspace, void *stream);
+                                     int64_t S, int64_t Do, int fmt, int np, void *workspace, void *stream);
+__attribute__((visibility("hidden")))
+bool lffn_internal_quad_np_built(int fmt, int np);
 __attribute__((visibility("hidden")))
 int64_t lffn_internal_quad_stream_bytes(int64_t B, int64_t T);
 __attribute__((visibility("hidden")))
@@ -90,7 +96,7 @@ int64_t lffn_internal_quad_record_stride(int64_t B, int np);
 __attribute__((visibility("hidden")))
 int lffn_internal_lookup_gather_quad_records(const uint32_t *records, int64_t record_stride, const void *tables,
                                              const float *bias, const float *residual, float *out, int64_t B,
-                                             int64_t T, int64_t S, int64_t Do, int np, void *stream);
+                                             int64_t T, int64_t S, int64_t Do, int fmt, int np, void *stream);
 
 // lookup_inner_quad.hip: the score gradient with four lanes per token and one owner per (token, table) (not exported)
 __attribute__((visibility("hidden")))

@@ -351,10 +351,12 @@ struct GatherPlan {
 
 // The four-lanes-per-token kernel: microseconds per table pair of a workgroup = a fixed part (the 64 KB
 // copy, the records, the barrier) + a part per pass of 256 tokens.  Measured on MI355X at 4, 6, 7 and 8
-// passes: 1.40, 1.74, 1.93, 2.18 us, the same for 128 x 256 x 768 fp32 tables (in the memory-side
-// cache) and 512 x 256 x 1024 (537 MB, beyond it: the touch by turns hides the difference).
+// passes of fp32 rows: 1.40, 1.74, 1.93, 2.18 us, the same for 128 x 256 x 768 fp32 tables (in the memory-side
+// cache) and 512 x 256 x 1024 (537 MB, beyond it: the touch by turns hides the difference).  A pass over
+// 16-bit rows covers twice the columns and is bound by the vector ALU: QUAD_US_PER_PAIR_PASS_16[format].
 constexpr double QUAD_MARGIN = 0.92;      // the form must promise this much to be worth its workspace
 constexpr double QUAD_US_PER_PAIR = 0.62, QUAD_US_PER_PAIR_PASS = 0.195;
+constexpr double QUAD_US_PER_PAIR_PASS_16[3] = {0.0, 0.355, 0.26};     // indexed by LFFN_ROWS_*: bfloat16, half (measured at 4 passes)
 
 template <bool BF16>
 GatherPlan plan_gather(int64_t B, int64_t T, int64_t S, int64_t Do) {
@@ -390,20 +392,24 @@ GatherPlan plan_gather(int64_t B, int64_t T, int64_t S, int64_t Do) {
 
 // The four-lanes-per-token form (lookup_gather_quad.hip; needs a workspace for its record stream): 128-byte
 // slices, 256*np tokens per workgroup, one round of 256 workgroups costs T/2 pairs x the measured cost of a
-// pair at np passes; plus the packing kernel.  fp32 rows, 256-row tables and an even number of them only.
-template <bool BF16>
-GatherPlan plan_quad(int64_t B, int64_t T, int64_t S, int64_t Do) {
+// pair at np passes; plus the packing kernel when the records come from [B, T] codes and scores (`pack`).
+// 256-row tables and an even number of them only.
+GatherPlan plan_quad(int fmt, int64_t B, int64_t T, int64_t S, int64_t Do, bool pack = true) {
     GatherPlan best{0, 0, 1e300};
-    if (BF16 || S != MAX_S || T < 8 || T % 2 != 0 || T > (1 << 20) || Do % 32 != 0 || B * T >= (int64_t(1) << 31) ||
-        2 * S * Do * 4 >= (int64_t(1) << 32))
+    const int esz = fmt == LFFN_ROWS_F32 ? 4 : 2;
+    const int cols = 128 / esz;
+    if (S != MAX_S || T < 8 || T % 2 != 0 || T > (1 << 20) || Do % cols != 0 || B * T >= (int64_t(1) << 31) ||
+        2 * S * Do * esz >= (int64_t(1) << 32))
         return best;
-    const int64_t nslices = Do / 32;
+    const int64_t nslices = Do / cols;
     if (((B + 1023) / 1024) * nslices < 192 || B * nslices > (int64_t(1) << 30)) return best;
+    const double per_pass = fmt == LFFN_ROWS_F32 ? QUAD_US_PER_PAIR_PASS : QUAD_US_PER_PAIR_PASS_16[fmt];
     for (int np : {4, 6, 7, 8}) {
+        if (!lffn_internal_quad_np_built(fmt, np)) continue;
         const int64_t tiles = (B + 256 * np - 1) / (256 * np);
         const int64_t rounds = (tiles * nslices + 255) / 256;
-        const double us = double(rounds) * double(T / 2) * (QUAD_US_PER_PAIR + np * QUAD_US_PER_PAIR_PASS) +
-                          double(B) * double(T) * 14.0 / 3e6 + 4.0;      // packing: 8 bytes read, 6 written per (token, table)
+        const double us = double(rounds) * double(T / 2) * (QUAD_US_PER_PAIR + np * per_pass) +
+                          (pack ? double(B) * double(T) * 14.0 / 3e6 + 4.0 : 0.0);     // packing: 8 bytes read, 6 written per (token, table)
         if (us < best.us) best = GatherPlan{3, np, us};
     }
     return best;
@@ -507,9 +513,9 @@ int64_t gather_pieces(int64_t B, int64_t T, int64_t S, int64_t Do) {
 // through the touch by turns, so it has no use for pieces), if it promises to beat what the other forms
 // get for the batch by QUAD_MARGIN: pieces, the one-launch LDS forms, the table split.  kind 0 otherwise.
 template <bool BF16>
-GatherPlan choose_quad(int64_t B, int64_t T, int64_t S, int64_t Do) {
+GatherPlan choose_quad(int64_t B, int64_t T, int64_t S, int64_t Do, bool pack = true) {
     const GatherPlan none{0, 0, 1e300};
-    const GatherPlan qp = plan_quad<BF16>(B, T, S, Do);
+    const GatherPlan qp = plan_quad(BF16 ? LFFN_ROWS_BF16 : LFFN_ROWS_F32, B, T, S, Do, pack);
     if (qp.kind != 3) return none;
     double other;
     const int64_t each = gather_pieces<BF16>(B, T, S, Do);
@@ -523,13 +529,21 @@ GatherPlan choose_quad(int64_t B, int64_t T, int64_t S, int64_t Do) {
     return qp.us < QUAD_MARGIN * other ? qp : none;
 }
 
+// four lanes per token: a tile size built for the row format, 256-row tables, an even number of them, whole
+// 128-byte slices, 32-bit offsets inside a table pair
+bool quad_plan_is_valid(int fmt, int np, int64_t B, int64_t T, int64_t S, int64_t Do) {
+    const int esz = fmt == LFFN_ROWS_F32 ? 4 : 2;
+    const int cols = 128 / esz;
+    return lffn_internal_quad_np_built(fmt, np) && S == MAX_S && T >= 2 && T % 2 == 0 && T <= (1 << 20) &&
+           Do % cols == 0 && B * T < (int64_t(1) << 31) && 2 * S * Do * esz < (int64_t(1) << 32) &&
+           B * (Do / cols) <= (int64_t(1) << 30);
+}
+
 template <bool BF16>
 bool plan_is_valid(const GatherPlan &p, int64_t B, int64_t T, int64_t S, int64_t Do) {
     if (p.kind == 0) return true;
-    if (p.kind == 3)        // four lanes per token: fp32 rows, an even number of tables, 32-bit offsets inside a table pair
-        return !BF16 && (p.np == 4 || p.np == 6 || p.np == 7 || p.np == 8) && S == MAX_S && T >= 2 && T % 2 == 0 &&
-               T <= (1 << 20) && Do % 32 == 0 && B * T < (int64_t(1) << 31) && 2 * S * Do * 4 < (int64_t(1) << 32) &&
-               B * (Do / 32) <= (int64_t(1) << 30);
+    if (p.kind == 3)        // four lanes per token
+        return quad_plan_is_valid(BF16 ? LFFN_ROWS_BF16 : LFFN_ROWS_F32, p.np, B, T, S, Do);
     if (p.kind != 1 && p.kind != 2) return false;
     const bool np_ok = BF16 ? (p.np == 4 || p.np == 8) : (p.np == 4 || p.np == 8 || p.np == 13 || p.np == 16);
     const int cols = (p.kind == 1 ? 256 : 128) / (BF16 ? 2 : 4);
@@ -557,7 +571,8 @@ int lookup_gather_entry(const int32_t *code, const float *score, const void *tab
         if (qp.kind == 3 && workspace_bytes >= lffn_internal_quad_stream_bytes(B, T) && (uintptr_t)code % 8 == 0 &&
             (uintptr_t)score % 8 == 0) {
             LFFN_REQUIRE(lffn_aligned16(workspace), LFFN_ERR_BAD_ARG);
-            return lffn_internal_lookup_gather_quad(code, score, tables, bias, residual, out, B, T, S, Do, qp.np, workspace, stream);
+            return lffn_internal_lookup_gather_quad(code, score, tables, bias, residual, out, B, T, S, Do,
+                                                    BF16 ? LFFN_ROWS_BF16 : LFFN_ROWS_F32, qp.np, workspace, stream);
         }
     }
     // Many tokens, tables that fit the 256 MB Infinity Cache: take the tokens in pieces, one launch
@@ -618,10 +633,9 @@ int lookup_gather_entry(const int32_t *code, const float *score, const void *tab
     }
     if (plan.kind == 0)
         return lffn_internal_lookup_gather_token_major(code, score, tables, bias, residual, out, B, T, S, Do, BF16, stream);
-    if (plan.kind == 3) {
-        if constexpr (BF16) return LFFN_ERR_UNSUPPORTED;
-        return lffn_internal_lookup_gather_quad(code, score, tables, bias, residual, out, B, T, S, Do, plan.np, quad_ws, stream);
-    }
+    if (plan.kind == 3)
+        return lffn_internal_lookup_gather_quad(code, score, tables, bias, residual, out, B, T, S, Do,
+                                                BF16 ? LFFN_ROWS_BF16 : LFFN_ROWS_F32, plan.np, quad_ws, stream);
     if (plan.kind == 2)
         return lffn_internal_lookup_gather_pair(code, score, tables, bias, residual, out, B, T, S, Do, BF16, plan.np, stream);
     const int np = plan.np;
@@ -642,6 +656,43 @@ int lookup_gather_entry(const int32_t *code, const float *score, const void *tab
             default: return launch_lds<false, 4>(a, st);
         }
     }
+}
+
+// Half rows (the row format of the reference's reduced-precision gather, gather_kernel_fp16.cu:6-62; fp32
+// sums here): the four-lanes-per-token kernel where the shape qualifies and the caller brings a workspace for
+// the records, the token-major kernel otherwise.  kind_req < 0: choose; 0 or 3: exactly that kernel.
+int lookup_gather_entry_f16(const int32_t *code, const float *score, const void *tables, const float *bias,
+                            const float *residual, float *out, int64_t B, int64_t T, int64_t S, int64_t Do, int kind_req,
+                            int tokens_req, void *stream, void *workspace, int64_t workspace_bytes) {
+    LFFN_REQUIRE(B >= 0 && T >= 0 && Do >= 1, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_is_pow2(S) && S <= (1 << 24) && T * S <= 0x7fffffff, LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(Do % 64 == 0 && Do <= (1 << 20) && T <= (1 << 24), LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(B <= (int64_t(1) << 31) - 1, LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(tables && out && ((code && score) || B * T == 0), LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_aligned16(tables) && lffn_aligned16(out) && (!bias || lffn_aligned16(bias)) &&
+                     (!residual || lffn_aligned16(residual)), LFFN_ERR_BAD_ARG);
+    if (B == 0) return LFFN_OK;
+    int np = 0;
+    if (kind_req < 0) {
+        const GatherPlan qp = plan_quad(LFFN_ROWS_F16, B, T, S, Do);
+        const double token_major_us = double(B) * double(T) * double(Do) * 2 / 9e6 + 5.0;
+        if (qp.kind == 3 && qp.us < QUAD_MARGIN * token_major_us && workspace &&
+            workspace_bytes >= lffn_internal_quad_stream_bytes(B, T) && lffn_aligned16(workspace) &&
+            (uintptr_t)code % 8 == 0 && (uintptr_t)score % 8 == 0)
+            np = qp.np;
+    } else if (kind_req == 3) {
+        LFFN_REQUIRE(tokens_req > 0 && tokens_req % 256 == 0, LFFN_ERR_BAD_ARG);
+        np = tokens_req / 256;
+        LFFN_REQUIRE(quad_plan_is_valid(LFFN_ROWS_F16, np, B, T, S, Do), LFFN_ERR_UNSUPPORTED);
+        LFFN_REQUIRE(workspace && workspace_bytes >= lffn_internal_quad_stream_bytes(B, T), LFFN_ERR_UNSUPPORTED);
+        LFFN_REQUIRE(lffn_aligned16(workspace) && (uintptr_t)code % 8 == 0 && (uintptr_t)score % 8 == 0, LFFN_ERR_BAD_ARG);
+    } else {
+        LFFN_REQUIRE(kind_req == 0, LFFN_ERR_UNSUPPORTED);       // the 16- and 8-lane LDS kernels are not built for half rows
+    }
+    if (np)
+        return lffn_internal_lookup_gather_quad(code, score, tables, bias, residual, out, B, T, S, Do, LFFN_ROWS_F16, np,
+                                                workspace, stream);
+    return lffn_internal_lookup_gather_token_major(code, score, tables, bias, residual, out, B, T, S, Do, LFFN_ROWS_F16, stream);
 }
 
 }  // namespace
@@ -670,12 +721,19 @@ extern "C" int lffn_lookup_gather_residual_bf16(const int32_t *code, const float
     return lookup_gather_entry<true>(code, score, tables, bias, residual, out, B, T, S, Do, -1, 0, stream);
 }
 
-extern "C" int lffn_lookup_gather_workspace_bytes(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t bf16,
+extern "C" int lffn_lookup_gather_workspace_bytes(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t row_format,
                                                   int64_t *bytes) {
-    LFFN_REQUIRE(bytes, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(bytes && row_format >= 0 && row_format <= 2, LFFN_ERR_BAD_ARG);
     *bytes = 0;
     if (B < 1 || T < 1 || Do < 1 || !lffn_is_pow2(S) || Do % 64 != 0 || B * T >= (int64_t(1) << 31)) return LFFN_OK;
-    if (!bf16 && choose_quad<false>(B, T, S, Do).kind == 3) {
+    if (row_format == LFFN_ROWS_F16) {
+        const GatherPlan qp = plan_quad(LFFN_ROWS_F16, B, T, S, Do);
+        if (qp.kind == 3 && qp.us < QUAD_MARGIN * (double(B) * double(T) * double(Do) * 2 / 9e6 + 5.0))
+            *bytes = lffn_internal_quad_stream_bytes(B, T);
+        return LFFN_OK;
+    }
+    const bool bf16 = row_format == LFFN_ROWS_BF16;
+    if ((bf16 ? choose_quad<true>(B, T, S, Do) : choose_quad<false>(B, T, S, Do)).kind == 3) {
         *bytes = lffn_internal_quad_stream_bytes(B, T);
         return LFFN_OK;
     }
@@ -685,6 +743,45 @@ extern "C" int lffn_lookup_gather_workspace_bytes(int64_t B, int64_t T, int64_t 
     const SplitPlan sp = bf16 ? plan_split<true>(B, T, S, Do) : plan_split<false>(B, T, S, Do);
     if (sp.nparts > 1 && sp.us < 0.85 * plan.us) *bytes = int64_t(sp.nparts) * B * Do * 4;
     return LFFN_OK;
+}
+
+// What the workspace entry points run for a shape when given a workspace of workspace_bytes: the tokens per
+// workgroup, and in *form 0 (token-major), 1 or 2 (tables per LDS buffer), 3 (four lanes per token, record
+// stream in the workspace) or 4 (table split: partial outputs in the workspace, 64-token passes of form 1).
+// A batch that is taken in pieces reports the form of a piece.
+extern "C" int lffn_lookup_gather_ws_plan(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t row_format,
+                                          int64_t workspace_bytes, int32_t *form) {
+    if (B < 0 || T < 0 || Do < 1 || !lffn_is_pow2(S) || Do % 64 != 0 || row_format < 0 || row_format > 2 || workspace_bytes < 0)
+        return LFFN_ERR_BAD_ARG;
+    int kind = 0, tokens = 0;
+    if (B >= 1 && T >= 1 && B * T < (int64_t(1) << 31)) {
+        const bool room = workspace_bytes >= lffn_internal_quad_stream_bytes(B, T);
+        if (row_format == LFFN_ROWS_F16) {
+            const GatherPlan qp = plan_quad(LFFN_ROWS_F16, B, T, S, Do);
+            if (qp.kind == 3 && room && qp.us < QUAD_MARGIN * (double(B) * double(T) * double(Do) * 2 / 9e6 + 5.0)) {
+                kind = 3; tokens = 256 * qp.np;
+            }
+        } else {
+            const bool bf16 = row_format == LFFN_ROWS_BF16;
+            const GatherPlan qp = bf16 ? choose_quad<true>(B, T, S, Do) : choose_quad<false>(B, T, S, Do);
+            if (qp.kind == 3 && room) {
+                kind = 3; tokens = 256 * qp.np;
+            } else {
+                int64_t each = bf16 ? gather_pieces<true>(B, T, S, Do) : gather_pieces<false>(B, T, S, Do);
+                if (each > B) each = B;
+                const GatherPlan plan = bf16 ? plan_gather<true>(each, T, S, Do) : plan_gather<false>(each, T, S, Do);
+                const SplitPlan sp = bf16 ? plan_split<true>(each, T, S, Do) : plan_split<false>(each, T, S, Do);
+                if (each == B && sp.nparts > 1 && sp.us < 0.85 * plan.us && workspace_bytes >= int64_t(sp.nparts) * B * Do * 4) {
+                    kind = 4; tokens = 64 * sp.np;
+                } else {
+                    kind = plan.kind;
+                    tokens = plan.kind == 0 ? 0 : (plan.kind == 1 ? 64 : 128) * plan.np;
+                }
+            }
+        }
+    }
+    if (form) *form = kind;
+    return tokens;
 }
 
 extern "C" int lffn_lookup_gather_ws_f32(const int32_t *code, const float *score, const float *tables,
@@ -703,6 +800,32 @@ extern "C" int lffn_lookup_gather_ws_bf16(const int32_t *code, const float *scor
     LFFN_REQUIRE(workspace_bytes >= 0 && (workspace || workspace_bytes == 0), LFFN_ERR_BAD_ARG);
     return lookup_gather_entry<true>(code, score, tables, bias, residual, out, B, T, S, Do, -1, 0, stream, workspace,
                                      workspace_bytes);
+}
+
+extern "C" int lffn_lookup_gather_ws_f16(const int32_t *code, const float *score, const uint16_t *tables,
+                                         const float *bias, const float *residual, float *out, void *workspace,
+                                         int64_t workspace_bytes, int64_t B, int64_t T, int64_t S, int64_t Do,
+                                         void *stream) {
+    LFFN_REQUIRE(workspace_bytes >= 0 && (workspace || workspace_bytes == 0), LFFN_ERR_BAD_ARG);
+    return lookup_gather_entry_f16(code, score, tables, bias, residual, out, B, T, S, Do, -1, 0, stream, workspace,
+                                   workspace_bytes);
+}
+
+extern "C" int lffn_lookup_gather_ws_planned_rows(const int32_t *code, const float *score, const void *tables,
+                                                  const float *bias, const float *residual, float *out, void *workspace,
+                                                  int64_t workspace_bytes, int64_t B, int64_t T, int64_t S, int64_t Do,
+                                                  int32_t row_format, int32_t tables_per_buffer,
+                                                  int32_t tokens_per_workgroup, void *stream) {
+    LFFN_REQUIRE(tables_per_buffer >= 0 && row_format >= 0 && row_format <= 2, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(workspace_bytes >= 0 && (workspace || workspace_bytes == 0), LFFN_ERR_BAD_ARG);
+    if (row_format == LFFN_ROWS_F16)
+        return lookup_gather_entry_f16(code, score, tables, bias, residual, out, B, T, S, Do, tables_per_buffer,
+                                       tokens_per_workgroup, stream, workspace, workspace_bytes);
+    if (row_format == LFFN_ROWS_BF16)
+        return lookup_gather_entry<true>(code, score, tables, bias, residual, out, B, T, S, Do, tables_per_buffer,
+                                         tokens_per_workgroup, stream, workspace, workspace_bytes);
+    return lookup_gather_entry<false>(code, score, tables, bias, residual, out, B, T, S, Do, tables_per_buffer,
+                                      tokens_per_workgroup, stream, workspace, workspace_bytes);
 }
 
 extern "C" int lffn_lookup_gather_planned_f32(const int32_t *code, const float *score, const float *tables,
@@ -743,12 +866,19 @@ extern "C" int lffn_lookup_gather_plan(int64_t B, int64_t T, int64_t S, int64_t 
 
 // ---------------------------------------------------------------- gather from a record stream
 
-extern "C" int lffn_lookup_gather_records_plan(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t *tokens_per_workgroup,
-                                               int64_t *record_stride, int64_t *bytes) {
-    LFFN_REQUIRE(tokens_per_workgroup && record_stride && bytes, LFFN_ERR_BAD_ARG);
+extern "C" int lffn_lookup_gather_records_plan_rows(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t row_format,
+                                                    int32_t *tokens_per_workgroup, int64_t *record_stride, int64_t *bytes) {
+    LFFN_REQUIRE(tokens_per_workgroup && record_stride && bytes && row_format >= 0 && row_format <= 2, LFFN_ERR_BAD_ARG);
     *tokens_per_workgroup = 0; *record_stride = 0; *bytes = 0;
     if (B < 1 || T < 1 || Do < 1 || !lffn_is_pow2(S) || Do % 64 != 0 || B * T >= (int64_t(1) << 31)) return LFFN_OK;
-    const GatherPlan qp = choose_quad<false>(B, T, S, Do);
+    GatherPlan qp;
+    if (row_format == LFFN_ROWS_F16) {
+        qp = plan_quad(LFFN_ROWS_F16, B, T, S, Do, false);
+        if (qp.kind == 3 && !(qp.us < QUAD_MARGIN * (double(B) * double(T) * double(Do) * 2 / 9e6 + 5.0))) qp.kind = 0;
+    } else {
+        // (the records are written by the projection kernel: no packing kernel to pay for)
+        qp = row_format == LFFN_ROWS_BF16 ? choose_quad<true>(B, T, S, Do, false) : choose_quad<false>(B, T, S, Do, false);
+    }
     if (qp.kind != 3) return LFFN_OK;
     *tokens_per_workgroup = 256 * qp.np;
     *record_stride = lffn_internal_quad_record_stride(B, qp.np);
@@ -756,16 +886,30 @@ extern "C" int lffn_lookup_gather_records_plan(int64_t B, int64_t T, int64_t S, 
     return LFFN_OK;
 }
 
-extern "C" int lffn_lookup_gather_records_f32(const uint32_t *records, int64_t record_stride, const float *tables,
-                                              const float *bias, const float *residual, float *out, int64_t B, int64_t T,
-                                              int64_t S, int64_t Do, int32_t tokens_per_workgroup, void *stream) {
-    LFFN_REQUIRE(B >= 0 && T >= 0 && Do >= 1 && tokens_per_workgroup > 0, LFFN_ERR_BAD_ARG);
+extern "C" int lffn_lookup_gather_records_plan(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t *tokens_per_workgroup,
+                                               int64_t *record_stride, int64_t *bytes) {
+    return lffn_lookup_gather_records_plan_rows(B, T, S, Do, LFFN_ROWS_F32, tokens_per_workgroup, record_stride, bytes);
+}
+
+extern "C" int lffn_lookup_gather_records_rows(const uint32_t *records, int64_t record_stride, const void *tables,
+                                               const float *bias, const float *residual, float *out, int64_t B, int64_t T,
+                                               int64_t S, int64_t Do, int32_t row_format, int32_t tokens_per_workgroup,
+                                               void *stream) {
+    LFFN_REQUIRE(B >= 0 && T >= 0 && Do >= 1 && tokens_per_workgroup > 0 && row_format >= 0 && row_format <= 2, LFFN_ERR_BAD_ARG);
     LFFN_REQUIRE(tokens_per_workgroup % 256 == 0, LFFN_ERR_BAD_ARG);
-    const GatherPlan plan{3, tokens_per_workgroup / 256, 0.0};
-    LFFN_REQUIRE(lffn_is_pow2(S) && Do % 64 == 0 && plan_is_valid<false>(plan, B, T, S, Do), LFFN_ERR_UNSUPPORTED);
+    const int np = tokens_per_workgroup / 256;
+    LFFN_REQUIRE(lffn_is_pow2(S) && Do % 64 == 0 && quad_plan_is_valid(row_format, np, B, T, S, Do), LFFN_ERR_UNSUPPORTED);
     LFFN_REQUIRE(tables && out && (records || B == 0), LFFN_ERR_BAD_ARG);
     LFFN_REQUIRE(lffn_aligned16(tables) && lffn_aligned16(out) && (!bias || lffn_aligned16(bias)) &&
                      (!residual || lffn_aligned16(residual)) && (uintptr_t)records % 4 == 0, LFFN_ERR_BAD_ARG);
     if (B == 0) return LFFN_OK;
-    return lffn_internal_lookup_gather_quad_records(records, record_stride, tables, bias, residual, out, B, T, S, Do, plan.np, stream);
+    return lffn_internal_lookup_gather_quad_records(records, record_stride, tables, bias, residual, out, B, T, S, Do,
+                                                    row_format, np, stream);
+}
+
+extern "C" int lffn_lookup_gather_records_f32(const uint32_t *records, int64_t record_stride, const float *tables,
+                                              const float *bias, const float *residual, float *out, int64_t B, int64_t T,
+                                              int64_t S, int64_t Do, int32_t tokens_per_workgroup, void *stream) {
+    return lffn_lookup_gather_records_rows(records, record_stride, tables, bias, residual, out, B, T, S, Do, LFFN_ROWS_F32,
+                                           tokens_per_workgroup, stream);
 }

@@ -32,6 +32,13 @@
 //     worth fits beside the two table buffers.)
 //
 // One barrier per table pair; the global -> LDS copy of pair k+1 has the whole of pair k's work to land.
+//
+// Row formats.  fp32 rows: the slice is 32 columns and a lane owns 8 of them.  16-bit rows (bfloat16, and
+// half, the format of the reference's own reduced-precision kernels, PL/gather/cuda/extension/
+// gather_kernel_fp16.cu:6-62): the slice is still 128 bytes = 64 columns, a lane owns 16 of them, and the
+// sums stay fp32 (the reference accumulates in half).  The LDS side is the same bytes either way; what
+// differs is the vector-ALU work per 16-byte piece: 4 multiply-adds (fp32), 8 widenings + 8 multiply-adds
+// (bfloat16: a shift or a mask per value), 8 v_fma_mix_f32 (half: the instruction widens its operand).
 #include "lffn_common.h"
 
 namespace {
@@ -41,7 +48,9 @@ constexpr int NWAVES = WG / 64;
 constexpr int MAX_S = 256;
 constexpr int XCDS = 8;
 constexpr int BUF_BYTES = MAX_S * 256;      // one table pair: S rows of 2 x 128 bytes; a power of two (bit 16)
-constexpr int SLICE_COLS = 32;
+constexpr int SLICE_BYTES = 128;            // a slice of a row: 32 fp32 columns or 64 16-bit columns
+constexpr int FMT_F32 = LFFN_ROWS_F32, FMT_BF16 = LFFN_ROWS_BF16, FMT_F16 = LFFN_ROWS_F16;
+constexpr int fmt_bytes(int fmt) { return fmt == FMT_F32 ? 4 : 2; }
 constexpr int QUAD_TOUCH_AHEAD = 3;         // pairs between the one being read and the one being touched
 
 // (code, score) of one token and one table pair in the order the token's quad takes the pair's tables
@@ -55,14 +64,14 @@ struct PairRecord {
 constexpr int REC_WORDS = 3;
 
 struct QuadArgs {
-    const char *tables;    // [T, S, Do] fp32
+    const char *tables;    // [T, S, Do] fp32, bfloat16 or half
     const float *bias;     // [Do] or null
     const float *residual; // [B, Do] or null: added to the result (may be the output buffer)
     float *out;            // [B, Do]
     int64_t B;
     int T, S, Do;          // T even, S = 256
     int ntiles, nslices, per_xcd;
-    int row_bytes;         // Do * 4
+    int row_bytes;         // Do * bytes per element
     const uint32_t *stream;     // [T/2][3][Bpad] record words written by pack_pairs_kernel
     int64_t Bpad;               // B rounded up to whole token tiles: tokens past B have all-zero records
 };
@@ -155,9 +164,38 @@ __global__ __launch_bounds__(256) void pack_pairs_kernel(const int32_t *code, co
     }
 }
 
-template <int NP, bool TOUCH>
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+// acc += w * (the EPV values of one 16-byte piece of a row)
+template <int FMT, int EPV>
+__device__ __forceinline__ void fma_piece(float (&ac)[EPV], float w, const u32x4 &v) {
+    if constexpr (FMT == FMT_F32) {
+        ac[0] = fmaf(__uint_as_float(v.x), w, ac[0]);
+        ac[1] = fmaf(__uint_as_float(v.y), w, ac[1]);
+        ac[2] = fmaf(__uint_as_float(v.z), w, ac[2]);
+        ac[3] = fmaf(__uint_as_float(v.w), w, ac[3]);
+    } else {
+        const unsigned q[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if constexpr (FMT == FMT_BF16) {
+                ac[2 * i] = fmaf(bf16_lo(q[i]), w, ac[2 * i]);
+                ac[2 * i + 1] = fmaf(bf16_hi(q[i]), w, ac[2 * i + 1]);
+            } else {
+                // (float)half * float + float: one v_fma_mix_f32 each
+                const half2_t h = __builtin_bit_cast(half2_t, q[i]);
+                ac[2 * i] = fmaf((float)h.x, w, ac[2 * i]);
+                ac[2 * i + 1] = fmaf((float)h.y, w, ac[2 * i + 1]);
+            }
+        }
+    }
+}
+
+template <int FMT, int NP, bool TOUCH>
 __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
     static_assert(NP >= 4 && NP <= 8, "a lane reads the records of passes l and l + 4");
+    constexpr int EPV = 16 / fmt_bytes(FMT);              // columns in a 16-byte piece
+    constexpr int SLICE_COLS = SLICE_BYTES / fmt_bytes(FMT);
     constexpr int WAVE_RECS = 16 * NP;                    // records a wavefront uses per table pair
     constexpr int REC_LOADS = (WAVE_RECS + 63) / 64;      // one-word-per-lane copy instructions per plane
     extern __shared__ uint4 lds[];                // 2 buffers of BUF_BYTES, the touches' sink, the wavefronts' records
@@ -180,20 +218,20 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
     const int half0 = quad & 1;
     const int64_t tok0 = int64_t(tile) * (256 * NP) + wave * 16 + quad;
 
-    // acc[p][h][e]: token tok0 + 256 p, column (half0 ^ h) * 16 + 4 l + e of the slice
-    float acc[NP][2][4];
+    // acc[p][h][e]: token tok0 + 256 p, column ((half0 ^ h) * 4 + l) * EPV + e of the slice
+    float acc[NP][2][EPV];
     {
-        float b[2][4];
+        float b[2][EPV];
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) b[h][e] = 0.f;
+            for (int e = 0; e < EPV; ++e) b[h][e] = 0.f;
         if (a.bias) {
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                const float *bp = a.bias + (size_t)slice * SLICE_COLS + (half0 ^ h) * 16 + l * 4;
+                const float *bp = a.bias + (size_t)slice * SLICE_COLS + ((half0 ^ h) * 4 + l) * EPV;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) b[h][e] = bp[e];
+                for (int e = 0; e < EPV; ++e) b[h][e] = bp[e];
             }
         }
 #pragma unroll
@@ -201,7 +239,7 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
 #pragma unroll
             for (int h = 0; h < 2; ++h)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) acc[p][h][e] = b[h][e];
+                for (int e = 0; e < EPV; ++e) acc[p][h][e] = b[h][e];
     }
 
     const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) uint4 *)lds;
@@ -210,7 +248,7 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
     // 2k+1; rows are Do*4 bytes apart, the second table S rows further down.  The four vectors of a lane
     // are 64 rows apart: one lane offset, four uniform bases.
     const size_t table_bytes = (size_t)a.S * a.row_bytes;
-    const char *slice_base = a.tables + (size_t)slice * 128;
+    const char *slice_base = a.tables + (size_t)slice * SLICE_BYTES;
     const size_t pair_stride = 2 * table_bytes;
     const size_t quarter = (size_t)(WG / 16) * a.row_bytes;
     const int npairs = a.T / 2;
@@ -295,12 +333,7 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
         // is still being added (its first table's two rows are consumed, their registers take the
         // next pass's first two reads; likewise the second table's), so a wavefront always has
         // two to four row reads in flight behind its multiply-adds.
-        auto fma4 = [&](float (&ac)[4], float w, const u32x4 &v) {
-            ac[0] = fmaf(__uint_as_float(v.x), w, ac[0]);
-            ac[1] = fmaf(__uint_as_float(v.y), w, ac[1]);
-            ac[2] = fmaf(__uint_as_float(v.z), w, ac[2]);
-            ac[3] = fmaf(__uint_as_float(v.w), w, ac[3]);
-        };
+        auto fma4 = [&](float (&ac)[EPV], float w, const u32x4 &v) { fma_piece<FMT, EPV>(ac, w, v); };
         // the record of pass P sits in lane P % 4 of the quad, in rec0 (P < 4) or rec1
         auto rows_of = [&](auto p_c) {
             constexpr int P = decltype(p_c)::value;
@@ -377,27 +410,29 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
         const int64_t tok = tok0 + p * 256;
         if (tok < a.B) {
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const size_t off = tok * a.Do + (size_t)slice * SLICE_COLS + (half0 ^ h) * 16 + l * 4;
-                float4 v = make_float4(acc[p][h][0], acc[p][h][1], acc[p][h][2], acc[p][h][3]);
-                if (a.residual) {
-                    const float4 rr = *reinterpret_cast<const float4 *>(a.residual + off);
-                    v.x += rr.x; v.y += rr.y; v.z += rr.z; v.w += rr.w;
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int q = 0; q < EPV / 4; ++q) {
+                    const size_t off = tok * a.Do + (size_t)slice * SLICE_COLS + ((half0 ^ h) * 4 + l) * EPV + 4 * q;
+                    float4 v = make_float4(acc[p][h][4 * q], acc[p][h][4 * q + 1], acc[p][h][4 * q + 2], acc[p][h][4 * q + 3]);
+                    if (a.residual) {
+                        const float4 rr = *reinterpret_cast<const float4 *>(a.residual + off);
+                        v.x += rr.x; v.y += rr.y; v.z += rr.z; v.w += rr.w;
+                    }
+                    *reinterpret_cast<float4 *>(a.out + off) = v;
                 }
-                *reinterpret_cast<float4 *>(a.out + off) = v;
-            }
         }
     }
 }
 
-template <int NP, bool TOUCH>
+template <int FMT, int NP, bool TOUCH>
 int launch_quad(QuadArgs a, hipStream_t stream) {
     a.ntiles = (int)((a.B + 256 * NP - 1) / (256 * NP));
     const int units = a.ntiles * a.nslices;
     a.per_xcd = (units + XCDS - 1) / XCDS;
     // two buffers, the touches' scratch, every wavefront's records of one table pair
     const size_t lds_bytes = size_t(2) * BUF_BYTES + TOUCH_SINK_BYTES + size_t(NWAVES) * 16 * NP * REC_WORDS * 4;
-    auto kern = lookup_gather_quad_kernel<NP, TOUCH>;
+    auto kern = lookup_gather_quad_kernel<FMT, NP, TOUCH>;
     static LdsGrant granted;      // one record per kernel instantiation
     if (!lffn_grant_dynamic_lds(reinterpret_cast<const void *>(kern), lds_bytes, granted)) return LFFN_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3(a.per_xcd * XCDS), dim3(WG), lds_bytes, stream, a);
@@ -412,33 +447,46 @@ int64_t lffn_internal_quad_stream_bytes(int64_t B, int64_t T) {
     return (T / 2) * (B + 2048) * (int64_t)(REC_WORDS * 4);
 }
 
+// Which tile sizes (passes of 256 tokens per workgroup) are built for a row format: the accumulators, 8 per
+// pass and lane for fp32 rows and 16 for 16-bit rows, must fit the 128 registers a lane of a 1024-lane
+// workgroup can have.
+bool lffn_internal_quad_np_built(int fmt, int np) {
+    if (fmt == FMT_F32) return np == 4 || np == 6 || np == 7 || np == 8;
+    return (fmt == FMT_BF16 || fmt == FMT_F16) && np == 4;
+}
+
 // Run the gather from a record stream [T/2][3][record_stride] (pack_pairs_kernel's layout; the projection
 // kernel of fht.hip writes the same) with 256*np tokens per workgroup.  The caller has checked that the
-// shape qualifies: fp32 rows, S = 256 (a table pair fills an LDS buffer), T even, Do a multiple of 32,
-// 2*S*Do*4 < 2^32 (32-bit lane offsets from a table pair's base), np one of {4, 6, 7, 8}.  record_stride:
-// whole tiles of 256*np tokens, at least B; what the records of tokens from B on hold does not matter
-// (their row numbers are bytes, always inside the LDS buffer, and their sums are not stored).
+// shape qualifies: S = 256 (a table pair fills an LDS buffer), T even, Do a multiple of the slice's columns
+// (32 for fp32 rows, 64 for 16-bit rows), 2*S*Do*element bytes < 2^32 (32-bit lane offsets from a table
+// pair's base), np built for the format.  record_stride: whole tiles of 256*np tokens, at least B; what the
+// records of tokens from B on hold does not matter (their row numbers are bytes, always inside the LDS
+// buffer, and their sums are not stored).
 int lffn_internal_lookup_gather_quad_records(const uint32_t *records, int64_t record_stride, const void *tables,
                                              const float *bias, const float *residual, float *out, int64_t B,
-                                             int64_t T, int64_t S, int64_t Do, int np, void *stream) {
-    if (!records || S != MAX_S || T % 2 != 0 || !(np == 4 || np == 6 || np == 7 || np == 8)) return LFFN_ERR_BAD_ARG;
+                                             int64_t T, int64_t S, int64_t Do, int fmt, int np, void *stream) {
+    if (!records || S != MAX_S || T % 2 != 0 || !lffn_internal_quad_np_built(fmt, np)) return LFFN_ERR_BAD_ARG;
     const int64_t tile_tokens = 256 * int64_t(np);
     if (record_stride % tile_tokens != 0 || record_stride < B) return LFFN_ERR_BAD_ARG;
+    const int esz = fmt_bytes(fmt);
+    if (Do % (SLICE_BYTES / esz) != 0) return LFFN_ERR_BAD_ARG;
     QuadArgs a{};
     a.tables = static_cast<const char *>(tables); a.bias = bias; a.residual = residual; a.out = out;
     a.B = B; a.T = (int)T; a.S = (int)S; a.Do = (int)Do;
-    a.nslices = (int)(Do / SLICE_COLS);
-    a.row_bytes = (int)(Do * 4);
+    a.nslices = (int)(Do * esz / SLICE_BYTES);
+    a.row_bytes = (int)(Do * esz);
     a.Bpad = record_stride;
     a.stream = records;
     hipStream_t st = static_cast<hipStream_t>(stream);
     // the touch by turns, always: tables beyond the 256 MB memory-side cache need it most (984 -> 736 us
     // at 512 tables x 256 x 1024 and 1024 tokens per workgroup)
+    if (fmt == FMT_BF16) return launch_quad<FMT_BF16, 4, true>(a, st);
+    if (fmt == FMT_F16) return launch_quad<FMT_F16, 4, true>(a, st);
     switch (np) {
-        case 8: return launch_quad<8, true>(a, st);
-        case 7: return launch_quad<7, true>(a, st);
-        case 6: return launch_quad<6, true>(a, st);
-        default: return launch_quad<4, true>(a, st);
+        case 8: return launch_quad<FMT_F32, 8, true>(a, st);
+        case 7: return launch_quad<FMT_F32, 7, true>(a, st);
+        case 6: return launch_quad<FMT_F32, 6, true>(a, st);
+        default: return launch_quad<FMT_F32, 4, true>(a, st);
     }
 }
 
@@ -451,13 +499,13 @@ int64_t lffn_internal_quad_record_stride(int64_t B, int np) {
 // lffn_internal_quad_stream_bytes(B, T) bytes, 16-byte aligned) and run the gather from it.
 int lffn_internal_lookup_gather_quad(const int32_t *code, const float *score, const void *tables,
                                      const float *bias, const float *residual, float *out, int64_t B, int64_t T,
-                                     int64_t S, int64_t Do, int np, void *workspace, void *stream) {
-    if (!workspace || S != MAX_S || T % 2 != 0 || !(np == 4 || np == 6 || np == 7 || np == 8)) return LFFN_ERR_BAD_ARG;
+                                     int64_t S, int64_t Do, int fmt, int np, void *workspace, void *stream) {
+    if (!workspace || S != MAX_S || T % 2 != 0 || !lffn_internal_quad_np_built(fmt, np)) return LFFN_ERR_BAD_ARG;
     uint32_t *recs = static_cast<uint32_t *>(workspace);
     const int64_t stride = lffn_internal_quad_record_stride(B, np);
     const dim3 grid((unsigned)((stride + 63) / 64), (unsigned)((T / 2 + 31) / 32));
     hipLaunchKernelGGL(pack_pairs_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), code, score, recs, B,
                        stride, (int)T, (int)S);
     if (hipGetLastError() != hipSuccess) return LFFN_ERR_LAUNCH;
-    return lffn_internal_lookup_gather_quad_records(recs, stride, tables, bias, residual, out, B, T, S, Do, np, stream);
+    return lffn_internal_lookup_gather_quad_records(recs, stride, tables, bias, residual, out, B, T, S, Do, fmt, np, stream);
 }

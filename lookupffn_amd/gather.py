@@ -1,6 +1,6 @@
 """Weighted gather-add operators: the reference's ``gather`` /
 ``weighted_gather_add`` surface (PL/gather/kernel.py, PL/gather/cuda/kernel.py) on the
-gfx950 kernels.  Rows may be float32 or bfloat16; weights, accumulation and
+gfx950 kernels.  Rows may be float32, bfloat16 or float16; weights, accumulation and
 outputs are float32."""
 from __future__ import annotations
 
@@ -30,7 +30,7 @@ def _check(indexes, a, b, names):
 def weighted_vector_gather_add(indexes, source, weights, use_torch=False):
     """outputs[b] = sum_i weights[b,i] * source[indexes[b,i]]   (PL/gather/cuda/kernel.py:22-70)."""
     _check(indexes, source, weights, "gather")
-    assert source.dtype in [torch.float32, torch.bfloat16], source.dtype
+    assert source.dtype in [torch.float32, torch.bfloat16, torch.float16], source.dtype
     assert weights.dtype == torch.float32, weights.dtype
     batch_size, index_size = indexes.shape
     source_size, vector_dim = source.shape
@@ -108,7 +108,7 @@ class WeightedVectorGatherAdd(Function):
         grad_outputs = grad_outputs.contiguous()
         indexes, source, weights = ctx.saved_tensors
         if source.dtype != torch.float32:
-            raise NotImplementedError("backward through bfloat16 rows is not built (inference format)")
+            raise NotImplementedError("backward through 16-bit rows is not built (inference formats)")
         grad_weights = indexed_inner_product(indexes, grad_outputs, source)
         grad_source = weighted_vector_scatter_add(indexes, grad_outputs, weights, source.shape[0])
         return None, grad_source, grad_weights
@@ -147,7 +147,7 @@ class LookupGather(Function):
     def backward(ctx, grad_outputs):
         code, score, tables = ctx.saved_tensors
         if tables.dtype != torch.float32:
-            raise NotImplementedError("backward through bfloat16 tables is not built (inference format)")
+            raise NotImplementedError("backward through 16-bit tables is not built (inference formats)")
         grad_outputs = grad_outputs.contiguous()
         T, S, Do = tables.shape
         grad_score = ops.lookup_inner(code, grad_outputs, tables) if ctx.needs_input_grad[1] else None

@@ -375,7 +375,7 @@ class LookupFFN(nn.Module):
               and all(q is None or (q.dtype == torch.float32 and q.is_cuda and q.is_contiguous()
                                     and q.device == self.tables.device) for q in small)
               and self.tables.is_cuda and self.tables.is_contiguous()
-              and self.tables.dtype in (torch.float32, torch.bfloat16) and self.output_size % 64 == 0)
+              and ops.row_format(self.tables.dtype) is not None and self.output_size % 64 == 0)
         form = None
         if ok and p.block_size == 1 and 8 <= p.padded_in_dim <= 1024:
             form = "diag"
@@ -409,9 +409,10 @@ class LookupFFN(nn.Module):
             # small batches: the whole layer in one launch
             return ops.lookup_ffn_fused_direct(x, st["ln_w"], st["ln_b"], st["eps"], st["diag"], st["pbias"],
                                                st["tables"], st["obias"], residual, st["decay"], st["res_coef"])
-        if st["tables"].dtype == torch.float32 and self.num_table % 2 == 0:
+        if self.num_table % 2 == 0:
             # many tokens: the projection kernel writes the gather kernel's record stream directly
-            plan = ops.lookup_gather_records_plan(x.shape[0], self.num_table, self.table_size, self.output_size)
+            plan = ops.lookup_gather_records_plan(x.shape[0], self.num_table, self.table_size, self.output_size,
+                                                  ops.row_format(st["tables"].dtype))
             records = None
             if plan is not None and st["form"] == "diag" and st["diag"].shape[2] >= 16:
                 records = ops.ln_project_hash_records_direct(x, st["ln_w"], st["ln_b"], st["eps"], st["diag"], st["pbias"],
@@ -460,7 +461,7 @@ class LookupFFN(nn.Module):
             else:
                 hidden_states = ln(hidden_states)
                 code, score = self.hash(hidden_states)
-        if self.output_size % 64 == 0 and self.tables.dtype in (torch.float32, torch.bfloat16):
+        if self.output_size % 64 == 0 and ops.row_format(self.tables.dtype) is not None:
             # table-local codes, offset and bias folded into the gather kernel
             return lookup_gather(code, score.float(), self.tables, self.bias.float(), residual)
         outputs = self.gather(code, score, self.tables)

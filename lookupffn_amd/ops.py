@@ -702,8 +702,10 @@ def _gather_add_impl(indexes, source, weights):
         fn, name = lib.lffn_gather_add_f32, "lffn_gather_add_f32"
     elif source.dtype == torch.bfloat16:
         fn, name = lib.lffn_gather_add_bf16, "lffn_gather_add_bf16"
+    elif source.dtype == torch.float16:
+        fn, name = lib.lffn_gather_add_f16, "lffn_gather_add_f16"
     else:
-        raise NotImplementedError(f"gather_add: source dtype {source.dtype} (float32 and bfloat16 rows are built)")
+        raise NotImplementedError(f"gather_add: source dtype {source.dtype} (float32, bfloat16 and float16 rows are built)")
     with _dev_guard(source):
         rc = fn(_lib.ptr(indexes), _lib.ptr(source), _lib.ptr(weights), _lib.ptr(out), B, I, S, Dv,
                 _lib.stream_of(source))
@@ -725,16 +727,24 @@ def _(indexes, source, weights):
 _RECORDS_PLANS = {}
 
 
-def lookup_gather_records_plan(B, T, S, Do):
+ROWS_F32, ROWS_BF16, ROWS_F16 = 0, 1, 2      # the C ABI's row_format values
+
+
+def row_format(dtype):
+    """The C ABI's row_format for a table dtype, or None for a dtype no gather kernel is built for."""
+    return {torch.float32: ROWS_F32, torch.bfloat16: ROWS_BF16, torch.float16: ROWS_F16}.get(dtype)
+
+
+def lookup_gather_records_plan(B, T, S, Do, fmt=ROWS_F32):
     """(tokens per workgroup, record stride in tokens, bytes of the stream) when the record-stream form of
-    the gather is the one to use for this shape (fp32 rows), else None.  Host-side query, cached."""
-    key = (B, T, S, Do)
+    the gather is the one to use for this shape and row format, else None.  Host-side query, cached."""
+    key = (B, T, S, Do, fmt)
     hit = _RECORDS_PLANS.get(key, False)
     if hit is not False:
         return hit
     tokens, stride, nbytes = ctypes.c_int32(0), ctypes.c_int64(0), ctypes.c_int64(0)
-    _lib.check(_lib.load().lffn_lookup_gather_records_plan(B, T, S, Do, ctypes.byref(tokens), ctypes.byref(stride),
-                                                           ctypes.byref(nbytes)), "lffn_lookup_gather_records_plan")
+    _lib.check(_lib.load().lffn_lookup_gather_records_plan_rows(B, T, S, Do, fmt, ctypes.byref(tokens), ctypes.byref(stride),
+                                                                ctypes.byref(nbytes)), "lffn_lookup_gather_records_plan_rows")
     plan = (tokens.value, stride.value, nbytes.value) if nbytes.value > 0 else None
     if len(_RECORDS_PLANS) < 4096:
         _RECORDS_PLANS[key] = plan
@@ -784,20 +794,22 @@ def ln_bh4_block_hash_records_direct(x, ln_w, ln_b, eps, w_folded, pbias, T, dec
 
 
 def lookup_gather_records_direct(records, plan, tables, bias, residual, B):
-    """out[b] = residual[b] + bias + sum_t score * row, from the record stream written for `plan`."""
+    """out[b] = residual[b] + bias + sum_t score * row, from the record stream written for `plan` (which was
+    made for the tables' row format)."""
     T, S, Do = tables.shape
-    _require(tables.dtype == torch.float32 and tables.is_contiguous() and records.numel() * 4 >= plan[2],
-             "tables: contiguous fp32; records: at least the plan's bytes")
+    fmt = row_format(tables.dtype)
+    _require(fmt is not None and tables.is_contiguous() and records.numel() * 4 >= plan[2],
+             "tables: contiguous float32, bfloat16 or float16; records: at least the plan's bytes")
     _require(residual is None or (residual.dtype == torch.float32 and residual.is_contiguous()
                                   and residual.device == tables.device and tuple(residual.shape) == (B, Do)),
              "residual: contiguous fp32 [B, Do] on the tables' device")
     out = torch.empty(B, Do, dtype=torch.float32, device=tables.device)
     with _dev_guard(tables):
-        rc = _lib.load().lffn_lookup_gather_records_f32(
+        rc = _lib.load().lffn_lookup_gather_records_rows(
             records.data_ptr(), plan[1], tables.data_ptr(), None if bias is None else bias.data_ptr(),
-            None if residual is None else residual.data_ptr(), out.data_ptr(), B, T, S, Do, plan[0], _lib.stream_of(tables))
+            None if residual is None else residual.data_ptr(), out.data_ptr(), B, T, S, Do, fmt, plan[0], _lib.stream_of(tables))
     if rc != 0:
-        _lib.check(rc, f"lffn_lookup_gather_records_f32(B={B}, T={T}, S={S}, Do={Do})")
+        _lib.check(rc, f"lffn_lookup_gather_records_rows(B={B}, T={T}, S={S}, Do={Do}, row_format={fmt})")
     return out
 
 
@@ -819,25 +831,25 @@ def _lookup_gather_impl(code, score, tables, bias, residual=None):
         assert residual.dtype == torch.float32 and residual.is_contiguous() and tuple(residual.shape) == (B, Do)
     out = torch.empty(B, Do, dtype=torch.float32, device=tables.device)
     lib = _lib.load()
-    if tables.dtype not in (torch.float32, torch.bfloat16):
-        raise NotImplementedError(f"lookup_gather: table dtype {tables.dtype} (float32 and bfloat16 are built)")
-    bf16 = tables.dtype == torch.bfloat16
-    # a few thousand tokens: the table-split form, which wants a workspace for its partial outputs
+    fmt = row_format(tables.dtype)
+    if fmt is None:
+        raise NotImplementedError(f"lookup_gather: table dtype {tables.dtype} (float32, bfloat16 and float16 are built)")
+    # many tokens: the four-lanes-per-token form, which wants a workspace for its record stream; a few
+    # thousand: the table-split form, which wants one for its partial outputs
     ws_bytes = ctypes.c_int64(0)
-    _lib.check(lib.lffn_lookup_gather_workspace_bytes(B, T, S, Do, int(bf16), ctypes.byref(ws_bytes)),
+    _lib.check(lib.lffn_lookup_gather_workspace_bytes(B, T, S, Do, fmt, ctypes.byref(ws_bytes)),
                "lffn_lookup_gather_workspace_bytes")
+    sfx = ("f32", "bf16", "f16")[fmt]
     with _dev_guard(tables):
-        if ws_bytes.value > 0:
-            fn, name = (lib.lffn_lookup_gather_ws_bf16, "lffn_lookup_gather_ws_bf16") if bf16 else \
-                (lib.lffn_lookup_gather_ws_f32, "lffn_lookup_gather_ws_f32")
-            ws = torch.empty(ws_bytes.value, dtype=torch.uint8, device=tables.device)
-            rc = fn(_lib.ptr(code), _lib.ptr(score), _lib.ptr(tables), _lib.ptr(bias), _lib.ptr(residual), _lib.ptr(out),
-                    _lib.ptr(ws), ws_bytes.value, B, T, S, Do, _lib.stream_of(tables))
+        if ws_bytes.value > 0 or fmt == ROWS_F16:
+            name = "lffn_lookup_gather_ws_" + sfx
+            ws = torch.empty(ws_bytes.value, dtype=torch.uint8, device=tables.device) if ws_bytes.value > 0 else None
+            rc = getattr(lib, name)(_lib.ptr(code), _lib.ptr(score), _lib.ptr(tables), _lib.ptr(bias), _lib.ptr(residual),
+                                    _lib.ptr(out), _lib.ptr(ws), ws_bytes.value, B, T, S, Do, _lib.stream_of(tables))
         else:
-            fn, name = (lib.lffn_lookup_gather_residual_bf16, "lffn_lookup_gather_residual_bf16") if bf16 else \
-                (lib.lffn_lookup_gather_residual_f32, "lffn_lookup_gather_residual_f32")
-            rc = fn(_lib.ptr(code), _lib.ptr(score), _lib.ptr(tables), _lib.ptr(bias), _lib.ptr(residual), _lib.ptr(out),
-                    B, T, S, Do, _lib.stream_of(tables))
+            name = "lffn_lookup_gather_residual_" + sfx
+            rc = getattr(lib, name)(_lib.ptr(code), _lib.ptr(score), _lib.ptr(tables), _lib.ptr(bias), _lib.ptr(residual),
+                                    _lib.ptr(out), B, T, S, Do, _lib.stream_of(tables))
     _lib.check(rc, f"{name}(B={B}, T={T}, S={S}, Do={Do})")
     return out
 

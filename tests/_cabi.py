@@ -218,12 +218,15 @@ def code_score_bwd(z, g):
     return host(out)
 
 
-def gather_add(idx, src, w, bf16=False):
+def gather_add(idx, src, w, bf16=False, fmt=None):
+    """fmt (ROWS_*) overrides bf16; 16-bit rows are given as uint16 bit patterns."""
     idd, sd, wd = dev(idx), dev(src), dev(w)
     B, I = idx.shape
     S, Dv = src.shape
     out = torch.full((B, Dv), float("nan"), dtype=torch.float32, device=DEV)
-    _call("lffn_gather_add_bf16" if bf16 else "lffn_gather_add_f32", p(idd), p(sd), p(wd), p(out), B, I, S, Dv)
+    if fmt is None:
+        fmt = ROWS_BF16 if bf16 else ROWS_F32
+    _call(("lffn_gather_add_f32", "lffn_gather_add_bf16", "lffn_gather_add_f16")[fmt], p(idd), p(sd), p(wd), p(out), B, I, S, Dv)
     return host(out)
 
 
@@ -251,6 +254,7 @@ def lookup_gather(code, score, tables, bias=None, bf16=False, plan=None, residua
 
 
 def lookup_gather_workspace_bytes(B, T, S, Do, bf16=False):
+    """bf16: False / True, or a row format (ROWS_*)."""
     n = ctypes.c_int64(-1)
     assert _lib.load().lffn_lookup_gather_workspace_bytes(B, T, S, Do, int(bf16), ctypes.byref(n)) == 0
     return n.value
@@ -286,6 +290,65 @@ def lookup_gather_ws_planned(code, score, tables, plan, bias=None, residual=None
                                                        ws_bytes, B, T, S, Do, plan[0], plan[1], None)
     torch.cuda.synchronize()
     return rc, host(out)
+
+
+ROWS_F32, ROWS_BF16, ROWS_F16 = 0, 1, 2
+
+
+def rows_of(tables_f32, fmt):
+    """fp32 tables in the row format `fmt`: (what the kernel is given, the values it multiplies as float64)."""
+    import oracle
+    if fmt == ROWS_F32:
+        return tables_f32, tables_f32.astype(np.float64)
+    if fmt == ROWS_BF16:
+        bits = oracle.bf16_round(tables_f32.reshape(-1, tables_f32.shape[-1])).reshape(tables_f32.shape)
+        return bits, oracle.bf16_widen(bits.reshape(-1, bits.shape[-1])).reshape(bits.shape).astype(np.float64)
+    half = tables_f32.astype(np.float16)
+    return half.view(np.uint16), half.astype(np.float64)
+
+
+def lookup_gather_ws_planned_rows(code, score, tables, fmt, plan, bias=None, residual=None, ws_bytes=None):
+    """lffn_lookup_gather_ws_planned_rows: exactly the kernel `plan` on rows of format `fmt` (tables: fp32, or
+    uint16 bit patterns of bfloat16 / half).  Returns (status, output)."""
+    cd, sd, td, bd = dev(code), dev(score), dev(tables), dev(bias)
+    rd = None if residual is None else dev(residual)
+    B, T = code.shape
+    _, S, Do = tables.shape
+    if ws_bytes is None:
+        ws_bytes = 6 * T * (B + 2048)
+    ws = torch.full((max(ws_bytes, 16) // 4,), float("nan"), dtype=torch.float32, device=DEV)
+    out = torch.full((B, Do), float("nan"), dtype=torch.float32, device=DEV)
+    rc = _lib.load().lffn_lookup_gather_ws_planned_rows(p(cd), p(sd), p(td), p(bd), p(rd), p(out), p(ws) if ws_bytes else None,
+                                                        ws_bytes, B, T, S, Do, fmt, plan[0], plan[1], None)
+    torch.cuda.synchronize()
+    return rc, host(out)
+
+
+def lookup_gather_ws_f16(code, score, tables_bits, bias=None, residual=None, ws_bytes=None):
+    cd, sd, td, bd = dev(code), dev(score), dev(tables_bits), dev(bias)
+    rd = None if residual is None else dev(residual)
+    B, T = code.shape
+    _, S, Do = tables_bits.shape
+    if ws_bytes is None:
+        ws_bytes = lookup_gather_workspace_bytes(B, T, S, Do, ROWS_F16)
+    ws = torch.full((max(ws_bytes, 16) // 4,), float("nan"), dtype=torch.float32, device=DEV)
+    out = torch.full((B, Do), float("nan"), dtype=torch.float32, device=DEV)
+    _call("lffn_lookup_gather_ws_f16", p(cd), p(sd), p(td), p(bd), p(rd), p(out), p(ws) if ws_bytes else None, ws_bytes,
+          B, T, S, Do)
+    return host(out)
+
+
+def lookup_gather_ws_plan(B, T, S, Do, fmt=0, ws_bytes=1 << 40):
+    form = ctypes.c_int32(-1)
+    tokens = _lib.load().lffn_lookup_gather_ws_plan(B, T, S, Do, fmt, ws_bytes, ctypes.byref(form))
+    return form.value, tokens
+
+
+def lookup_gather_records_plan_rows(B, T, S, Do, fmt):
+    tokens, stride, nbytes = ctypes.c_int32(-1), ctypes.c_int64(-1), ctypes.c_int64(-1)
+    assert _lib.load().lffn_lookup_gather_records_plan_rows(B, T, S, Do, fmt, ctypes.byref(tokens), ctypes.byref(stride),
+                                                            ctypes.byref(nbytes)) == 0
+    return tokens.value, stride.value, nbytes.value
 
 
 def lookup_gather_records_plan(B, T, S, Do):

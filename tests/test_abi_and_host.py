@@ -178,7 +178,11 @@ def test_workspace_queries_are_host_side_plans():
     for shape in ((16384, 128, 128, 768), (256, 32, 256, 256), (4096, 16, 256, 768),
                   (2048, 128, 512, 768), (2048, 128, 256, 100), (0, 128, 256, 768)):
         assert gather_ws(*shape) == 0, shape
-    assert gather_ws(16384, 128, 256, 768, 1) == 0 and gather_ws(65536, 128, 256, 768, 1) == 0      # bf16 rows
+    # 16-bit rows (1 bfloat16, 2 half): the record stream as well, from 16384 tokens on at these tables
+    for fmt in (1, 2):
+        assert gather_ws(16384, 128, 256, 768, fmt) == 64 * (16384 + 2048) * 12
+        assert gather_ws(16384, 512, 256, 1024, fmt) == 256 * (16384 + 2048) * 12
+        assert gather_ws(8192, 128, 256, 768, fmt) == 0
     # many tokens, fp32 rows, 256-row tables, an even number of them: the four-lanes-per-token kernel, which
     # wants 12 bytes per (token, table pair) for its record stream (whole token tiles: up to 2048 tokens more)
     assert gather_ws(16384, 128, 256, 768) == 64 * (16384 + 2048) * 12
@@ -199,6 +203,21 @@ def test_workspace_queries_are_host_side_plans():
     assert plan(8192, 128, 256, 768) == (2, 1024)               # fewer tokens: two tables per buffer
     assert plan(256, 32, 256, 256) == (0, 0)                    # too few tokens to stage tables: token-major
     assert plan(16384, 128, 512, 768) == (0, 0)                 # tables too long for the LDS buffers
+    # what the workspace entry points run, given a workspace: (form, tokens per workgroup); form 3 = four lanes
+    # per token from a record stream, 4 = table split
+    def ws_plan(B, T, S, Do, fmt=0, ws=1 << 40):
+        form = ctypes.c_int32(-1)
+        tokens = lib.lffn_lookup_gather_ws_plan(B, T, S, Do, fmt, ws, ctypes.byref(form))
+        return form.value, tokens
+
+    assert ws_plan(16384, 128, 256, 768) == (3, 1792)           # RoBERTa-base: 10 tiles x 24 slices
+    assert ws_plan(16384, 512, 256, 1024) == (3, 2048)
+    assert ws_plan(16384, 512, 256, 1024, 1) == (3, 1024) and ws_plan(16384, 512, 256, 1024, 2) == (3, 1024)
+    assert ws_plan(16384, 128, 256, 768, 0, 0) == plan(16384, 128, 256, 768)       # no workspace: the plain entry's kernel
+    assert ws_plan(2048, 128, 256, 768) == (4, 512)             # table split
+    assert ws_plan(2048, 128, 256, 768, 2) == (0, 0)            # half rows, few tokens: token-major
+    assert ws_plan(256, 32, 256, 256) == (0, 0)
+    assert lib.lffn_lookup_gather_ws_plan(16384, 128, 256, 768, 3, 0, None) == _lib.LFFN_ERR_BAD_ARG
     # sorted scatter: pairs + offsets + transposed codes and scores + packed gradient, for at most 16384 tokens
     one = scatter_ws(16384, 128, 256, 768)
     assert one >= 16384 * 128 * 8 + 16384 * 768 * 4

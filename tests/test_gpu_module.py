@@ -88,11 +88,14 @@ def test_layer_forward_eval_matches_oracle(H, T, Do, bs):
 # (tokens as batch x sequence, hidden, tables, columns, block size): BASELINE.json configs 2 and 3, and config 2 with the
 # reference's shipped block size; all take the many-token path (projection kernel writing the record stream,
 # four-lanes-per-token gather)
-MANY_TOKEN_LAYERS = [((32, 512), 768, 128, 768, 1), ((32, 512), 1024, 512, 1024, 1), ((32, 512), 768, 128, 768, 64)]
+MANY_TOKEN_LAYERS = [((32, 512), 768, 128, 768, 1, torch.float32), ((32, 512), 1024, 512, 1024, 1, torch.float32),
+                     ((32, 512), 768, 128, 768, 64, torch.float32),
+                     # config 3 with 16-bit tables (bfloat16; half, the reference's reduced-precision row format)
+                     ((32, 512), 1024, 512, 1024, 1, torch.bfloat16), ((32, 512), 1024, 512, 1024, 1, torch.float16)]
 
 
-@pytest.mark.parametrize("shape,H,T,Do,bs", MANY_TOKEN_LAYERS)
-def test_layer_forward_eval_many_tokens_matches_oracle(shape, H, T, Do, bs):
+@pytest.mark.parametrize("shape,H,T,Do,bs,tdtype", MANY_TOKEN_LAYERS)
+def test_layer_forward_eval_many_tokens_matches_oracle(shape, H, T, Do, bs, tdtype):
     """LookupFFN.eval() at 16384 tokens: the record-stream path of LookupFFN._forward_inference, on a sample of
     tokens against the oracle."""
     from lookupffn_amd import ops
@@ -101,8 +104,9 @@ def test_layer_forward_eval_many_tokens_matches_oracle(shape, H, T, Do, bs):
     layer = lookupffn_amd.LookupFFN(_config(hidden_size=H, ffn_num_table=T, block_size=bs), Do).eval().to(DEV)
     with torch.no_grad():
         layer.hash.projection.bias.normal_(0, 0.05)
+    layer.tables.data = layer.tables.data.to(tdtype)
     B = shape[0] * shape[1]
-    assert ops.lookup_gather_records_plan(B, T, S, Do) is not None         # this shape takes the record stream
+    assert ops.lookup_gather_records_plan(B, T, S, Do, ops.row_format(tdtype)) is not None     # this shape takes the record stream
     x = torch.randn(*shape, H, device=DEV) * 1.5 + 0.3
     with torch.no_grad():
         out = layer(x)
@@ -277,6 +281,26 @@ def test_bf16_tables_inference():
         out = layer(x)
     assert out.dtype == torch.float32
     assert relmax(npf(out), npf(ref)) <= 1e-2
+
+
+def test_f16_tables_inference_and_general_gather():
+    """Half rows, the row format of the reference's reduced-precision kernels (gather_kernel_fp16.cu), with fp32
+    sums: the layer at a small batch (token-major kernel) and weighted_gather_add on arbitrary indices."""
+    torch.manual_seed(8)
+    layer = lookupffn_amd.LookupFFN(_config(), 128).eval().to(DEV)
+    x = torch.randn(40, 192, device=DEV)
+    with torch.no_grad():
+        ref = layer(x)
+        layer.tables.data = layer.tables.data.to(torch.float16)
+        out = layer(x)
+    assert out.dtype == torch.float32 and relmax(npf(out), npf(ref)) <= 1e-2
+    rng = np.random.RandomState(8)
+    src = torch.tensor((0.02 * rng.randn(500, 192)).astype(np.float16), device=DEV)
+    idx_np = rng.randint(0, 500, size=(77, 6)).astype(np.int32)
+    w = torch.tensor((1 - rng.rand(77, 6)).astype(np.float32), device=DEV)
+    got = lookupffn_amd.weighted_gather_add(torch.tensor(idx_np, device=DEV), src, w)
+    want = oracle.gather_add(idx_np, npf(src).astype(np.float64), npf(w).astype(np.float64))
+    assert got.dtype == torch.float32 and relmax(npf(got), want) <= 1e-5
 
 
 def test_reference_call_sequence_of_lookup_gather():

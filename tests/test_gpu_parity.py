@@ -887,8 +887,10 @@ def test_lookup_gather_workspace_query_is_zero_where_the_plain_form_is_as_fast()
     for shape in ((16384, 32, 256, 768), (8, 128, 256, 768), (4096, 16, 256, 768), (0, 4, 16, 64),
                   (16384, 128, 128, 768), (16384, 127, 256, 768)):
         assert cabi.lookup_gather_workspace_bytes(*shape) == 0, shape
-    for shape in ((16384, 128, 256, 768), (65536, 128, 256, 768), (16384, 512, 256, 1024)):
+    for shape in ((8192, 128, 256, 768), (16384, 32, 256, 768), (16384, 128, 128, 768)):
         assert cabi.lookup_gather_workspace_bytes(*shape, bf16=True) == 0, shape
+    for shape in ((8192, 128, 256, 768), (2048, 32, 256, 768), (16384, 128, 128, 768)):     # half rows: token-major there
+        assert cabi.lookup_gather_workspace_bytes(*shape, bf16=cabi.ROWS_F16) == 0, shape
 
 
 # The four-lanes-per-token kernel (form 3), every tile size that is built, forced onto shapes it would not
@@ -914,6 +916,51 @@ def test_lookup_gather_quad_kernels_match_oracle(B, T, S, Do, plan):
     assert np.array_equal(cabi.lookup_gather_ws_planned(dirty, w, tables, plan, bias=bias)[1], got)
     rc, got_r = cabi.lookup_gather_ws_planned(code, w, tables, plan, residual=res)
     assert rc == 0 and relmax(got_r, want - bias + res) <= 1e-5
+
+
+# The same kernel on 16-bit rows (bfloat16 and half, fp32 sums): 64-column slices, 1024 tokens per workgroup
+QUAD16_SHAPES = [(3000, 20, 256, 256), (4133, 6, 256, 384), (1793, 34, 256, 128), (1, 2, 256, 64), (2050, 8, 256, 192)]
+
+
+@pytest.mark.parametrize("fmt", [cabi.ROWS_BF16, cabi.ROWS_F16])
+@pytest.mark.parametrize("B,T,S,Do", QUAD16_SHAPES)
+def test_lookup_gather_quad_kernels_16bit_rows_match_oracle(B, T, S, Do, fmt):
+    rng = np.random.RandomState(B + T + S + Do + fmt)
+    tables, code, idx, w = _rand_gather(rng, B, T, S, Do)
+    bias = (0.001 * rng.randn(Do)).astype(np.float32)
+    res = rng.randn(B, Do).astype(np.float32)
+    bits, wide = cabi.rows_of(tables, fmt)
+    rc, got = cabi.lookup_gather_ws_planned_rows(code, w, bits, fmt, (3, 1024), bias=bias)
+    assert rc == 0 and not np.isnan(got).any()
+    # the float64 sum over the 16-bit values the kernel reads: fp32 accumulation, 1e-5
+    want = oracle.gather_add(idx, wide.reshape(T * S, Do), w.astype(np.float64)) + bias
+    assert relmax(got, want) <= 1e-5
+    # and 1e-2 against the sum over the fp32 values the rows were rounded from
+    assert relmax(got, oracle.gather_add(idx, tables.reshape(T * S, Do).astype(np.float64), w.astype(np.float64)) + bias) <= 1e-2
+    # every token against the token-major kernel on the same rows
+    tm = cabi.gather_add(idx, bits.reshape(T * S, Do), w, fmt=fmt)
+    assert relmax(got, tm.astype(np.float64) + bias) <= 2e-6
+    dirty = (code + S * rng.randint(0, 5, size=code.shape)).astype(np.int32)      # bits above log2(S) are ignored
+    assert np.array_equal(cabi.lookup_gather_ws_planned_rows(dirty, w, bits, fmt, (3, 1024), bias=bias)[1], got)
+    rc, got_r = cabi.lookup_gather_ws_planned_rows(code, w, bits, fmt, (3, 1024), residual=res)
+    assert rc == 0 and relmax(got_r, want - bias + res) <= 1e-5
+    if fmt == cabi.ROWS_BF16:
+        assert relmax(got, oracle.gather_add_bf16(idx, bits.reshape(T * S, Do), w) + bias) <= 1e-5
+
+
+def test_lookup_gather_quad_16bit_refusals():
+    from lookupffn_amd import _lib
+    rng = np.random.RandomState(5)
+    tables, code, idx, w = _rand_gather(rng, 300, 20, 256, 64)
+    for fmt in (cabi.ROWS_BF16, cabi.ROWS_F16):
+        bits, _ = cabi.rows_of(tables, fmt)
+        assert cabi.lookup_gather_ws_planned_rows(code, w, bits, fmt, (3, 2048))[0] == _lib.LFFN_ERR_UNSUPPORTED   # 8 passes: fp32 rows only
+        assert cabi.lookup_gather_ws_planned_rows(code, w, bits, fmt, (3, 1024), ws_bytes=0)[0] == _lib.LFFN_ERR_UNSUPPORTED
+        assert cabi.lookup_gather_ws_planned_rows(code, w, bits, 3, (3, 1024))[0] == _lib.LFFN_ERR_BAD_ARG          # no such row format
+    half, _ = cabi.rows_of(tables, cabi.ROWS_F16)
+    assert cabi.lookup_gather_ws_planned_rows(code, w, half, cabi.ROWS_F16, (1, 256))[0] == _lib.LFFN_ERR_UNSUPPORTED   # not built for half rows
+    rc, got = cabi.lookup_gather_ws_planned_rows(code, w, half, cabi.ROWS_F16, (0, 0))
+    assert rc == 0 and np.array_equal(got, cabi.gather_add(idx, half.reshape(20 * 256, 64), w, fmt=cabi.ROWS_F16))
 
 
 def test_lookup_gather_quad_refusals():
@@ -1438,36 +1485,51 @@ def test_config3_gather_full_size(config3, bf16):
     assert np.array_equal(got, cabi.lookup_gather(c["code"], c["w"], src.reshape(T, S, Do), c["bias"], bf16=bf16))
 
 
-def test_config3_gather_record_stream_full_size(config3):
-    """Config 3 through the form the layer and bench.py run there: lffn_lookup_gather_ws_f32 packs the record
-    stream and launches the four-lanes-per-token kernel (2048-token tiles, 256 table pairs, 4 KB rows)."""
+@pytest.mark.parametrize("fmt", [cabi.ROWS_F32, cabi.ROWS_BF16, cabi.ROWS_F16])
+def test_config3_gather_record_stream_full_size(config3, fmt):
+    """Config 3 through the form the layer and bench.py run there: lffn_lookup_gather_ws_* packs the record
+    stream and launches the four-lanes-per-token kernel (fp32 rows: 2048-token tiles over 32 slices; bfloat16
+    and half rows: 1024-token tiles over 16 slices of 64 columns; 256 table pairs)."""
     c = config3
     B, T, S, Do = c["B"], c["T"], c["S"], c["Do"]
-    nbytes = cabi.lookup_gather_workspace_bytes(B, T, S, Do)
+    nbytes = cabi.lookup_gather_workspace_bytes(B, T, S, Do, fmt)
     assert nbytes > 0 and nbytes % 12 == 0 and nbytes < B * Do * 4            # the record stream, not the table split
-    assert cabi.lookup_gather_records_plan(B, T, S, Do) == CONFIG3_RECORD_PLAN
-    flat = c["tables"].reshape(T * S, Do)
-    got = cabi.lookup_gather_ws(c["code"], c["w"], c["tables"], c["bias"])
+    tokens = CONFIG3_RECORD_PLAN[0] if fmt == cabi.ROWS_F32 else 1024
+    assert cabi.lookup_gather_records_plan_rows(B, T, S, Do, fmt) == (tokens, 16384, 6 * T * 16384)
+    assert cabi.lookup_gather_ws_plan(B, T, S, Do, fmt, nbytes) == (3, tokens)
+    bits, _ = cabi.rows_of(c["tables"], fmt)
+    flat = bits.reshape(T * S, Do)
+    widen = {cabi.ROWS_F32: lambda r: r, cabi.ROWS_BF16: oracle.bf16_widen, cabi.ROWS_F16: lambda r: r.view(np.float16)}[fmt]
+
+    def ws_entry(residual=None):
+        if fmt == cabi.ROWS_F16:
+            return cabi.lookup_gather_ws_f16(c["code"], c["w"], bits, c["bias"], residual=residual)
+        return cabi.lookup_gather_ws(c["code"], c["w"], bits, c["bias"], bf16=fmt == cabi.ROWS_BF16, residual=residual)
+    got = ws_entry()
     assert not np.isnan(got).any()
     sub = c["sub"]
-    rows, ridx = _rows64(flat, c["idx"][sub])
-    want = oracle.gather_add(ridx, rows, c["w"][sub].astype(np.float64)) + c["bias"]
+    uniq, inv = np.unique(c["idx"][sub], return_inverse=True)
+    ridx = inv.reshape(c["idx"][sub].shape).astype(np.int32)
+    want = oracle.gather_add(ridx, widen(flat[uniq]).astype(np.float64), c["w"][sub].astype(np.float64)) + c["bias"]
     assert relmax(got[sub], want) <= 1e-5
-    # every token against the plain entry point (same rows; the two tables of a pair added in either order)
-    assert relmax(got, cabi.lookup_gather(c["code"], c["w"], c["tables"], c["bias"])) <= 2e-6
+    if fmt != cabi.ROWS_F32:        # against the fp32 rows the 16-bit ones were rounded from
+        rows32, _ = _rows64(c["tables"].reshape(T * S, Do), c["idx"][sub])
+        assert relmax(got[sub], oracle.gather_add(ridx, rows32, c["w"][sub].astype(np.float64)) + c["bias"]) <= 1e-2
+    # every token against the token-major kernel on the same rows (the two tables of a pair added in either order)
+    assert relmax(got, cabi.gather_add(c["idx"], flat, c["w"], fmt=fmt).astype(np.float64) + c["bias"]) <= 2e-6
     # checksum over all tokens: sum_b out[b] = B * bias + sum_{t,s} cnt[t,s] * tables[t,s]
     want_sum = B * c["bias"].astype(np.float64)
     for t0 in range(0, T, 64):
-        want_sum = want_sum + np.einsum("ts,tsd->d", c["cnt"][t0:t0 + 64], flat[t0 * S:(t0 + 64) * S].reshape(64, S, Do).astype(np.float64))
+        want_sum = want_sum + np.einsum("ts,tsd->d", c["cnt"][t0:t0 + 64],
+                                        widen(flat[t0 * S:(t0 + 64) * S]).reshape(64, S, Do).astype(np.float64))
     assert relmax(got.astype(np.float64).sum(0), want_sum) <= 1e-5
     # a second launch gives the same bits; so does the same tile size named explicitly
-    assert np.array_equal(got, cabi.lookup_gather_ws(c["code"], c["w"], c["tables"], c["bias"]))
-    rc, forced = cabi.lookup_gather_ws_planned(c["code"], c["w"], c["tables"], (3, CONFIG3_RECORD_PLAN[0]), bias=c["bias"])
+    assert np.array_equal(got, ws_entry())
+    rc, forced = cabi.lookup_gather_ws_planned_rows(c["code"], c["w"], bits, fmt, (3, tokens), bias=c["bias"])
     assert rc == 0 and np.array_equal(got, forced)
     # the residual goes into the store: the same sums plus the residual, rounded once more
     res = np.random.default_rng(36).standard_normal((B, Do), dtype=np.float32)
-    got_r = cabi.lookup_gather_ws(c["code"], c["w"], c["tables"], c["bias"], residual=res)
-    assert np.array_equal(got_r, got + res)
+    assert np.array_equal(ws_entry(residual=res), got + res)
 
 
 def test_config3_inner_product_full_size(config3):
