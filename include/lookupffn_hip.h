@@ -602,6 +602,26 @@ int lffn_lookup_scatter_sorted_f32(const int32_t *code, const float *score, cons
                                    int64_t Do, int32_t accumulate, void *stream);
 
 /*
+ * Both gradients of the layer's gather in one call, sharing one workspace (the size
+ * lffn_lookup_scatter_workspace_bytes reports; the call is refused where that is 0):
+ *   grad_score[b, t]     = < g[b, :], tables[t, code[b,t] & (S-1), :] >                       overwritten
+ *   grad_tables[t, s, :] = sum over the tokens b with code[b,t] = s of score[b,t] * g[b, :]   overwritten,
+ *                                                                     or added to when accumulate != 0
+ * i.e. lffn_lookup_inner_f32 and lffn_lookup_scatter_sorted_f32 with their common work done once: per
+ * chunk of 16384 tokens one kernel transposes code and score and copies g slice-major, and the
+ * score-gradient kernel and the sorted scatter both read that copy (for the score gradient, a token
+ * tile's slice of g is then contiguous instead of one 128-byte line per row).  Results are bit-identical
+ * to the two separate calls.  grad_score or grad_tables may be NULL (that gradient is not computed; tables
+ * is needed for the former only, score for the latter only).  Do % 64 == 0, S <= 512.
+ * Replaces WeightedVectorGatherAdd.backward (PL/gather/cuda/kernel.py:190-202: indexed_inner_product +
+ * weighted_vector_scatter_add, kernels gather_kernel_fp32.cu:49-157) with the index offset of
+ * PL/lookup.py:126.
+ */
+int lffn_lookup_backward_f32(const int32_t *code, const float *score, const float *g, const float *tables,
+                             float *grad_score, float *grad_tables, void *workspace, int64_t workspace_bytes,
+                             int64_t B, int64_t T, int64_t S, int64_t Do, int32_t accumulate, void *stream);
+
+/*
  * The indexed inner product as the layer's backward issues it: table-local codes,
  *   grad_score[b, t] = < g[b, :], tables[t, code[b,t] & (S-1), :] >
  * code: [B, T] int32; g: [B, Do]; tables: [T, S, Do] fp32; grad_score: [B, T],

@@ -91,6 +91,7 @@ SIGNATURES = {
     "lffn_lookup_scatter_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, ctypes.c_int32, _vp],
     "lffn_lookup_scatter_workspace_bytes": [_i64, _i64, _i64, _i64, ctypes.POINTER(ctypes.c_int64)],
     "lffn_lookup_scatter_sorted_f32": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, ctypes.c_int32, _vp],
+    "lffn_lookup_backward_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, ctypes.c_int32, _vp],
     "lffn_lookup_inner_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
 }
 

@@ -98,6 +98,12 @@ int lffn_internal_lookup_gather_quad_records(const uint32_t *records, int64_t re
                                              const float *bias, const float *residual, float *out, int64_t B,
                                              int64_t T, int64_t S, int64_t Do, int fmt, int np, void *stream);
 
+// lookup_inner.hip: the four-lanes-per-token score gradient where the shape qualifies (not exported)
+__attribute__((visibility("hidden")))
+bool lffn_internal_lookup_inner_quad_try(const int32_t *code, const float *g, int64_t g_token_stride,
+                                         int64_t g_slice_stride, const void *tables, float *grad_score, int64_t B,
+                                         int64_t T, int64_t S, int64_t Do, void *stream, int *rc);
+
 // lookup_inner_quad.hip: the score gradient with four lanes per token and one owner per (token, table) (not exported)
 __attribute__((visibility("hidden")))
 int lffn_internal_lookup_inner_quad(const int32_t *code, const float *g, int64_t g_token_stride, int64_t g_slice_stride,

@@ -247,6 +247,24 @@ int launch_inner(const InnerArgs &a, hipStream_t stream) {
 
 }  // namespace
 
+// The four-lanes-per-token kernel (lookup_inner_quad.hip) where the shape qualifies: S = 256, T even, tiles of
+// 1024 tokens x chunks of 4 or 2 table pairs; 4 when that still gives the chip a round of workgroups (the g
+// values are fetched once per chunk and slice), 2 otherwise, and not at all when even 2 leaves most of the chip
+// idle.  g: token b's 32 columns of slice s at g + b * g_token_stride + s * g_slice_stride floats.  Returns
+// false when the shape does not qualify (nothing launched), true with the launch status in *rc otherwise.
+bool lffn_internal_lookup_inner_quad_try(const int32_t *code, const float *g, int64_t g_token_stride,
+                                         int64_t g_slice_stride, const void *tables, float *grad_score, int64_t B,
+                                         int64_t T, int64_t S, int64_t Do, void *stream, int *rc) {
+    if (!(S == MAX_S && T % 2 == 0 && Do % 32 == 0 && B >= 1 && reinterpret_cast<uintptr_t>(code) % 8 == 0 &&
+          2 * S * Do * 4 < (int64_t(1) << 32)))
+        return false;
+    const int64_t tiles = (B + 1023) / 1024, pairs = T / 2;
+    const int c = tiles * ((pairs + 3) / 4) >= 200 ? 4 : (tiles * ((pairs + 1) / 2) >= 96 ? 2 : 0);
+    if (!c || tiles * ((pairs + c - 1) / c) > (int64_t(1) << 30)) return false;
+    *rc = lffn_internal_lookup_inner_quad(code, g, g_token_stride, g_slice_stride, tables, grad_score, B, T, S, Do, 4, c, stream);
+    return true;
+}
+
 extern "C" int lffn_lookup_inner_f32(const int32_t *code, const float *g, const float *tables, float *grad_score,
                                      int64_t B, int64_t T, int64_t S, int64_t Do, void *stream) {
     LFFN_REQUIRE(B >= 0 && T >= 0 && Do >= 1, LFFN_ERR_BAD_ARG);
@@ -261,10 +279,9 @@ extern "C" int lffn_lookup_inner_f32(const int32_t *code, const float *g, const 
     // Four lanes per token, one owner per (token, table) (lookup_inner_quad.hip): tiles of 1024 tokens x
     // chunks of 4 or 2 table pairs; 4 when that still gives the chip a round of workgroups (the g values are
     // fetched once per chunk and slice), and the form below when even 2 leaves most of it idle.
-    if (S == MAX_S && T % 2 == 0 && reinterpret_cast<uintptr_t>(code) % 8 == 0 && 2 * S * Do * 4 < (int64_t(1) << 32)) {
-        const int64_t tiles = (B + 1023) / 1024, pairs = T / 2;
-        const int c = tiles * ((pairs + 3) / 4) >= 200 ? 4 : (tiles * ((pairs + 1) / 2) >= 96 ? 2 : 0);
-        if (c && tiles * ((pairs + c - 1) / c) <= (int64_t(1) << 30)) return lffn_internal_lookup_inner_quad(code, g, Do, 32, tables, grad_score, B, T, S, Do, 4, c, stream);
+    {
+        int rc = LFFN_OK;
+        if (lffn_internal_lookup_inner_quad_try(code, g, Do, 32, tables, grad_score, B, T, S, Do, stream, &rc)) return rc;
     }
 
     // LDS form: table fits the buffers, and enough (token tile, slice) units to fill most CUs

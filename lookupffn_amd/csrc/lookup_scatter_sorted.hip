@@ -410,14 +410,14 @@ extern "C" int lffn_lookup_scatter_workspace_bytes(int64_t B, int64_t T, int64_t
     return LFFN_OK;
 }
 
-extern "C" int lffn_lookup_scatter_sorted_f32(const int32_t *code, const float *score, const float *g,
-                                              float *grad_tables, void *workspace, int64_t workspace_bytes,
-                                              int64_t B, int64_t T, int64_t S, int64_t Do, int32_t accumulate,
-                                              void *stream) {
-    LFFN_REQUIRE(B >= 0 && T >= 0 && S >= 1 && Do >= 1, LFFN_ERR_BAD_ARG);
-    LFFN_REQUIRE(sorted_supported(B, T, S, Do), LFFN_ERR_UNSUPPORTED);
-    LFFN_REQUIRE(code && score && g && grad_tables && workspace, LFFN_ERR_BAD_ARG);
-    LFFN_REQUIRE(lffn_aligned16(grad_tables) && lffn_aligned16(g) && lffn_aligned16(workspace), LFFN_ERR_BAD_ARG);
+namespace {
+
+// The sorted scatter over chunks of CHUNK tokens and, when grad_score is given, the score gradient of each
+// chunk from the same slice-major copy of g the scatter reads (lookup_prep_kernel writes it once per chunk).
+// grad_tables may be null (score gradient only).
+int sorted_backward(const int32_t *code, const float *score, const float *g, const float *tables, float *grad_score,
+                    float *grad_tables, void *workspace, int64_t workspace_bytes, int64_t B, int64_t T, int64_t S,
+                    int64_t Do, int32_t accumulate, void *stream) {
     const Workspace w = workspace_layout(B, T, S, Do);
     LFFN_REQUIRE(workspace_bytes >= w.total, LFFN_ERR_BAD_ARG);
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -436,12 +436,23 @@ extern "C" int lffn_lookup_scatter_sorted_f32(const int32_t *code, const float *
         pa.g_packed = reinterpret_cast<float *>(base + w.g_packed);
         pa.B = Bc; pa.Bp = Bp; pa.T = (int)T; pa.S = (int)S; pa.Do = (int)Do;
         pa.tiles_t = (int)((T + 63) / 64);
-        const int64_t transpose_blocks = (Bp / 64) * pa.tiles_t, pack_blocks = (Bc + PACK_TOKENS - 1) / PACK_TOKENS;
+        // (score gradient only: the codes and scores need no transposing, only g its slice-major copy)
+        const int64_t transpose_blocks = grad_tables ? (Bp / 64) * pa.tiles_t : 0;
+        const int64_t pack_blocks = (Bc + PACK_TOKENS - 1) / PACK_TOKENS;
         LFFN_REQUIRE(transpose_blocks + pack_blocks <= 0x7fffffff, LFFN_ERR_UNSUPPORTED);
         pa.transpose_blocks = (int)transpose_blocks;
         hipLaunchKernelGGL(lookup_prep_kernel, dim3((unsigned)(transpose_blocks + pack_blocks)), dim3(256), 0, st, pa);
         int rc = lffn_launch_status();
         if (rc != LFFN_OK) return rc;
+
+        if (grad_score) {
+            // token b's 32 columns of slice s sit at g_packed + (s * Bc + b) * 32
+            if (!lffn_internal_lookup_inner_quad_try(pa.code, pa.g_packed, SC, Bc * SC, tables, grad_score + c0 * T, Bc, T, S,
+                                                     Do, stream, &rc))
+                rc = lffn_lookup_inner_f32(pa.code, pa.g, tables, grad_score + c0 * T, Bc, T, S, Do, stream);
+            if (rc != LFFN_OK) return rc;
+        }
+        if (!grad_tables) continue;
 
         SortArgs sa{};
         sa.code = pa.code_t; sa.score = pa.score_t; sa.pairs = pairs; sa.off8 = off8;
@@ -463,4 +474,37 @@ extern "C" int lffn_lookup_scatter_sorted_f32(const int32_t *code, const float *
         if (rc != LFFN_OK) return rc;
     }
     return LFFN_OK;
+}
+
+}  // namespace
+
+extern "C" int lffn_lookup_scatter_sorted_f32(const int32_t *code, const float *score, const float *g,
+                                              float *grad_tables, void *workspace, int64_t workspace_bytes,
+                                              int64_t B, int64_t T, int64_t S, int64_t Do, int32_t accumulate,
+                                              void *stream) {
+    LFFN_REQUIRE(B >= 0 && T >= 0 && S >= 1 && Do >= 1, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(sorted_supported(B, T, S, Do), LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(code && score && g && grad_tables && workspace, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_aligned16(grad_tables) && lffn_aligned16(g) && lffn_aligned16(workspace), LFFN_ERR_BAD_ARG);
+    return sorted_backward(code, score, g, nullptr, nullptr, grad_tables, workspace, workspace_bytes, B, T, S, Do, accumulate,
+                           stream);
+}
+
+// Both gradients of the layer's gather in one call with one workspace (lffn_lookup_scatter_workspace_bytes):
+//   grad_score[b,t]  = < g[b,:], tables[t, code[b,t], :] >           (overwritten)
+//   grad_tables[t,s] = sum over b with code[b,t] = s of score[b,t] * g[b,:]   (overwritten, or added to)
+// Per chunk of 16384 tokens: one kernel transposes code and score and copies g slice-major, the score-gradient
+// kernel and the sorted scatter both read that copy.
+extern "C" int lffn_lookup_backward_f32(const int32_t *code, const float *score, const float *g, const float *tables,
+                                        float *grad_score, float *grad_tables, void *workspace,
+                                        int64_t workspace_bytes, int64_t B, int64_t T, int64_t S, int64_t Do,
+                                        int32_t accumulate, void *stream) {
+    LFFN_REQUIRE(B >= 0 && T >= 0 && S >= 1 && Do >= 1, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(sorted_supported(B, T, S, Do) && Do % 64 == 0, LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(code && g && workspace && (grad_score || grad_tables), LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE((!grad_score || tables) && (!grad_tables || score), LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_aligned16(g) && lffn_aligned16(workspace) && (!grad_tables || lffn_aligned16(grad_tables)) &&
+                     (!tables || lffn_aligned16(tables)), LFFN_ERR_BAD_ARG);
+    return sorted_backward(code, score, g, tables, grad_score, grad_tables, workspace, workspace_bytes, B, T, S, Do,
+                           accumulate, stream);
 }

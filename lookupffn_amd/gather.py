@@ -150,8 +150,12 @@ class LookupGather(Function):
             raise NotImplementedError("backward through 16-bit tables is not built (inference formats)")
         grad_outputs = grad_outputs.contiguous()
         T, S, Do = tables.shape
-        grad_score = ops.lookup_inner(code, grad_outputs, tables) if ctx.needs_input_grad[1] else None
-        grad_tables = ops.lookup_scatter(code, score, grad_outputs, S) if ctx.needs_input_grad[2] else None
+        if ctx.needs_input_grad[1] and ctx.needs_input_grad[2]:
+            # one call: the score gradient and the sorted scatter share the slice-major copy of the gradient
+            grad_score, grad_tables = ops.lookup_backward(code, score, grad_outputs, tables)
+        else:
+            grad_score = ops.lookup_inner(code, grad_outputs, tables) if ctx.needs_input_grad[1] else None
+            grad_tables = ops.lookup_scatter(code, score, grad_outputs, S) if ctx.needs_input_grad[2] else None
         grad_bias = ops.column_sums(grad_outputs) if (ctx.has_bias and ctx.needs_input_grad[3]) else None
         grad_residual = grad_outputs if (ctx.has_residual and ctx.needs_input_grad[4]) else None
         return None, grad_score, grad_tables, grad_bias, grad_residual

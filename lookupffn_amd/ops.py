@@ -962,6 +962,53 @@ def _(code, score, g, S):
     return g.new_empty(code.shape[1], S, g.shape[1])
 
 
+_L.define("lookup_backward(Tensor code, Tensor score, Tensor g, Tensor tables) -> (Tensor, Tensor)")
+
+
+def lookup_backward_is_fused(B, T, S, Do):
+    """Both gradients of the gather go through one call (lffn_lookup_backward_f32: the sorted scatter and the
+    score gradient sharing one slice-major copy of g) for this shape."""
+    if B * T * Do < SORTED_SCATTER_MIN_WORK or Do % 64 != 0:
+        return False
+    ws_bytes = ctypes.c_int64(0)
+    _lib.check(_lib.load().lffn_lookup_scatter_workspace_bytes(B, T, S, Do, ctypes.byref(ws_bytes)),
+               "lffn_lookup_scatter_workspace_bytes")
+    return ws_bytes.value > 0
+
+
+def _lookup_backward_impl(code, score, g, tables):
+    """(grad_score [B, T], grad_tables [T, S, Do]) of out = sum_t score * tables[t, code]; g = grad of out."""
+    _lib.require_gpu(code, score, g, tables)
+    assert g.dim() == 2 and g.dtype == torch.float32 and g.is_contiguous()
+    assert score.dtype == torch.float32 and score.is_contiguous() and tuple(score.shape) == tuple(code.shape)
+    assert tables.dim() == 3 and tables.dtype == torch.float32 and tables.is_contiguous()
+    B, T = code.shape
+    Tt, S, Do = tables.shape
+    assert Tt == T and g.shape[0] == B and g.shape[1] == Do and _is_pow2(S)
+    _check_gather_args(code, max(T * S, 1), Do)
+    if not lookup_backward_is_fused(B, T, S, Do):
+        return _lookup_inner_impl(code, g, tables), _lookup_scatter_impl(code, score, g, S)
+    lib = _lib.load()
+    ws_bytes = ctypes.c_int64(0)
+    _lib.check(lib.lffn_lookup_scatter_workspace_bytes(B, T, S, Do, ctypes.byref(ws_bytes)), "lffn_lookup_scatter_workspace_bytes")
+    grad_score = torch.empty(B, T, dtype=torch.float32, device=g.device)          # both fully overwritten
+    grad_tables = torch.empty(T, S, Do, dtype=torch.float32, device=g.device)
+    ws = torch.empty(ws_bytes.value, dtype=torch.uint8, device=g.device)
+    with _dev_guard(g):
+        rc = lib.lffn_lookup_backward_f32(_lib.ptr(code), _lib.ptr(score), _lib.ptr(g), _lib.ptr(tables), _lib.ptr(grad_score),
+                                          _lib.ptr(grad_tables), _lib.ptr(ws), ws_bytes.value, B, T, S, Do, 0, _lib.stream_of(g))
+    _lib.check(rc, f"lffn_lookup_backward_f32(B={B}, T={T}, S={S}, Do={Do})")
+    return grad_score, grad_tables
+
+
+_L.impl("lookup_backward", _lookup_backward_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::lookup_backward")
+def _(code, score, g, tables):
+    return g.new_empty(code.shape[0], code.shape[1]), g.new_empty(tables.shape)
+
+
 _L.define("lookup_inner(Tensor code, Tensor g, Tensor tables) -> Tensor")
 
 
@@ -1011,4 +1058,5 @@ lookup_gather = torch.ops.lookupffn.lookup_gather
 indexed_inner_product = torch.ops.lookupffn.indexed_inner_product
 scatter_add = torch.ops.lookupffn.scatter_add
 lookup_scatter = torch.ops.lookupffn.lookup_scatter
+lookup_backward = torch.ops.lookupffn.lookup_backward
 lookup_inner = torch.ops.lookupffn.lookup_inner

@@ -433,6 +433,23 @@ def lookup_scatter_sorted(code, score, g, S, accumulate=False, init=None):
     return host(out)
 
 
+def lookup_backward(code, score, g, tables, accumulate=False, init=None, want=(True, True)):
+    """lffn_lookup_backward_f32 -> (grad_score [B, T] or None, grad_tables [T, S, Do] or None)."""
+    cd, sd, gd, td = dev(code), dev(score), dev(g), dev(tables)
+    B, T = code.shape
+    _, S, Do = tables.shape
+    nbytes = lookup_scatter_workspace_bytes(B, T, S, Do)
+    assert nbytes > 0
+    ws = torch.full((nbytes // 4,), 0x7f7f7f7f, dtype=torch.int32, device=DEV)      # scratch: any contents
+    gs = torch.full((B, T), float("nan"), dtype=torch.float32, device=DEV) if want[0] else None
+    gt = None
+    if want[1]:
+        gt = torch.full((T, S, Do), float("nan"), dtype=torch.float32, device=DEV) if init is None else dev(init)
+    _call("lffn_lookup_backward_f32", p(cd), p(sd), p(gd), p(td), p(gs), p(gt), p(ws), nbytes, B, T, S, Do,
+          1 if accumulate else 0)
+    return (None if gs is None else host(gs)), (None if gt is None else host(gt))
+
+
 def lookup_inner(code, g, tables):
     cd, gd, td = dev(code), dev(g), dev(tables)
     B, T = code.shape

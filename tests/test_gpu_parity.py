@@ -1320,6 +1320,65 @@ def test_lookup_scatter_sorted_full_size_zipf():
     assert relmax(got, cabi.lookup_scatter(code, w, g, S)) <= 1e-5                # the LDS form
 
 
+BACKWARD_CASES = [(256, 32, 256, 256), (65, 5, 256, 192), (4100, 16, 256, 768), (3000, 6, 64, 128), (2050, 3, 512, 64)]
+
+
+@pytest.mark.parametrize("B,T,S,Do", BACKWARD_CASES)
+def test_lookup_backward_matches_oracle_and_the_separate_entry_points(B, T, S, Do):
+    """lffn_lookup_backward_f32: both gradients from one call and one workspace, against the float64 oracle and,
+    bit for bit, against lffn_lookup_inner_f32 and lffn_lookup_scatter_sorted_f32."""
+    rng = np.random.RandomState(B + T + S + Do)
+    tables, code, idx, w = _rand_gather(rng, B, T, S, Do)
+    g = rng.randn(B, Do).astype(np.float32)
+    gs, gt = cabi.lookup_backward(code, w, g, tables)
+    assert not np.isnan(gs).any() and not np.isnan(gt).any()
+    flat = tables.reshape(T * S, Do)
+    assert relmax(gs, oracle.indexed_inner_product(idx, g.astype(np.float64), flat.astype(np.float64))) <= 1e-5
+    assert relmax(gt.reshape(T * S, Do), oracle.scatter_add(idx, g.astype(np.float64), w.astype(np.float64), T * S)) <= 1e-5
+    assert np.array_equal(gt, cabi.lookup_scatter_sorted(code, w, g, S))
+    assert relmax(gs, cabi.lookup_inner(code, g, tables)) <= 2e-6
+    # either gradient alone; accumulation into an existing table gradient
+    only_s, none_t = cabi.lookup_backward(code, w, g, tables, want=(True, False))
+    assert none_t is None and relmax(only_s, gs) <= 2e-6          # (small shapes: the form with atomics, any order)
+    none_s, only_t = cabi.lookup_backward(code, w, g, tables, want=(False, True))
+    assert none_s is None and np.array_equal(only_t, gt)
+    init = rng.randn(T, S, Do).astype(np.float32)
+    _, acc = cabi.lookup_backward(code, w, g, tables, accumulate=True, init=init)
+    assert np.array_equal(acc, cabi.lookup_scatter_sorted(code, w, g, S, accumulate=True, init=init))
+
+
+def test_lookup_backward_full_size_zipf():
+    """BASELINE.json config 5 through the one-call backward: config-2 shape, codes Zipf(1.1)."""
+    rng = np.random.RandomState(41)
+    B, T, S, Do = 16384, 128, 256, 768
+    p = 1.0 / np.arange(1, S + 1) ** 1.1
+    p /= p.sum()
+    code = rng.choice(S, size=(B, T), p=p).astype(np.int32)
+    w = (1.0 - rng.rand(B, T)).astype(np.float32)
+    g = rng.randn(B, Do).astype(np.float32)
+    tables = (0.02 * rng.randn(T, S, Do)).astype(np.float32)
+    gs, gt = cabi.lookup_backward(code, w, g, tables)
+    # table gradient: column sums, a few tables in full, the sorted entry point bit for bit
+    assert relmax(gt.astype(np.float64).sum(1), w.astype(np.float64).T @ g.astype(np.float64)) <= 1e-5
+    for t in (0, 77, 127):
+        want_t = oracle.scatter_add(code[:, t:t + 1], g.astype(np.float64), w[:, t:t + 1].astype(np.float64), S)
+        assert relmax(gt[t], want_t) <= 1e-5
+    assert np.array_equal(gt, cabi.lookup_scatter_sorted(code, w, g, S))
+    # score gradient: a token sample against the oracle, every (token, table) against the separate entry point
+    # (the same additions in the same order: bit-identical), the duality with the forward, and a second call
+    sub = np.unique(np.concatenate([rng.choice(B, 64, replace=False), np.arange(B - 40, B), np.arange(0, 8)]))
+    idx = code + (np.arange(T, dtype=np.int32) * S)[None]
+    want = oracle.indexed_inner_product(idx[sub], g[sub].astype(np.float64), tables.reshape(T * S, Do).astype(np.float64))
+    assert relmax(gs[sub], want) <= 1e-5
+    assert np.array_equal(gs, cabi.lookup_inner(code, g, tables))
+    fwd = cabi.lookup_gather(code, w, tables, None)
+    lhs = float((fwd.astype(np.float64) * g).sum())
+    rhs = float((gs.astype(np.float64) * w).sum())
+    assert abs(lhs - rhs) <= 1e-5 * max(abs(lhs), 1.0) * 10
+    gs2, gt2 = cabi.lookup_backward(code, w, g, tables)
+    assert np.array_equal(gs, gs2) and np.array_equal(gt, gt2)
+
+
 def test_lookup_scatter_full_size_zipf_properties():
     # BASELINE.json config 5: config-2 shape, codes Zipf(1.1) over 256 entries
     rng = np.random.RandomState(41)
