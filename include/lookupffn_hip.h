@@ -171,7 +171,18 @@ int lffn_ln_bh4_block_hash_f32(const float *x, const float *ln_weight, const flo
  * the caller forms it (a batched product over the tokens) and applies mode 2.
  * Replaces what autograd records for bh4_cuda with block_size == 64 (PL/bh4/kernel.py:23-36)
  * and the mix of BH4._forward (PL/lookup.py:36-37).
+ *
+ * lffn_ln_bh4_block_hash_train_f32: the same with the layer's LayerNorm (PL/lookup.py:99) run on the
+ * token tile as it is loaded, as in lffn_ln_bh4_block_hash_f32; row_stats [B, 2] receives every row's
+ * mean and 1/sigma.  The normalised rows are not stored: lffn_ln_bh4_block_wgrad_f32 forms them again
+ * from x and row_stats (the same operations in the same order), and g_x of lffn_bh4_block_bwd_f32 is
+ * then the gradient w.r.t. the LayerNorm output, which lffn_layer_norm_bwd_f32 takes back to x.
  */
+int lffn_ln_bh4_block_hash_train_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
+                                     const float *w_folded, const float *proj_bias, int32_t *codes, float *scores,
+                                     float *z, float *stage_inputs, float *row_stats, int64_t B, int64_t H,
+                                     int64_t D, int64_t R, int64_t J, int64_t T, int64_t block_size, float decay,
+                                     float residual, void *stream);
 int lffn_bh4_block_hash_train_f32(const float *x, const float *w_folded, const float *proj_bias,
                                   int32_t *codes, float *scores, float *z, float *stage_inputs,
                                   int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
@@ -255,6 +266,24 @@ int lffn_lookup_ffn_fused_f32(const float *x, const float *ln_weight, const floa
                               float residual, void *stream);
 
 /*
+ * The same call with the layer's parameters and sizes in a block the caller fills once per parameter set
+ * (plain data: the library keeps no pointer to it after the call returns).  For callers whose per-call cost
+ * matters at small batches: through a foreign-function interface every argument is converted on every call,
+ * and at 256 tokens the kernel takes 7 microseconds.  Same checks, same kernel, same results.
+ */
+typedef struct lffn_fused_layer {
+    const float *ln_weight, *ln_bias;       /* [H], both NULL for no LayerNorm */
+    const float *diag;                      /* [R, J, D] */
+    const float *proj_bias;                 /* [T*8] or NULL */
+    const float *tables;                    /* [T, S, Do] */
+    const float *out_bias;                  /* [Do] or NULL */
+    int64_t H, D, R, J, T, S, Do;
+    float ln_eps, decay, residual;
+} lffn_fused_layer;
+int lffn_lookup_ffn_fused_layer_f32(const lffn_fused_layer *layer, const float *x, const float *residual_in,
+                                    float *out, int64_t B, void *stream);
+
+/*
  * Weight gradient of the BH4 module with 64 x 64 blocks, all stages in one launch, in the
  * folded basis: for stage s = r * J + j and block n
  *   g_folded[s][n][o][i] += sum_b stage_grads[s][b][64n + o] * u_s[b][64n + i]
@@ -267,6 +296,11 @@ int lffn_lookup_ffn_fused_f32(const float *x, const float *ln_weight, const floa
  */
 int lffn_bh4_block_wgrad_f32(const float *stage_grads, const float *x, const float *stage_inputs, float *g_folded,
                              int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t block_size, void *stream);
+/* The same with u_s = LayerNorm(x) for j = 0, formed on load from x, ln_weight, ln_bias [H] and the row_stats
+ * [B, 2] lffn_ln_bh4_block_hash_train_f32 kept (PL/lookup.py:99 in front of PL/bh4/kernel.py:32). */
+int lffn_ln_bh4_block_wgrad_f32(const float *stage_grads, const float *x, const float *ln_weight, const float *ln_bias,
+                                const float *row_stats, const float *stage_inputs, float *g_folded, int64_t B,
+                                int64_t H, int64_t D, int64_t R, int64_t J, int64_t block_size, void *stream);
 
 /*
  * The tail of the BH4 module and the hash in one pass, for any block size:

@@ -41,6 +41,9 @@ SIGNATURES = {
                                   ctypes.c_float, ctypes.c_float, _vp],
     "lffn_bh4_block_hash_train_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                       ctypes.c_float, ctypes.c_float, _vp],
+    "lffn_ln_bh4_block_hash_train_f32": [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
+                                         _i64, _i64, _f32, _f32, _vp],
+    "lffn_ln_bh4_block_wgrad_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp],
     "lffn_bh4_fold_mode_f32": [_vp, _vp, _i64, _i64, ctypes.c_int32, _vp],
     "lffn_bh4_block_bwd_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                ctypes.c_float, ctypes.c_float, _vp],
@@ -94,6 +97,15 @@ SIGNATURES = {
     "lffn_lookup_backward_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, ctypes.c_int32, _vp],
     "lffn_lookup_inner_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
 }
+
+class FusedLayer(ctypes.Structure):
+    """struct lffn_fused_layer of include/lookupffn_hip.h."""
+    _fields_ = [("ln_weight", _vp), ("ln_bias", _vp), ("diag", _vp), ("proj_bias", _vp), ("tables", _vp), ("out_bias", _vp),
+                ("H", _i64), ("D", _i64), ("R", _i64), ("J", _i64), ("T", _i64), ("S", _i64), ("Do", _i64),
+                ("ln_eps", _f32), ("decay", _f32), ("residual", _f32)]
+
+
+SIGNATURES["lffn_lookup_ffn_fused_layer_f32"] = [ctypes.POINTER(FusedLayer), _vp, _vp, _vp, _i64, _vp]
 
 _lib = None
 _lock = threading.Lock()

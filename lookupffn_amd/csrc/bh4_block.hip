@@ -104,6 +104,7 @@ struct BlockArgs {
     uint32_t *records;     // hash form, instead of codes and scores: the record stream of the
     int64_t rec_stride;    // four-lanes-per-token gather, [T/2][3][rec_stride] (see lookup_gather_quad.hip)
     float *z_out;          // [B, T*8] or null    (hash form: z kept for the backward)
+    float *row_stats;      // [B, 2] or null: LayerNorm's mean and 1/sigma of every row, kept for the backward
     float *stage_save;     // forward: [R, J-1, B, D] inputs of stages 1..J-1, or null;
                            // backward: [R, J, B, D] gradient before the product of each stage
     const float *gz;       // [B, T*8]            (backward form: gradient of z)
@@ -254,6 +255,8 @@ __global__ __launch_bounds__(256 * HV / NH, HV == 1 ? 2 : 1) void bh4_block_kern
                     if (lane == 0) {
                         stats[2 * (wave * RPW + i)] = mean;
                         stats[2 * (wave * RPW + i) + 1] = rstd;
+                        const int64_t tok = tok_base + wave * RPW + i;
+                        if (a.row_stats && r == 0 && tok < B) *reinterpret_cast<float2 *>(a.row_stats + 2 * tok) = make_float2(mean, rstd);
                     }
                 }
             }
@@ -744,6 +747,31 @@ extern "C" int lffn_bh4_block_hash_train_f32(const float *x, const float *w_fold
                  LFFN_ERR_BAD_ARG);
     BlockArgs a{};
     a.x = x; a.wf = w_folded; a.pbias = proj_bias; a.codes = codes; a.scores = scores; a.z_out = z;
+    a.stage_save = stage_inputs; a.B = B; a.H = (int)H; a.R = (int)R; a.J = (int)J; a.T = (int)T;
+    a.decay = decay; a.residual = residual;
+    return dispatch_block<true>(a, D, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int lffn_ln_bh4_block_hash_train_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
+                                                const float *w_folded, const float *proj_bias, int32_t *codes,
+                                                float *scores, float *z, float *stage_inputs, float *row_stats,
+                                                int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
+                                                int64_t block_size, float decay, float residual, void *stream) {
+    LFFN_REQUIRE(B >= 0 && R >= 1 && J >= 1 && D >= 1 && H >= 1 && H <= D && T >= 1, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(H % 4 == 0 && J <= 64, LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(block_size == BS && lffn_is_pow2(D) && D >= BS && D <= 1024, LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(R <= 4096 && B <= (int64_t(1) << 31) - 1 && T <= (1 << 24), LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(T * 8 <= R * D && ln_eps >= 0.f, LFFN_ERR_BAD_ARG);
+    if (B == 0) return LFFN_OK;
+    LFFN_REQUIRE(x && ln_weight && ln_bias && w_folded && codes && scores && z && row_stats && (stage_inputs || J == 1),
+                 LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_aligned16(x) && lffn_aligned16(w_folded) && lffn_aligned16(z) && lffn_aligned16(ln_weight) &&
+                     lffn_aligned16(ln_bias) && (uintptr_t)row_stats % 8 == 0 &&
+                     (!proj_bias || lffn_aligned16(proj_bias)) && (!stage_inputs || lffn_aligned16(stage_inputs)),
+                 LFFN_ERR_BAD_ARG);
+    BlockArgs a{};
+    a.x = x; a.ln_w = ln_weight; a.ln_b = ln_bias; a.ln_eps = ln_eps; a.wf = w_folded; a.pbias = proj_bias;
+    a.codes = codes; a.scores = scores; a.z_out = z; a.row_stats = row_stats;
     a.stage_save = stage_inputs; a.B = B; a.H = (int)H; a.R = (int)R; a.J = (int)J; a.T = (int)T;
     a.decay = decay; a.residual = residual;
     return dispatch_block<true>(a, D, static_cast<hipStream_t>(stream));

@@ -1007,6 +1007,14 @@ extern "C" int lffn_lookup_ffn_fused_f32(const float *x, const float *ln_weight,
     return lffn_launch_status();
 }
 
+extern "C" int lffn_lookup_ffn_fused_layer_f32(const lffn_fused_layer *layer, const float *x, const float *residual_in,
+                                               float *out, int64_t B, void *stream) {
+    LFFN_REQUIRE(layer, LFFN_ERR_BAD_ARG);
+    return lffn_lookup_ffn_fused_f32(x, layer->ln_weight, layer->ln_bias, layer->ln_eps, layer->diag, layer->proj_bias,
+                                     layer->tables, layer->out_bias, residual_in, out, B, layer->H, layer->D, layer->R,
+                                     layer->J, layer->T, layer->S, layer->Do, layer->decay, layer->residual, stream);
+}
+
 extern "C" int lffn_fht_f16(const uint16_t *in, uint16_t *out, int64_t B, int64_t D, void *stream) {
     return fht16_entry<false>(in, out, B, D, stream);
 }

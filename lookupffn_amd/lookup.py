@@ -309,6 +309,49 @@ class LnProjectHash(torch.autograd.Function):
                 g_bias if (ctx.has_bias and need[5]) else None, None, None)
 
 
+class LnBlockProjectHash(torch.autograd.Function):
+    """LayerNorm -> BH4 with 64 x 64 blocks -> mix -> bias -> 8-bit code + score as one differentiable operator
+    (PL/lookup.py:99 in front of PL/bh4/kernel.py:23-36 and PL/lookup.py:29-39).  Forward: BlockProjectHash's
+    kernel with LayerNorm run on the token tile as it is loaded; it keeps every row's mean and 1/sigma
+    instead of the normalised rows.  Backward: BlockProjectHash's, with the weight-gradient kernel forming
+    LayerNorm(x) on load for the first stage of every repeat, then the LayerNorm backward kernel."""
+
+    @staticmethod
+    def forward(ctx, x, ln_weight, ln_bias, eps, weight, bias, T, decay):
+        x = x.contiguous()
+        w = weight.contiguous()
+        folded = ops.bh4_fold_mode(w, 0)
+        code, score, z, stage_in, stats = ops.ln_bh4_block_hash_train(x, ln_weight, ln_bias, float(eps), folded, bias, T,
+                                                                      float(decay), float(1 - decay))
+        ctx.save_for_backward(x, ln_weight, ln_bias, w, z, stage_in, stats)
+        ctx.eps = float(eps)
+        ctx.has_bias = bias is not None
+        ctx.decay = float(decay)
+        ctx.mark_non_differentiable(code)
+        return code, score
+
+    @staticmethod
+    def backward(ctx, _g_code, g_score):
+        x, ln_weight, ln_bias, w, z, stage_in, stats = ctx.saved_tensors
+        R, J, NB, bs, _ = w.shape
+        B, H = x.shape
+        T = g_score.shape[1]
+        need = ctx.needs_input_grad
+        g_z = ops.code_score_bwd(z.reshape(B, T, 8), g_score.contiguous()).reshape(B, T * 8)
+        g_h, stage_g = ops.bh4_block_bwd(g_z, ops.bh4_fold_mode(w, 1), H, ctx.decay, 1 - ctx.decay)
+        g_w = None
+        if need[4]:
+            g_folded = ops.ln_bh4_block_wgrad(stage_g.reshape(R * J, B, NB * bs), x, ln_weight, ln_bias, stats, stage_in,
+                                              R, J).view_as(w)
+            g_w = ops.bh4_fold_mode(g_folded, 2)
+        g_x = g_lw = g_lb = None
+        if need[0] or need[1] or need[2]:
+            g_x, g_lw, g_lb = ops.layer_norm_bwd(x, ln_weight, ctx.eps, g_h)      # adds the R repeats' gradients
+        g_bias = ops.column_sums(g_z) if (ctx.has_bias and need[5]) else None
+        return (g_x if need[0] else None, g_lw if need[1] else None, g_lb if need[2] else None, None, g_w, g_bias,
+                None, None)
+
+
 class LookupFFN(nn.Module):
     """PL/lookup.py:79-130."""
 
@@ -392,6 +435,9 @@ class LookupFFN(nn.Module):
                       if form == "diag" else None),
                 pbias=None if p.bias is None else p.bias.detach(), tables=self.tables.detach(),
                 obias=self.bias.detach(), decay=float(p.decay_coeff), res_coef=float(1 - p.decay_coeff))
+            if state["one_launch"]:
+                state["block"] = ops.fused_layer_block(state["ln_w"], state["ln_b"], state["eps"], state["diag"], state["pbias"],
+                                                       state["tables"], state["obias"], state["decay"], state["res_coef"])
         self._inference_cache = (key, state)
         return state
 
@@ -407,8 +453,7 @@ class LookupFFN(nn.Module):
             residual = residual.contiguous()
         if st["one_launch"] and x.shape[0] <= self.FUSED_LAYER_MAX_TOKENS:
             # small batches: the whole layer in one launch
-            return ops.lookup_ffn_fused_direct(x, st["ln_w"], st["ln_b"], st["eps"], st["diag"], st["pbias"],
-                                               st["tables"], st["obias"], residual, st["decay"], st["res_coef"])
+            return ops.lookup_ffn_fused_block(st["block"], x, residual)
         if self.num_table % 2 == 0:
             # many tokens: the projection kernel writes the gather kernel's record stream directly
             plan = ops.lookup_gather_records_plan(x.shape[0], self.num_table, self.table_size, self.output_size,
@@ -455,6 +500,11 @@ class LookupFFN(nn.Module):
                 p = self.hash.projection
                 code, score = LnProjectHash.apply(hidden_states, ln.weight, ln.bias, ln.eps, p.weight, p.bias,
                                                   self.num_table, p.decay_coeff)
+            elif ln_kernel_ok and self.hash.can_fuse_block_training(hidden_states):
+                # training, 64 x 64 blocks: LayerNorm inside the matrix-core kernel; the weight gradient forms it again on load
+                p = self.hash.projection
+                code, score = LnBlockProjectHash.apply(hidden_states, ln.weight, ln.bias, ln.eps, p.weight, p.bias,
+                                                       self.num_table, p.decay_coeff)
             elif ln_kernel_ok:
                 hidden_states = LayerNormFn.apply(hidden_states.contiguous(), ln.weight, ln.bias, ln.eps)
                 code, score = self.hash(hidden_states)
@@ -471,6 +521,10 @@ class LookupFFN(nn.Module):
     def forward(self, hidden_states, residual=None):
         """PL/lookup.py:110-118.  ``residual`` (not in the reference; shape [..., output_size]) is
         added to the result inside the gather kernel: the encoder layer's "FFN(x) + x"."""
+        if hidden_states.dim() == 2 and residual is None:
+            # already [tokens, hidden]: nothing to reshape (at a few hundred tokens the layer is one launch of
+            # a few microseconds and every view made here shows in its time)
+            return self._forward(hidden_states, None)
         shape = hidden_states.shape[:-1]
         dim = hidden_states.shape[-1]
         tokens = math.prod(shape)

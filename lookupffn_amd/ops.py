@@ -296,6 +296,78 @@ def _(x, w_folded, bias, T, decay, residual):
             x.new_empty(R, max(J - 1, 0), B, NB * bs))
 
 
+_L.define("ln_bh4_block_hash_train(Tensor x, Tensor ln_w, Tensor ln_b, float eps, Tensor w_folded, Tensor? bias, int T, "
+          "float decay, float residual) -> (Tensor, Tensor, Tensor, Tensor, Tensor)")
+
+
+def _ln_bh4_block_hash_train_impl(x, ln_w, ln_b, eps, w_folded, bias, T, decay, residual):
+    """LayerNorm inside the kernel -> (codes [B,T], scores [B,T], z [B,T*8], stage_inputs [R,J-1,B,D],
+    row_stats [B,2] = every row's mean and 1/sigma)."""
+    _lib.require_gpu(x, ln_w, ln_b, w_folded, bias)
+    assert x.dim() == 2 and w_folded.dim() == 5
+    for t in (x, ln_w, ln_b, w_folded):
+        assert t.dtype == torch.float32 and t.is_contiguous()
+    B, H = x.shape
+    R, J, NB, bs, _ = w_folded.shape
+    D = NB * bs
+    assert H <= D and T * 8 <= R * D and ln_w.numel() == H and ln_b.numel() == H
+    if bias is not None:
+        assert bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == T * 8
+    codes = torch.empty(B, T, dtype=torch.int32, device=x.device)
+    scores = torch.empty(B, T, dtype=torch.float32, device=x.device)
+    z = torch.empty(B, T * 8, dtype=torch.float32, device=x.device)
+    stage_in = torch.empty(R, max(J - 1, 0), B, D, dtype=torch.float32, device=x.device)
+    stats = torch.empty(B, 2, dtype=torch.float32, device=x.device)
+    with _dev_guard(x):
+        rc = _lib.load().lffn_ln_bh4_block_hash_train_f32(
+            _lib.ptr(x), _lib.ptr(ln_w), _lib.ptr(ln_b), eps, _lib.ptr(w_folded), _lib.ptr(bias), _lib.ptr(codes),
+            _lib.ptr(scores), _lib.ptr(z), _lib.ptr(stage_in) if J > 1 else None, _lib.ptr(stats), B, H, D, R, J, T, bs,
+            decay, residual, _lib.stream_of(x))
+    _lib.check(rc, f"lffn_ln_bh4_block_hash_train_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T})")
+    return codes, scores, z, stage_in, stats
+
+
+_L.impl("ln_bh4_block_hash_train", _ln_bh4_block_hash_train_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::ln_bh4_block_hash_train")
+def _(x, ln_w, ln_b, eps, w_folded, bias, T, decay, residual):
+    B = x.shape[0]
+    R, J, NB, bs, _ = w_folded.shape
+    return (torch.empty(B, T, dtype=torch.int32, device=x.device), x.new_empty(B, T), x.new_empty(B, T * 8),
+            x.new_empty(R, max(J - 1, 0), B, NB * bs), x.new_empty(B, 2))
+
+
+_L.define("ln_bh4_block_wgrad(Tensor stage_grads, Tensor x, Tensor ln_w, Tensor ln_b, Tensor row_stats, Tensor stage_inputs, "
+          "int R, int J) -> Tensor")
+
+
+def _ln_bh4_block_wgrad_impl(stage_grads, x, ln_w, ln_b, row_stats, stage_inputs, R, J):
+    """bh4_block_wgrad with LayerNorm(x) as the input of every repeat's first stage, formed on load."""
+    _lib.require_gpu(stage_grads, x, ln_w, ln_b, row_stats, stage_inputs)
+    for t in (stage_grads, x, ln_w, ln_b, row_stats, stage_inputs):
+        assert t.dtype == torch.float32 and t.is_contiguous()
+    S, B, D = stage_grads.shape
+    assert S == R * J and x.shape[0] == B and stage_inputs.numel() == R * (J - 1) * B * D
+    assert tuple(row_stats.shape) == (B, 2) and ln_w.numel() == x.shape[1] and ln_b.numel() == x.shape[1]
+    g = torch.zeros(S, D // 64, 64, 64, dtype=torch.float32, device=x.device)
+    with _dev_guard(x):
+        rc = _lib.load().lffn_ln_bh4_block_wgrad_f32(_lib.ptr(stage_grads), _lib.ptr(x), _lib.ptr(ln_w), _lib.ptr(ln_b),
+                                                     _lib.ptr(row_stats), _lib.ptr(stage_inputs), _lib.ptr(g), B, x.shape[1],
+                                                     D, R, J, 64, _lib.stream_of(x))
+    _lib.check(rc, f"lffn_ln_bh4_block_wgrad_f32(B={B}, H={x.shape[1]}, D={D}, R={R}, J={J})")
+    return g
+
+
+_L.impl("ln_bh4_block_wgrad", _ln_bh4_block_wgrad_impl, "CUDA")
+
+
+@torch.library.register_fake("lookupffn::ln_bh4_block_wgrad")
+def _(stage_grads, x, ln_w, ln_b, row_stats, stage_inputs, R, J):
+    S, B, D = stage_grads.shape
+    return x.new_empty(S, D // 64, 64, 64)
+
+
 _L.define("bh4_block_bwd(Tensor g_z, Tensor w_folded_t, int H, float decay, float residual) -> (Tensor, Tensor)")
 
 
@@ -421,6 +493,33 @@ def lookup_ffn_fused_direct(x, ln_w, ln_b, eps, diag, pbias, tables, obias, resi
             out.data_ptr(), B, H, D, R, J, T, S, Do, decay, residual_coef, _lib.stream_of(x))
     if rc != 0:
         _lib.check(rc, f"lffn_lookup_ffn_fused_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T}, S={S}, Do={Do})")
+    return out
+
+
+def fused_layer_block(ln_w, ln_b, eps, diag, pbias, tables, obias, decay, residual_coef):
+    """The parameter block of lffn_lookup_ffn_fused_layer_f32 for a set of (checked, contiguous, fp32, same-device)
+    parameters, with the entry point and a byref to the block: what lookup_ffn_fused_block takes.  The tensors
+    must outlive the block (LookupFFN keeps both in one cache entry)."""
+    R, J, D = diag.shape
+    T, S, Do = tables.shape
+    blk = _lib.FusedLayer(ln_w.data_ptr(), ln_b.data_ptr(), diag.data_ptr(), None if pbias is None else pbias.data_ptr(),
+                          tables.data_ptr(), None if obias is None else obias.data_ptr(), ln_w.numel(), D, R, J, T, S, Do,
+                          eps, decay, residual_coef)
+    return (_lib.load().lffn_lookup_ffn_fused_layer_f32, ctypes.byref(blk), blk, ln_w.numel(), Do, tables.device)
+
+
+def lookup_ffn_fused_block(block, x, residual):
+    """lookup_ffn_fused_direct through the parameter block: six arguments cross the foreign-function interface
+    instead of twenty-one."""
+    fn, ref, _keep, H, Do, device = block
+    if x.dtype != torch.float32 or x.dim() != 2 or x.shape[1] != H or x.device != device or not x.is_contiguous():
+        raise ValueError("x: contiguous fp32 [B, H] on the parameters' device")
+    B = x.shape[0]
+    out = torch.empty((B, Do), dtype=torch.float32, device=device)
+    with _dev_guard(x):
+        rc = fn(ref, x.data_ptr(), None if residual is None else residual.data_ptr(), out.data_ptr(), B, _lib.stream_of(x))
+    if rc != 0:
+        _lib.check(rc, f"lffn_lookup_ffn_fused_layer_f32(B={B}, H={H}, Do={Do})")
     return out
 
 
@@ -1045,6 +1144,8 @@ bh4_fold_mode = torch.ops.lookupffn.bh4_fold_mode
 bh4_block_hash_train = torch.ops.lookupffn.bh4_block_hash_train
 bh4_block_bwd = torch.ops.lookupffn.bh4_block_bwd
 bh4_block_wgrad = torch.ops.lookupffn.bh4_block_wgrad
+ln_bh4_block_hash_train = torch.ops.lookupffn.ln_bh4_block_hash_train
+ln_bh4_block_wgrad = torch.ops.lookupffn.ln_bh4_block_wgrad
 lookup_ffn_fused = torch.ops.lookupffn.lookup_ffn_fused
 layer_norm_bwd = torch.ops.lookupffn.layer_norm_bwd
 ln_bh4_block_hash = torch.ops.lookupffn.ln_bh4_block_hash

@@ -115,6 +115,32 @@ def bh4_block_train(x, w, bias, T, decay=0.7):
     return host(codes), host(scores), host(z), host(st)[:, :J - 1]
 
 
+def ln_bh4_block_train(x, ln_w, ln_b, eps, w, bias, T, decay=0.7):
+    """-> codes, scores, z, stage_inputs [R, J-1, B, D], row_stats [B, 2]"""
+    xd, lw, lb, wd, bd = dev(x), dev(ln_w), dev(ln_b), dev(w), dev(bias)
+    B, H = x.shape
+    R, J, NB, bs, _ = w.shape
+    D = NB * bs
+    wf = torch.empty_like(wd)
+    _call("lffn_bh4_fold_mode_f32", p(wd), p(wf), R * J * NB, bs, 0)
+    codes = torch.full((B, T), -1, dtype=torch.int32, device=DEV)
+    scores = torch.full((B, T), float("nan"), dtype=torch.float32, device=DEV)
+    z = torch.full((B, T * 8), float("nan"), dtype=torch.float32, device=DEV)
+    st = torch.full((R, max(J - 1, 1), B, D), float("nan"), dtype=torch.float32, device=DEV)
+    stats = torch.full((B, 2), float("nan"), dtype=torch.float32, device=DEV)
+    _call("lffn_ln_bh4_block_hash_train_f32", p(xd), p(lw), p(lb), float(np.float32(eps)), p(wf), p(bd), p(codes), p(scores),
+          p(z), p(st), p(stats), B, H, D, R, J, T, bs, float(np.float32(decay)), float(np.float32(1 - decay)))
+    return host(codes), host(scores), host(z), host(st)[:, :J - 1], host(stats)
+
+
+def ln_bh4_block_wgrad(stage_grads, x, ln_w, ln_b, stats, stage_inputs, R, J):
+    sg, xd, lw, lb, sd, si = dev(stage_grads), dev(x), dev(ln_w), dev(ln_b), dev(stats), dev(stage_inputs)
+    S, B, D = stage_grads.shape
+    g = torch.zeros(S, D // 64, 64, 64, dtype=torch.float32, device=DEV)
+    _call("lffn_ln_bh4_block_wgrad_f32", p(sg), p(xd), p(lw), p(lb), p(sd), p(si), p(g), B, x.shape[1], D, R, J, 64)
+    return host(g)
+
+
 def bh4_block_bwd(g_z, w, H, decay=0.7):
     """-> g_x [R, B, H], stage_grads [R, J, B, D]"""
     gd, wd = dev(g_z), dev(w)
@@ -151,6 +177,21 @@ def lookup_ffn_fused(x, ln_w, ln_b, eps, diag, pbias, tables, obias, residual, d
     out = torch.full((B, Do), float("nan"), dtype=torch.float32, device=DEV)
     _call("lffn_lookup_ffn_fused_f32", p(xd), p(lw), p(lb), float(np.float32(eps)), p(dd), p(pb), p(td), p(ob), p(rs),
           p(out), B, H, D, R, J, T, S, Do, float(np.float32(decay)), float(np.float32(1 - decay)))
+    return host(out)
+
+
+def lookup_ffn_fused_layer(x, ln_w, ln_b, eps, diag, pbias, tables, obias, residual, decay=0.7):
+    """lffn_lookup_ffn_fused_layer_f32: the same call with the parameters in a struct lffn_fused_layer."""
+    xd, dd, td = dev(x), dev(diag), dev(tables)
+    lw, lb = (None, None) if ln_w is None else (dev(ln_w), dev(ln_b))
+    pb, ob, rs = dev(pbias), dev(obias), dev(residual)
+    B, H = x.shape
+    R, J, D = diag.shape
+    T, S, Do = tables.shape
+    blk = _lib.FusedLayer(p(lw), p(lb), p(dd), p(pb), p(td), p(ob), H, D, R, J, T, S, Do, float(np.float32(eps)),
+                          float(np.float32(decay)), float(np.float32(1 - decay)))
+    out = torch.full((B, Do), float("nan"), dtype=torch.float32, device=DEV)
+    _call("lffn_lookup_ffn_fused_layer_f32", ctypes.byref(blk), p(xd), p(rs), p(out), B)
     return host(out)
 
 

@@ -327,6 +327,40 @@ def test_bh4_block_training_kernels_match_float64(B, H, D, R, T):
         assert relmax(g_x[r], want_x) <= 1e-5, r
 
 
+@pytest.mark.parametrize("B,H,D,R,T", [(70, 768, 1024, 1, 128), (33, 256, 256, 2, 64), (600, 500, 512, 1, 64)])
+def test_ln_bh4_block_training_kernels(B, H, D, R, T):
+    """LayerNorm inside the training forward (lffn_ln_bh4_block_hash_train_f32) and formed again on load in the
+    weight gradient (lffn_ln_bh4_block_wgrad_f32): against the same kernels without LayerNorm fed the normalised rows."""
+    rng = np.random.RandomState(B + H + T)
+    J, bs = 4, 64
+    x = (rng.randn(B, H) * 1.5 + 0.3).astype(np.float32)
+    ln_w = (1 + 0.1 * rng.randn(H)).astype(np.float32)
+    ln_b = (0.1 * rng.randn(H)).astype(np.float32)
+    w = (rng.randn(R, J, D // bs, bs, bs) / math.sqrt(bs * D)).astype(np.float32)
+    bias = (0.05 * rng.randn(T * 8)).astype(np.float32)
+    codes, scores, z, st, stats = cabi.ln_bh4_block_train(x, ln_w, ln_b, 1e-5, w, bias, T)
+    # the rows' statistics against float64
+    x64 = x.astype(np.float64)
+    mean, var = x64.mean(1), x64.var(1)
+    np.testing.assert_allclose(stats[:, 0], mean, rtol=0, atol=1e-6 * np.abs(x).max())
+    np.testing.assert_allclose(stats[:, 1], 1 / np.sqrt(var + 1e-5), rtol=2e-6)
+    # LayerNorm from the kernel's own statistics, its operations in fp32: the rows the kernel multiplied
+    h = ((x - stats[:, :1]) * stats[:, 1:2] * ln_w + ln_b).astype(np.float32)
+    assert relmax(h, oracle.layernorm(x64, ln_w, ln_b, 1e-5)) <= 1e-5
+    # the same kernel without LayerNorm on those rows: the same codes, scores, z and stage inputs
+    codes2, scores2, z2, st2 = cabi.bh4_block_train(h, w, bias, T)
+    assert np.array_equal(z, z2) and np.array_equal(codes, codes2) and np.array_equal(scores, scores2)
+    assert np.array_equal(st, st2)
+    # the hash form used for inference runs the same LayerNorm: the same codes
+    codes3, scores3 = cabi.ln_bh4_block_hash(x, ln_w, ln_b, 1e-5, w, bias, T)
+    assert np.array_equal(codes, codes3) and np.array_equal(scores, scores3)
+    # weight gradient: LayerNorm on load against the plain kernel on the normalised rows
+    sg = rng.randn(R * J, B, D).astype(np.float32)
+    g_ln = cabi.ln_bh4_block_wgrad(sg, x, ln_w, ln_b, stats, st.reshape(R, J - 1, B, D), R, J)
+    g_plain = cabi.bh4_block_wgrad(sg, h, st.reshape(R, J - 1, B, D), R, J)
+    assert relmax(g_ln, g_plain) <= 1e-5
+
+
 @pytest.mark.parametrize("B,H,D,R,J", [(1000, 1024, 1024, 1, 2), (515, 768, 1024, 2, 2), (70, 100, 256, 1, 3),
                                        (2050, 512, 512, 1, 1), (3, 64, 64, 2, 1), (0, 64, 64, 1, 2)])
 def test_bh4_block_wgrad_matches_float64(B, H, D, R, J):
@@ -377,6 +411,8 @@ def test_lookup_ffn_fused_matches_the_two_kernel_form(B, H, D, R, J, T, Do, with
     got = cabi.lookup_ffn_fused(x, ln_w, ln_b, 1e-5, diag, pbias, tables, obias, res)
     assert not np.isnan(got).any()
     assert relmax(got, want + obias + res) <= 1e-5       # same codes and scores (same kernel body), fp32 row sums
+    # the same call with the parameters handed over in a struct lffn_fused_layer
+    assert np.array_equal(got, cabi.lookup_ffn_fused_layer(x, ln_w, ln_b, 1e-5, diag, pbias, tables, obias, res))
     got = cabi.lookup_ffn_fused(x, ln_w, ln_b, 1e-5, diag, None, tables, None, None)
     if with_ln:
         code, score, _ = cabi.ln_project_hash(x, ln_w, ln_b, 1e-5, diag, np.zeros(T * 8, np.float32), T)
