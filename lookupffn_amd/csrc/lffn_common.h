@@ -82,21 +82,23 @@ static inline bool lffn_grant_dynamic_lds(const void *kernel, size_t lds_bytes, 
 }
 
 // lookup_gather_quad.hip: the two-tables-per-buffer LDS gather with four lanes per token (not exported);
-// fmt is one of LFFN_ROWS_*
+// fmt is one of LFFN_ROWS_*, tokens the tokens per workgroup (a multiple of 16)
 __attribute__((visibility("hidden")))
 int lffn_internal_lookup_gather_quad(const int32_t *code, const float *score, const void *tables,
                                      const float *bias, const float *residual, float *out, int64_t B, int64_t T,
-                                     int64_t S, int64_t Do, int fmt, int np, void *workspace, void *stream);
+                                     int64_t S, int64_t Do, int fmt, int tokens, void *workspace, void *stream);
 __attribute__((visibility("hidden")))
 bool lffn_internal_quad_np_built(int fmt, int np);
 __attribute__((visibility("hidden")))
+int lffn_internal_quad_passes(int fmt, int64_t tokens);
+__attribute__((visibility("hidden")))
 int64_t lffn_internal_quad_stream_bytes(int64_t B, int64_t T);
 __attribute__((visibility("hidden")))
-int64_t lffn_internal_quad_record_stride(int64_t B, int np);
+int64_t lffn_internal_quad_record_stride(int64_t B, int fmt, int64_t tokens);
 __attribute__((visibility("hidden")))
 int lffn_internal_lookup_gather_quad_records(const uint32_t *records, int64_t record_stride, const void *tables,
                                              const float *bias, const float *residual, float *out, int64_t B,
-                                             int64_t T, int64_t S, int64_t Do, int fmt, int np, void *stream);
+                                             int64_t T, int64_t S, int64_t Do, int fmt, int tokens, void *stream);
 
 // lookup_inner.hip: the four-lanes-per-token score gradient where the shape qualifies (not exported)
 __attribute__((visibility("hidden")))

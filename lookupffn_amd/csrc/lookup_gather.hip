@@ -347,6 +347,7 @@ int launch_lds(const LdsGatherArgs &a, hipStream_t stream) {
 struct GatherPlan {
     int kind, np;
     double us;             // predicted time
+    int tile = 0;          // kind 3: tokens per workgroup (a multiple of 16 in (256 * (np - 1), 256 * np])
 };
 
 // The four-lanes-per-token kernel: microseconds per table pair of a workgroup = a fixed part (the 64 KB
@@ -406,11 +407,18 @@ GatherPlan plan_quad(int fmt, int64_t B, int64_t T, int64_t S, int64_t Do, bool 
     const double per_pass = fmt == LFFN_ROWS_F32 ? QUAD_US_PER_PAIR_PASS : QUAD_US_PER_PAIR_PASS_16[fmt];
     for (int np : {4, 6, 7, 8}) {
         if (!lffn_internal_quad_np_built(fmt, np)) continue;
+        // as many tiles as tiles of np full passes would take, the tokens spread evenly over them (in groups of
+        // 16): the last pass is then short for some of a workgroup's wavefronts, which leave it out.  What a short
+        // pass costs was measured as about half a pass plus its share of the reads.
         const int64_t tiles = (B + 256 * np - 1) / (256 * np);
+        int64_t tile = (((B + tiles - 1) / tiles) + 15) & ~int64_t(15);
+        if (tile <= 256 * (np - 1)) tile = 256 * (np - 1) + 16;
+        const int64_t rem = tile - 256 * (np - 1);                                 // tokens in the last pass: 16 .. 256
+        const double passes = double(np - 1) + (rem == 256 ? 1.0 : 0.5 + 0.5 * double(rem) / 256.0);
         const int64_t rounds = (tiles * nslices + 255) / 256;
-        const double us = double(rounds) * double(T / 2) * (QUAD_US_PER_PAIR + np * per_pass) +
+        const double us = double(rounds) * double(T / 2) * (QUAD_US_PER_PAIR + passes * per_pass) +
                           (pack ? double(B) * double(T) * 14.0 / 3e6 + 4.0 : 0.0);     // packing: 8 bytes read, 6 written per (token, table)
-        if (us < best.us) best = GatherPlan{3, np, us};
+        if (us < best.us) best = GatherPlan{3, np, us, (int)tile};
     }
     return best;
 }
@@ -529,12 +537,14 @@ GatherPlan choose_quad(int64_t B, int64_t T, int64_t S, int64_t Do, bool pack = 
     return qp.us < QUAD_MARGIN * other ? qp : none;
 }
 
-// four lanes per token: a tile size built for the row format, 256-row tables, an even number of them, whole
-// 128-byte slices, 32-bit offsets inside a table pair
-bool quad_plan_is_valid(int fmt, int np, int64_t B, int64_t T, int64_t S, int64_t Do) {
+// four lanes per token: a tile (tokens per workgroup: whole groups of 16, its last pass not empty) whose number
+// of passes is built for the row format, 256-row tables, an even number of them, whole 128-byte slices, 32-bit
+// offsets inside a table pair
+bool quad_plan_is_valid(int fmt, int64_t tile, int64_t B, int64_t T, int64_t S, int64_t Do) {
     const int esz = fmt == LFFN_ROWS_F32 ? 4 : 2;
     const int cols = 128 / esz;
-    return lffn_internal_quad_np_built(fmt, np) && S == MAX_S && T >= 2 && T % 2 == 0 && T <= (1 << 20) &&
+    const int np = lffn_internal_quad_passes(fmt, tile);
+    return np != 0 && tile > 256 * (np - 1) && S == MAX_S && T >= 2 && T % 2 == 0 && T <= (1 << 20) &&
            Do % cols == 0 && B * T < (int64_t(1) << 31) && 2 * S * Do * esz < (int64_t(1) << 32) &&
            B * (Do / cols) <= (int64_t(1) << 30);
 }
@@ -543,7 +553,7 @@ template <bool BF16>
 bool plan_is_valid(const GatherPlan &p, int64_t B, int64_t T, int64_t S, int64_t Do) {
     if (p.kind == 0) return true;
     if (p.kind == 3)        // four lanes per token
-        return quad_plan_is_valid(BF16 ? LFFN_ROWS_BF16 : LFFN_ROWS_F32, p.np, B, T, S, Do);
+        return quad_plan_is_valid(BF16 ? LFFN_ROWS_BF16 : LFFN_ROWS_F32, p.tile, B, T, S, Do);
     if (p.kind != 1 && p.kind != 2) return false;
     const bool np_ok = BF16 ? (p.np == 4 || p.np == 8) : (p.np == 4 || p.np == 8 || p.np == 13 || p.np == 16);
     const int cols = (p.kind == 1 ? 256 : 128) / (BF16 ? 2 : 4);
@@ -572,7 +582,7 @@ int lookup_gather_entry(const int32_t *code, const float *score, const void *tab
             (uintptr_t)score % 8 == 0) {
             LFFN_REQUIRE(lffn_aligned16(workspace), LFFN_ERR_BAD_ARG);
             return lffn_internal_lookup_gather_quad(code, score, tables, bias, residual, out, B, T, S, Do,
-                                                    BF16 ? LFFN_ROWS_BF16 : LFFN_ROWS_F32, qp.np, workspace, stream);
+                                                    BF16 ? LFFN_ROWS_BF16 : LFFN_ROWS_F32, qp.tile, workspace, stream);
         }
     }
     // Many tokens, tables that fit the 256 MB Infinity Cache: take the tokens in pieces, one launch
@@ -621,9 +631,15 @@ int lookup_gather_entry(const int32_t *code, const float *score, const void *tab
         }
     } else {
         plan.kind = kind_req;
-        const int per_np = kind_req == 1 ? 64 : (kind_req == 3 ? 256 : 128);
-        plan.np = kind_req == 0 ? 0 : tokens_req / per_np;
-        LFFN_REQUIRE(kind_req == 0 || (tokens_req > 0 && tokens_req % per_np == 0), LFFN_ERR_BAD_ARG);
+        if (kind_req == 3) {          // any whole number of 16-token groups; the passes follow from it
+            LFFN_REQUIRE(tokens_req > 0 && tokens_req % 16 == 0, LFFN_ERR_BAD_ARG);
+            plan.tile = tokens_req;
+            plan.np = lffn_internal_quad_passes(BF16 ? LFFN_ROWS_BF16 : LFFN_ROWS_F32, tokens_req);
+        } else {
+            const int per_np = kind_req == 1 ? 64 : 128;
+            plan.np = kind_req == 0 ? 0 : tokens_req / per_np;
+            LFFN_REQUIRE(kind_req == 0 || (tokens_req > 0 && tokens_req % per_np == 0), LFFN_ERR_BAD_ARG);
+        }
         LFFN_REQUIRE(plan_is_valid<BF16>(plan, B, T, S, Do), LFFN_ERR_UNSUPPORTED);
         if (plan.kind == 3) {       // needs the record stream's workspace
             LFFN_REQUIRE(workspace && workspace_bytes >= lffn_internal_quad_stream_bytes(B, T), LFFN_ERR_UNSUPPORTED);
@@ -635,7 +651,7 @@ int lookup_gather_entry(const int32_t *code, const float *score, const void *tab
         return lffn_internal_lookup_gather_token_major(code, score, tables, bias, residual, out, B, T, S, Do, BF16, stream);
     if (plan.kind == 3)
         return lffn_internal_lookup_gather_quad(code, score, tables, bias, residual, out, B, T, S, Do,
-                                                BF16 ? LFFN_ROWS_BF16 : LFFN_ROWS_F32, plan.np, quad_ws, stream);
+                                                BF16 ? LFFN_ROWS_BF16 : LFFN_ROWS_F32, plan.tile, quad_ws, stream);
     if (plan.kind == 2)
         return lffn_internal_lookup_gather_pair(code, score, tables, bias, residual, out, B, T, S, Do, BF16, plan.np, stream);
     const int np = plan.np;
@@ -672,25 +688,25 @@ int lookup_gather_entry_f16(const int32_t *code, const float *score, const void 
     LFFN_REQUIRE(lffn_aligned16(tables) && lffn_aligned16(out) && (!bias || lffn_aligned16(bias)) &&
                      (!residual || lffn_aligned16(residual)), LFFN_ERR_BAD_ARG);
     if (B == 0) return LFFN_OK;
-    int np = 0;
+    int tile = 0;
     if (kind_req < 0) {
         const GatherPlan qp = plan_quad(LFFN_ROWS_F16, B, T, S, Do);
         const double token_major_us = double(B) * double(T) * double(Do) * 2 / 9e6 + 5.0;
         if (qp.kind == 3 && qp.us < QUAD_MARGIN * token_major_us && workspace &&
             workspace_bytes >= lffn_internal_quad_stream_bytes(B, T) && lffn_aligned16(workspace) &&
             (uintptr_t)code % 8 == 0 && (uintptr_t)score % 8 == 0)
-            np = qp.np;
+            tile = qp.tile;
     } else if (kind_req == 3) {
-        LFFN_REQUIRE(tokens_req > 0 && tokens_req % 256 == 0, LFFN_ERR_BAD_ARG);
-        np = tokens_req / 256;
-        LFFN_REQUIRE(quad_plan_is_valid(LFFN_ROWS_F16, np, B, T, S, Do), LFFN_ERR_UNSUPPORTED);
+        LFFN_REQUIRE(tokens_req > 0 && tokens_req % 16 == 0, LFFN_ERR_BAD_ARG);
+        tile = tokens_req;
+        LFFN_REQUIRE(quad_plan_is_valid(LFFN_ROWS_F16, tile, B, T, S, Do), LFFN_ERR_UNSUPPORTED);
         LFFN_REQUIRE(workspace && workspace_bytes >= lffn_internal_quad_stream_bytes(B, T), LFFN_ERR_UNSUPPORTED);
         LFFN_REQUIRE(lffn_aligned16(workspace) && (uintptr_t)code % 8 == 0 && (uintptr_t)score % 8 == 0, LFFN_ERR_BAD_ARG);
     } else {
         LFFN_REQUIRE(kind_req == 0, LFFN_ERR_UNSUPPORTED);       // the 16- and 8-lane LDS kernels are not built for half rows
     }
-    if (np)
-        return lffn_internal_lookup_gather_quad(code, score, tables, bias, residual, out, B, T, S, Do, LFFN_ROWS_F16, np,
+    if (tile)
+        return lffn_internal_lookup_gather_quad(code, score, tables, bias, residual, out, B, T, S, Do, LFFN_ROWS_F16, tile,
                                                 workspace, stream);
     return lffn_internal_lookup_gather_token_major(code, score, tables, bias, residual, out, B, T, S, Do, LFFN_ROWS_F16, stream);
 }
@@ -759,13 +775,13 @@ extern "C" int lffn_lookup_gather_ws_plan(int64_t B, int64_t T, int64_t S, int64
         if (row_format == LFFN_ROWS_F16) {
             const GatherPlan qp = plan_quad(LFFN_ROWS_F16, B, T, S, Do);
             if (qp.kind == 3 && room && qp.us < QUAD_MARGIN * (double(B) * double(T) * double(Do) * 2 / 9e6 + 5.0)) {
-                kind = 3; tokens = 256 * qp.np;
+                kind = 3; tokens = qp.tile;
             }
         } else {
             const bool bf16 = row_format == LFFN_ROWS_BF16;
             const GatherPlan qp = bf16 ? choose_quad<true>(B, T, S, Do) : choose_quad<false>(B, T, S, Do);
             if (qp.kind == 3 && room) {
-                kind = 3; tokens = 256 * qp.np;
+                kind = 3; tokens = qp.tile;
             } else {
                 int64_t each = bf16 ? gather_pieces<true>(B, T, S, Do) : gather_pieces<false>(B, T, S, Do);
                 if (each > B) each = B;
@@ -861,7 +877,7 @@ extern "C" int lffn_lookup_gather_plan(int64_t B, int64_t T, int64_t S, int64_t 
     if (B < 0 || T < 0 || Do < 1 || !lffn_is_pow2(S) || Do % 64 != 0) return LFFN_ERR_BAD_ARG;
     const GatherPlan plan = bf16 ? plan_gather<true>(B, T, S, Do) : plan_gather<false>(B, T, S, Do);
     if (tables_per_buffer) *tables_per_buffer = plan.kind;
-    return plan.kind == 0 ? 0 : (plan.kind == 1 ? 64 : (plan.kind == 3 ? 256 : 128)) * plan.np;
+    return plan.kind == 0 ? 0 : (plan.kind == 1 ? 64 : 128) * plan.np;
 }
 
 // ---------------------------------------------------------------- gather from a record stream
@@ -880,8 +896,8 @@ extern "C" int lffn_lookup_gather_records_plan_rows(int64_t B, int64_t T, int64_
         qp = row_format == LFFN_ROWS_BF16 ? choose_quad<true>(B, T, S, Do, false) : choose_quad<false>(B, T, S, Do, false);
     }
     if (qp.kind != 3) return LFFN_OK;
-    *tokens_per_workgroup = 256 * qp.np;
-    *record_stride = lffn_internal_quad_record_stride(B, qp.np);
+    *tokens_per_workgroup = qp.tile;
+    *record_stride = lffn_internal_quad_record_stride(B, row_format, qp.tile);
     *bytes = (T / 2) * 3 * *record_stride * 4;
     return LFFN_OK;
 }
@@ -896,15 +912,15 @@ extern "C" int lffn_lookup_gather_records_rows(const uint32_t *records, int64_t 
                                                int64_t S, int64_t Do, int32_t row_format, int32_t tokens_per_workgroup,
                                                void *stream) {
     LFFN_REQUIRE(B >= 0 && T >= 0 && Do >= 1 && tokens_per_workgroup > 0 && row_format >= 0 && row_format <= 2, LFFN_ERR_BAD_ARG);
-    LFFN_REQUIRE(tokens_per_workgroup % 256 == 0, LFFN_ERR_BAD_ARG);
-    const int np = tokens_per_workgroup / 256;
-    LFFN_REQUIRE(lffn_is_pow2(S) && Do % 64 == 0 && quad_plan_is_valid(row_format, np, B, T, S, Do), LFFN_ERR_UNSUPPORTED);
+    LFFN_REQUIRE(tokens_per_workgroup % 16 == 0, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_is_pow2(S) && Do % 64 == 0 && quad_plan_is_valid(row_format, tokens_per_workgroup, B, T, S, Do),
+                 LFFN_ERR_UNSUPPORTED);
     LFFN_REQUIRE(tables && out && (records || B == 0), LFFN_ERR_BAD_ARG);
     LFFN_REQUIRE(lffn_aligned16(tables) && lffn_aligned16(out) && (!bias || lffn_aligned16(bias)) &&
                      (!residual || lffn_aligned16(residual)) && (uintptr_t)records % 4 == 0, LFFN_ERR_BAD_ARG);
     if (B == 0) return LFFN_OK;
     return lffn_internal_lookup_gather_quad_records(records, record_stride, tables, bias, residual, out, B, T, S, Do,
-                                                    row_format, np, stream);
+                                                    row_format, tokens_per_workgroup, stream);
 }
 
 extern "C" int lffn_lookup_gather_records_f32(const uint32_t *records, int64_t record_stride, const float *tables,

@@ -71,9 +71,10 @@ struct QuadArgs {
     int64_t B;
     int T, S, Do;          // T even, S = 256
     int ntiles, nslices, per_xcd;
+    int tile_tokens;       // tokens per tile: a multiple of 16 in ((NP - 1) * 256, NP * 256]
     int row_bytes;         // Do * bytes per element
     const uint32_t *stream;     // [T/2][3][Bpad] record words written by pack_pairs_kernel
-    int64_t Bpad;               // B rounded up to whole token tiles: tokens past B have all-zero records
+    int64_t Bpad;               // words per plane: covers every token slot of every tile (lffn_internal_quad_record_stride)
 };
 
 // global_load_lds_dwordx4 / _dword with a scalar base and a 32-bit lane offset: lane i of the
@@ -216,7 +217,13 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
     // 128-byte segment comes first
     const bool second_first = (quad & 2) != 0;
     const int half0 = quad & 1;
-    const int64_t tok0 = int64_t(tile) * (256 * NP) + wave * 16 + quad;
+    // Tile `tile` holds tokens [tile * tile_tokens, (tile + 1) * tile_tokens), in groups of 16: group p * 16 + wave
+    // is pass p of wavefront `wave`.  tile_tokens need not fill the last pass: the wavefronts whose group of that
+    // pass lies beyond the tile leave the pass out (the launch balances the tiles: 16384 tokens over 10 workgroups
+    // are 1648 each, six passes and seven of sixteen wavefronts in the seventh, instead of nine full tiles of
+    // 1792 and a tenth that is mostly padding).
+    const int64_t tok0 = int64_t(tile) * a.tile_tokens + wave * 16 + quad;
+    const bool last_pass = (NP - 1) * 256 + wave * 16 < a.tile_tokens;        // uniform over the wavefront
 
     // acc[p][h][e]: token tok0 + 256 p, column ((half0 ^ h) * 4 + l) * EPV + e of the slice
     float acc[NP][2][EPV];
@@ -281,7 +288,7 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
     // at rec_lds + 4 (w * WAVE_RECS + r).  Copy instruction (w, n) brings word w of records 64n .. 64n+63
     // (lane i: record 64n + i), one word per lane.
     const uint32_t rec_lds = lds0 + 2u * BUF_BYTES + TOUCH_SINK_BYTES + (uint32_t)wave * (WAVE_RECS * REC_WORDS * 4);
-    const char *rec_base = reinterpret_cast<const char *>(a.stream + int64_t(tile) * (256 * NP) + wave * 16);
+    const char *rec_base = reinterpret_cast<const char *>(a.stream + int64_t(tile) * a.tile_tokens + wave * 16);
     const size_t plane_bytes = (size_t)a.Bpad * 4;
     // byte offset of word 0 of record (pass, quad) from rec_base: pass * 256 tokens further on
     const uint32_t rec_off = (uint32_t)(((lane >> 4) * 256 + (lane & 15)) * 4);
@@ -327,6 +334,12 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
     LdsRecord rec1 = read_record<WAVE_RECS>(rec_read1);
     __syncthreads();
 
+    // The loop over the table pairs for a wavefront that takes NPW of the NP passes (NP, or NP - 1 when its group
+    // of the last pass lies beyond the tile): two copies of the loop, chosen once, so that neither has a branch
+    // inside (a conditional in the loop body, even a uniform one, costs this kernel hundreds of spilled
+    // registers).  Both copies meet at the same barriers.
+    auto run_pairs = [&](auto npw_c) {
+    constexpr int NPW = decltype(npw_c)::value;
     for (int k = 0; k < npairs; ++k) {
 
         // Software pipeline over the passes: a pass's four rows are requested while the pass before
@@ -367,9 +380,9 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
             turn = turn + 1 == a.ntiles ? 0 : turn + 1;
         }
         __builtin_amdgcn_sched_barrier(0);
-        static_for<NP>([&](auto p_c) {
+        static_for<NPW>([&](auto p_c) {
             constexpr int P = decltype(p_c)::value;
-            constexpr bool MORE = P + 1 < NP;
+            constexpr bool MORE = P + 1 < NPW;
             using PN = std::integral_constant<int, MORE ? P + 1 : P>;
             if constexpr (MORE) pk = rows_of(PN{});
             const float w0 = score_of(p_c, I0{});
@@ -403,12 +416,15 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
         rec1 = read_record<WAVE_RECS>(rec_read1);
         __syncthreads();
     }
+    };
+    if (last_pass) run_pairs(std::integral_constant<int, NP>{});
+    else run_pairs(std::integral_constant<int, NP - 1>{});
     __builtin_amdgcn_s_waitcnt(WAIT_VMCNT_0);         // nothing may still be writing this workgroup's LDS when it ends
 
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
         const int64_t tok = tok0 + p * 256;
-        if (tok < a.B) {
+        if (tok < a.B && (p < NP - 1 || last_pass)) {
 #pragma unroll
             for (int h = 0; h < 2; ++h)
 #pragma unroll
@@ -427,7 +443,7 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
 
 template <int FMT, int NP, bool TOUCH>
 int launch_quad(QuadArgs a, hipStream_t stream) {
-    a.ntiles = (int)((a.B + 256 * NP - 1) / (256 * NP));
+    a.ntiles = (int)((a.B + a.tile_tokens - 1) / a.tile_tokens);
     const int units = a.ntiles * a.nslices;
     a.per_xcd = (units + XCDS - 1) / XCDS;
     // two buffers, the touches' scratch, every wavefront's records of one table pair
@@ -441,8 +457,8 @@ int launch_quad(QuadArgs a, hipStream_t stream) {
 
 }  // namespace
 
-// Bytes of the record stream for a shape: T/2 table pairs x the tokens rounded up to whole tiles
-// (at most 256 * 8 tokens more than B, whatever the tile size).
+// Bytes of the record stream for a shape: T/2 table pairs x the token slots of all tiles (fewer than 2048
+// more than B, whatever the tile size).
 int64_t lffn_internal_quad_stream_bytes(int64_t B, int64_t T) {
     return (T / 2) * (B + 2048) * (int64_t)(REC_WORDS * 4);
 }
@@ -455,19 +471,37 @@ bool lffn_internal_quad_np_built(int fmt, int np) {
     return (fmt == FMT_BF16 || fmt == FMT_F16) && np == 4;
 }
 
+// Passes a tile of `tokens` tokens takes: the smallest built number that covers it, or 0 (tokens: a multiple
+// of 16 in [16, 2048]).
+int lffn_internal_quad_passes(int fmt, int64_t tokens) {
+    if (tokens < 16 || tokens > 2048 || tokens % 16 != 0) return 0;
+    const int need = (int)((tokens + 255) / 256);
+    for (int np = need; np <= 8; ++np)
+        if (lffn_internal_quad_np_built(fmt, np)) return np;
+    return 0;
+}
+
+// Words per plane of the record stream for B tokens in tiles of `tokens`: the last tile's slots run to its
+// last pass's end whatever B is, since the gather copies a workgroup's records by whole passes.
+int64_t lffn_internal_quad_record_stride(int64_t B, int fmt, int64_t tokens) {
+    const int np = lffn_internal_quad_passes(fmt, tokens);
+    const int64_t ntiles = (B + tokens - 1) / tokens;
+    return (ntiles > 0 ? (ntiles - 1) * tokens : 0) + 256 * int64_t(np);      // < B + 2048
+}
+
 // Run the gather from a record stream [T/2][3][record_stride] (pack_pairs_kernel's layout; the projection
-// kernel of fht.hip writes the same) with 256*np tokens per workgroup.  The caller has checked that the
+// kernel of fht.hip writes the same) with `tokens` tokens per workgroup.  The caller has checked that the
 // shape qualifies: S = 256 (a table pair fills an LDS buffer), T even, Do a multiple of the slice's columns
 // (32 for fp32 rows, 64 for 16-bit rows), 2*S*Do*element bytes < 2^32 (32-bit lane offsets from a table
-// pair's base), np built for the format.  record_stride: whole tiles of 256*np tokens, at least B; what the
-// records of tokens from B on hold does not matter (their row numbers are bytes, always inside the LDS
-// buffer, and their sums are not stored).
+// pair's base), a tile size the format is built for.  record_stride: at least
+// lffn_internal_quad_record_stride(B, fmt, tokens); what the records of tokens from B on hold does not matter
+// (their row numbers are bytes, always inside the LDS buffer, and their sums are not stored).
 int lffn_internal_lookup_gather_quad_records(const uint32_t *records, int64_t record_stride, const void *tables,
                                              const float *bias, const float *residual, float *out, int64_t B,
-                                             int64_t T, int64_t S, int64_t Do, int fmt, int np, void *stream) {
-    if (!records || S != MAX_S || T % 2 != 0 || !lffn_internal_quad_np_built(fmt, np)) return LFFN_ERR_BAD_ARG;
-    const int64_t tile_tokens = 256 * int64_t(np);
-    if (record_stride % tile_tokens != 0 || record_stride < B) return LFFN_ERR_BAD_ARG;
+                                             int64_t T, int64_t S, int64_t Do, int fmt, int tokens, void *stream) {
+    const int np = lffn_internal_quad_passes(fmt, tokens);
+    if (!records || S != MAX_S || T % 2 != 0 || np == 0 || tokens <= 256 * (np - 1)) return LFFN_ERR_BAD_ARG;
+    if (record_stride < lffn_internal_quad_record_stride(B, fmt, tokens)) return LFFN_ERR_BAD_ARG;
     const int esz = fmt_bytes(fmt);
     if (Do % (SLICE_BYTES / esz) != 0) return LFFN_ERR_BAD_ARG;
     QuadArgs a{};
@@ -475,6 +509,7 @@ int lffn_internal_lookup_gather_quad_records(const uint32_t *records, int64_t re
     a.B = B; a.T = (int)T; a.S = (int)S; a.Do = (int)Do;
     a.nslices = (int)(Do * esz / SLICE_BYTES);
     a.row_bytes = (int)(Do * esz);
+    a.tile_tokens = tokens;
     a.Bpad = record_stride;
     a.stream = records;
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -490,22 +525,17 @@ int lffn_internal_lookup_gather_quad_records(const uint32_t *records, int64_t re
     }
 }
 
-int64_t lffn_internal_quad_record_stride(int64_t B, int np) {
-    const int64_t tile_tokens = 256 * int64_t(np);
-    return (B + tile_tokens - 1) / tile_tokens * tile_tokens;
-}
-
 // Pack the (code, score) pairs into the record stream in `workspace` (at least
 // lffn_internal_quad_stream_bytes(B, T) bytes, 16-byte aligned) and run the gather from it.
 int lffn_internal_lookup_gather_quad(const int32_t *code, const float *score, const void *tables,
                                      const float *bias, const float *residual, float *out, int64_t B, int64_t T,
-                                     int64_t S, int64_t Do, int fmt, int np, void *workspace, void *stream) {
-    if (!workspace || S != MAX_S || T % 2 != 0 || !lffn_internal_quad_np_built(fmt, np)) return LFFN_ERR_BAD_ARG;
+                                     int64_t S, int64_t Do, int fmt, int tokens, void *workspace, void *stream) {
+    if (!workspace || S != MAX_S || T % 2 != 0 || lffn_internal_quad_passes(fmt, tokens) == 0) return LFFN_ERR_BAD_ARG;
     uint32_t *recs = static_cast<uint32_t *>(workspace);
-    const int64_t stride = lffn_internal_quad_record_stride(B, np);
+    const int64_t stride = lffn_internal_quad_record_stride(B, fmt, tokens);
     const dim3 grid((unsigned)((stride + 63) / 64), (unsigned)((T / 2 + 31) / 32));
     hipLaunchKernelGGL(pack_pairs_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), code, score, recs, B,
                        stride, (int)T, (int)S);
     if (hipGetLastError() != hipSuccess) return LFFN_ERR_LAUNCH;
-    return lffn_internal_lookup_gather_quad_records(recs, stride, tables, bias, residual, out, B, T, S, Do, fmt, np, stream);
+    return lffn_internal_lookup_gather_quad_records(recs, stride, tables, bias, residual, out, B, T, S, Do, fmt, tokens, stream);
 }

@@ -210,7 +210,7 @@ def test_workspace_queries_are_host_side_plans():
         tokens = lib.lffn_lookup_gather_ws_plan(B, T, S, Do, fmt, ws, ctypes.byref(form))
         return form.value, tokens
 
-    assert ws_plan(16384, 128, 256, 768) == (3, 1792)           # RoBERTa-base: 10 tiles x 24 slices
+    assert ws_plan(16384, 128, 256, 768) == (3, 1648)           # RoBERTa-base: 10 tiles of 103 groups of 16 tokens x 24 slices
     assert ws_plan(16384, 512, 256, 1024) == (3, 2048)
     assert ws_plan(16384, 512, 256, 1024, 1) == (3, 1024) and ws_plan(16384, 512, 256, 1024, 2) == (3, 1024)
     assert ws_plan(16384, 128, 256, 768, 0, 0) == plan(16384, 128, 256, 768)       # no workspace: the plain entry's kernel

@@ -517,7 +517,7 @@ def test_ln_project_hash_matches_oracle(H, D, R, T):
 # workgroup of the projection kernel and a quad; two repeats of a short transform (rows shared by four
 # tokens per wavefront); an odd number of table pairs
 # what lffn_lookup_gather_records_plan picks at configs 2 and 3: (tokens per workgroup, record stride, bytes)
-CONFIG2_RECORD_PLAN = (1792, 17920, 6 * 128 * 17920)        # 10 tiles x 24 slices
+CONFIG2_RECORD_PLAN = (1648, 16624, 6 * 128 * 16624)        # 10 tiles of 103 groups of 16 tokens x 24 slices
 CONFIG3_RECORD_PLAN = (2048, 16384, 6 * 512 * 16384)        # 8 tiles x 32 slices
 RECORD_LAYERS = [(16384, 768, 1024, 1, 128, 768, None), (4099, 768, 1024, 1, 128, 768, (1024, 5120)),
                  (5000, 100, 128, 2, 30, 128, (1536, 6144)), (2050, 64, 64, 1, 6, 64, (2048, 4096)),
@@ -614,7 +614,9 @@ def test_record_stream_plan_and_refusals():
     assert bad(4096, 256, None, None, 256, 3000, 20, 256, 256, 1000) == _lib.LFFN_ERR_BAD_ARG            # not whole passes
     assert bad(4096, 256, None, None, 256, 3000, 20, 256, 256, 1280) == _lib.LFFN_ERR_UNSUPPORTED        # 5 passes: not built
     assert bad(4096, 256, None, None, 256, 3000, 21, 256, 256, 1024) == _lib.LFFN_ERR_UNSUPPORTED        # odd T
-    assert bad(4000, 256, None, None, 256, 3000, 20, 256, 256, 1024) == _lib.LFFN_ERR_BAD_ARG            # stride not whole tiles
+    assert bad(3008, 256, None, None, 256, 3000, 20, 256, 256, 1024) == _lib.LFFN_ERR_BAD_ARG            # stride short of the last tile's passes
+    assert bad(4096, 256, None, None, 256, 3000, 20, 256, 256, 1032) == _lib.LFFN_ERR_BAD_ARG            # not whole groups of 16
+    assert bad(4096, 256, None, None, 256, 3000, 20, 256, 256, 1040) == _lib.LFFN_ERR_UNSUPPORTED        # 5 passes: not built
     assert bad(2048, 256, None, None, 256, 3000, 20, 256, 256, 1024) == _lib.LFFN_ERR_BAD_ARG            # stride < B
     assert lib.lffn_ln_project_hash_records_f32(256, 256, 256, 1e-5, 256, None, 256, 100, 300, 64, 64, 1, 4, 6, 0.7, 0.3, None) \
         == _lib.LFFN_ERR_BAD_ARG                                                                         # stride < B
@@ -932,7 +934,9 @@ def test_lookup_gather_workspace_query_is_zero_where_the_plain_form_is_as_fast()
 # The four-lanes-per-token kernel (form 3), every tile size that is built, forced onto shapes it would not
 # be chosen for.  (B, T, 256, Do): token counts that end inside a tile, a wavefront and a quad; 1 to 17
 # table pairs; one column slice and several.
-QUAD_PLANS = [(3, 1024), (3, 1536), (3, 1792), (3, 2048)]
+QUAD_PLANS = [(3, 1024), (3, 1536), (3, 1792), (3, 2048),
+              # tiles whose last pass is short for some or most of a workgroup's wavefronts
+              (3, 1648), (3, 784), (3, 2032), (3, 1296)]
 QUAD_SHAPES = [(3000, 20, 256, 256), (4133, 6, 256, 384), (1793, 34, 256, 128), (1, 2, 256, 64), (2050, 8, 256, 192)]
 
 
@@ -1151,7 +1155,7 @@ def test_four_lane_gather_and_record_layer_on_random_shapes():
         want = np.einsum("bt,btd->bd", score.astype(np.float64), tables[np.arange(T)[None, :], code].astype(np.float64))
         want = want + (0 if bias is None else bias) + (0 if res is None else res)
         scale = np.abs(want).max()
-        for tok in (1024, 1536, 1792, 2048):
+        for tok in (1024, 1536, 1792, 2048, 1648, 784, 2032):
             rc, got = cabi.lookup_gather_ws_planned(code, score, tables, (3, tok), bias=bias, residual=res)
             assert rc == 0 and np.abs(got - want).max() <= 1e-5 * scale, (it, B, T, Do, tok)
         got = cabi.lookup_gather_ws(code, score, tables, bias, residual=res)
@@ -1163,8 +1167,8 @@ def test_four_lane_gather_and_record_layer_on_random_shapes():
         T = 2 * int(rng.randint(1, R * D // 16 + 1))
         Do = int(rng.choice([64, 128, 256]))
         B = int(rng.choice([1, 3, 5, 31, 33, 257, 1000, 2049]))
-        tok = int(rng.choice([1024, 1536, 1792, 2048]))
-        stride = -(-B // tok) * tok
+        tok = int(rng.choice([1024, 1536, 1792, 2048, 1648, 1008]))
+        stride = -(-B // tok) * tok + 256
         x = (rng.randn(B, H) * 1.5 + 0.3).astype(np.float32)
         ln_w = (1 + 0.1 * rng.randn(H)).astype(np.float32)
         ln_b = (0.1 * rng.randn(H)).astype(np.float32)
