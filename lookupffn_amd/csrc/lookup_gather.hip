@@ -407,18 +407,21 @@ GatherPlan plan_quad(int fmt, int64_t B, int64_t T, int64_t S, int64_t Do, bool 
     const double per_pass = fmt == LFFN_ROWS_F32 ? QUAD_US_PER_PAIR_PASS : QUAD_US_PER_PAIR_PASS_16[fmt];
     for (int np : {4, 6, 7, 8}) {
         if (!lffn_internal_quad_np_built(fmt, np)) continue;
-        // as many tiles as tiles of np full passes would take, the tokens spread evenly over them (in groups of
-        // 16): the last pass is then short for some of a workgroup's wavefronts, which leave it out.  What a short
-        // pass costs was measured as about half a pass plus its share of the reads.
-        const int64_t tiles = (B + 256 * np - 1) / (256 * np);
-        int64_t tile = (((B + tiles - 1) / tiles) + 15) & ~int64_t(15);
-        if (tile <= 256 * (np - 1)) tile = 256 * (np - 1) + 16;
-        const int64_t rem = tile - 256 * (np - 1);                                 // tokens in the last pass: 16 .. 256
-        const double passes = double(np - 1) + (rem == 256 ? 1.0 : 0.5 + 0.5 * double(rem) / 256.0);
-        const int64_t rounds = (tiles * nslices + 255) / 256;
-        const double us = double(rounds) * double(T / 2) * (QUAD_US_PER_PAIR + passes * per_pass) +
-                          (pack ? double(B) * double(T) * 14.0 / 3e6 + 4.0 : 0.0);     // packing: 8 bytes read, 6 written per (token, table)
-        if (us < best.us) best = GatherPlan{3, np, us, (int)tile};
+        // Tiles of np passes, the tokens spread evenly over them in groups of 16: from as few tiles as np full
+        // passes allow up to as many as still need np passes.  The last pass is then short for some of a
+        // workgroup's wavefronts, which leave it out; what a short pass costs was measured as about half a pass
+        // plus its share of the reads.  More, shorter tiles can fill workgroup slots that fewer, fuller ones leave
+        // idle (16384 tokens x 12 slices of 16-bit rows: 21 tiles of 784 tokens = 252 workgroups, not 16 x 12 = 192).
+        for (int64_t tiles = (B + 256 * np - 1) / (256 * np);; ++tiles) {
+            const int64_t tile = (((B + tiles - 1) / tiles) + 15) & ~int64_t(15);
+            if (tile <= 256 * (np - 1)) break;
+            const int64_t rem = tile - 256 * (np - 1);                                 // tokens in the last pass: 16 .. 256
+            const double passes = double(np - 1) + (rem == 256 ? 1.0 : 0.5 + 0.5 * double(rem) / 256.0);
+            const int64_t rounds = (tiles * nslices + 255) / 256;
+            const double us = double(rounds) * double(T / 2) * (QUAD_US_PER_PAIR + passes * per_pass) +
+                              (pack ? double(B) * double(T) * 14.0 / 3e6 + 4.0 : 0.0);     // packing: 8 bytes read, 6 written per (token, table)
+            if (us < best.us) best = GatherPlan{3, np, us, (int)tile};
+        }
     }
     return best;
 }
