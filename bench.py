@@ -1,6 +1,6 @@
 """Benchmark of the LookupFFN hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg1|cfg3|cfg3bf16|cfg2b64|cfg4|cfg5]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg1|cfg3|cfg3bf16|cfg3f16|cfg2b64|cmp512|cfg4|cfg5]
 
 A step is one forward pass of the layer over one batch of synthetic tokens that
 is already resident in HBM: fused LayerNorm+projection+hash kernel -> gather-add
@@ -17,6 +17,9 @@ kernel (+bias), i.e. LookupFFN.forward in eval mode.  Prints ONE JSON line:
                and the "logical" rate (every row read counted as memory traffic)
                as logical_gbps.  Small shapes run the token-major form (rows from
                L2): there the bound is "hbm" and achieved counts the compulsory bytes.
+               16-bit rows (cfg3bf16, cfg3f16) halve the LDS bytes and are bound by the
+               vector ALU instead (bound "valu": widenings + multiply-adds per second
+               against 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz), the LDS rate beside it.
   cpu_baseline the CPU oracle (OpenMP C restatement of the reference's layer) on a
                bounded sample of the same workload, on the host cores of this box
 
@@ -79,6 +82,9 @@ LDS_READ_PEAK_GBS = 256 * 256 * 2.4
 LDS_PROBED_GBS = 145 * 256 * 2.4          # what that probe reads for the gather's access pattern
 LDS_PEAK_BASIS = ("256 B/clk/CU x 256 CUs x 2.4 GHz; a read-only ds_read_b128 probe on this part reaches 180 B/clk/CU "
                   "(linear) and 145 B/clk/CU (16 lanes per random 256-byte row, this kernel's pattern)")
+# Vector ALU: 4 SIMDs x 16 lanes per CU, one fp32 operation per lane and clock (packed fp32 instructions are
+# switched off in this build), 256 CUs at 2.4 GHz
+VALU_PEAK_GOPS = 256 * 4 * 16 * 2.4
 # L2 read path: 16 channels x 128 B/clk per XCD, 8 XCDs, 2.4 GHz
 L2_READ_PEAK_GBS = 16 * 128 * 8 * 2.4
 # HBM-side bytes per launch of the gather (cfg5: scatter) kernels measured with rocprofv3 --pmc
@@ -86,11 +92,12 @@ L2_READ_PEAK_GBS = 16 * 128 * 8 * 2.4
 # measured on; the summaries are kept under profiles/.  Reported only while the library still runs
 # that form for the workload (a figure for another kernel would be stale).
 MEASURED_TRAFFIC = {
-    "cfg2": {"bytes": 268604915, "form": "record stream (four lanes per token), 1792 tokens per workgroup"},
-    "cfg2b64": {"bytes": 268655264, "form": "record stream (four lanes per token), 1792 tokens per workgroup"},
-    "cfg3": {"bytes": 1092682313, "form": "record stream (four lanes per token), 2048 tokens per workgroup"},
-    "cfg3bf16": {"bytes": 1393399611, "form": "1 table(s) per LDS buffer, 512 tokens per workgroup"},
-    "cfg5": {"bytes": 944068093, "form": "sorted"},
+    "cfg2": {"bytes": 253976359, "form": "record stream (four lanes per token), 1648 tokens per workgroup"},
+    "cfg2b64": {"bytes": 254108069, "form": "record stream (four lanes per token), 1648 tokens per workgroup"},
+    "cfg3": {"bytes": 1089426341, "form": "record stream (four lanes per token), 2048 tokens per workgroup"},
+    "cfg3bf16": {"bytes": 752371096, "form": "record stream (four lanes per token), 1024 tokens per workgroup"},
+    "cfg3f16": {"bytes": 768074365, "form": "record stream (four lanes per token), 1024 tokens per workgroup"},
+    "cfg5": {"bytes": 943818300, "form": "sorted"},
 }
 
 
@@ -609,7 +616,22 @@ def main():
     hbm = {"compulsory_bytes": compulsory, "frac_of_peak": compulsory / (gather_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
            "measured_traffic_bytes": traffic,
            "measured_frac_of_peak": None if traffic is None else traffic / (gather_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
-    if lds_bound:
+    if lds_bound and fmt != 0 and form.startswith("record stream"):
+        # 16-bit rows in the four-lanes kernel: half the LDS bytes per column, and one (half: v_fma_mix_f32) or two
+        # (bfloat16: widen, multiply-add) vector-ALU operations per column and (token, table): that kernel is bound
+        # by vector-ALU issue, not by the LDS
+        vec_ops = B * T * Do * (2 if fmt == 1 else 1)
+        achieved = vec_ops / (gather_ms * 1e-3) / 1e9
+        lds_rate = row_bytes / (gather_ms * 1e-3) / 1e9
+        roofline = {"bound": "valu", "kernel": "lookup_gather: " + form, "achieved": achieved, "peak": VALU_PEAK_GOPS,
+                    "unit": "Gop/s", "frac": achieved / VALU_PEAK_GOPS,
+                    "peak_basis": "256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz, one fp32 operation per lane and clock (no packed "
+                                  "fp32); counted: " + ("a widening and a multiply-add" if fmt == 1 else "one v_fma_mix_f32") +
+                                  " per column of every (token, table) row",
+                    "traffic": traffic, "vector_ops": vec_ops, "avg_kernel_ms": gather_ms,
+                    "lds": {"row_read_bytes": row_bytes, "achieved_gbps": lds_rate, "frac_of_peak": lds_rate / LDS_READ_PEAK_GBS},
+                    "hbm": hbm, "logical_gbps": logical_gbps, "algorithmic_bytes": gather_bytes}
+    elif lds_bound:
         achieved = row_bytes / (gather_ms * 1e-3) / 1e9
         roofline = {"bound": "lds", "kernel": "lookup_gather: " + form, "achieved": achieved, "peak": LDS_READ_PEAK_GBS,
                     "unit": "GB/s", "frac": achieved / LDS_READ_PEAK_GBS, "frac_of_probed": achieved / LDS_PROBED_GBS,
