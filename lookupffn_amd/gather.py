@@ -31,7 +31,12 @@ def weighted_vector_gather_add(indexes, source, weights, use_torch=False):
     """outputs[b] = sum_i weights[b,i] * source[indexes[b,i]]   (PL/gather/cuda/kernel.py:22-70)."""
     _check(indexes, source, weights, "gather")
     assert source.dtype in [torch.float32, torch.bfloat16, torch.float16], source.dtype
-    assert weights.dtype == torch.float32, weights.dtype
+    assert weights.dtype in [torch.float32, torch.float16], weights.dtype
+    half_call = weights.dtype == torch.float16
+    if half_call:
+        # the reference's half-precision call (PL/gather/cuda/kernel.py:64-67): half rows, half weights, half
+        # result.  Here the sums are fp32 and the result is rounded to half once
+        assert source.dtype == torch.float16, source.dtype
     batch_size, index_size = indexes.shape
     source_size, vector_dim = source.shape
     assert weights.shape[0] == batch_size and weights.shape[1] == index_size
@@ -49,6 +54,8 @@ def weighted_vector_gather_add(indexes, source, weights, use_torch=False):
         for batch_idx in range(batch_size):
             output_list.append(checkpoint(mini_batching, source, indexes, weights, batch_idx, use_reentrant=False))
         return torch.stack(output_list, dim=0)
+    if half_call:
+        return ops.gather_add(indexes, source, weights.float()).half()
     return ops.gather_add(indexes, source, weights)
 
 

@@ -301,6 +301,10 @@ def test_f16_tables_inference_and_general_gather():
     got = lookupffn_amd.weighted_gather_add(torch.tensor(idx_np, device=DEV), src, w)
     want = oracle.gather_add(idx_np, npf(src).astype(np.float64), npf(w).astype(np.float64))
     assert got.dtype == torch.float32 and relmax(npf(got), want) <= 1e-5
+    # the reference's half-precision call shape: half rows, half weights, half result (rounded once from the fp32 sum)
+    got16 = lookupffn_amd.weighted_gather_add(torch.tensor(idx_np, device=DEV), src, w.half())
+    want16 = oracle.gather_add(idx_np, npf(src).astype(np.float64), npf(w.half()).astype(np.float64))
+    assert got16.dtype == torch.float16 and relmax(npf(got16), want16) <= 2 ** -10
 
 
 def test_reference_call_sequence_of_lookup_gather():
