@@ -46,6 +46,9 @@ __global__ __launch_bounds__(256) void bh4_wgrad_kernel(const float *__restrict_
     const float *p = stage_grads + (size_t)s * B * D;
     const float *u = j == 0 ? x : stage_inputs + (size_t)(r * (J - 1) + j - 1) * B * D;
     const int Hu = j == 0 ? H : D, ldu = Hu;
+    // a block of the first stage that lies wholly in the zero padding beyond column H has a zero input,
+    // hence a zero gradient: g keeps what it holds (768 columns padded to 1024: 4 of 16 blocks)
+    if (n * BS >= Hu) return;                      // uniform over the workgroup
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int c = lane & 15;
