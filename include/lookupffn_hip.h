@@ -356,10 +356,11 @@ int lffn_ln_project_hash_f32(const float *x, const float *ln_weight, const float
  *
  * lffn_lookup_gather_records_plan: host-side query.  When this form is the one to use for a shape
  * (fp32 rows, S = 256, an even number of tables, enough tokens: the conditions under which
- * lffn_lookup_gather_workspace_bytes asks for a record stream) it sets *tokens_per_workgroup (1024,
- * 1536, 1792 or 2048), *record_stride (B rounded up to whole workgroup tiles) and *bytes (the size of
- * the stream: 6 * T * record_stride); otherwise all three are 0 and the caller uses the other entry
- * points.
+ * lffn_lookup_gather_workspace_bytes asks for a record stream, without the cost of the packing kernel)
+ * it sets *tokens_per_workgroup (a multiple of 16 up to 2048: the tokens are spread evenly over the
+ * workgroups of a slice), *record_stride (words per plane: the token slots of all tiles, fewer than
+ * B + 2048) and *bytes (the size of the stream: 6 * T * record_stride); otherwise all three are 0 and
+ * the caller uses the other entry points.
  *
  * lffn_ln_project_hash_records_f32: lffn_ln_project_hash_f32 (ln_weight and ln_bias both NULL: no
  * LayerNorm, as lffn_project_hash_f32) with its codes and scores written as records: 4-byte aligned
@@ -371,8 +372,9 @@ int lffn_ln_project_hash_f32(const float *x, const float *ln_weight, const float
  * D >= 16.  The layout is private to these entry points: write it with this call only.
  *
  * lffn_lookup_gather_records_f32: out[b,:] = residual[b,:] + bias + sum_t score[b,t] * tables[t, code[b,t], :]
- * from such a stream, with the tokens_per_workgroup and record_stride the plan gave.  Results are
- * bit-identical to lffn_lookup_gather_ws_f32's for the same shape.  bias and residual may be NULL.
+ * from such a stream, with the tokens_per_workgroup the plan gave and a record_stride of at least the
+ * plan's.  Results are bit-identical to lffn_lookup_gather_ws_f32's for the same shape.  bias and
+ * residual may be NULL.
  *
  * lffn_lookup_gather_records_plan_rows / lffn_lookup_gather_records_rows: the same two calls for any
  * row format (row_format 0 fp32, 1 bfloat16, 2 half; tables typed accordingly).  16-bit rows run 1024
@@ -553,11 +555,13 @@ int lffn_lookup_gather_plan(int64_t B, int64_t T, int64_t S, int64_t Do, int32_t
  * bf16 512, 1024), ignored for 0.  LFFN_ERR_UNSUPPORTED if that kernel is not built or
  * the shape does not meet its conditions (S <= 256, Do a multiple of the slice width).
  * lffn_lookup_gather_ws_planned_f32 also takes residual and a workspace and with them
- * form 3, the four-lanes-per-token kernel (tokens_per_workgroup 1024, 1536, 1792 or
- * 2048; S = 256, T even, Do a multiple of 32; the workspace must hold the record
- * stream, 6 * T * (B + 2048) bytes, or the call is refused with LFFN_ERR_UNSUPPORTED).
+ * form 3, the four-lanes-per-token kernel (tokens_per_workgroup any multiple of 16
+ * from 784 to 2048: a workgroup takes its tokens in passes of 256, 4 to 8 of them, and
+ * wavefronts whose share of the last pass lies beyond the tile leave it out; S = 256, T
+ * even, Do a multiple of 32; the workspace must hold the record stream, 6 * T * (B + 2048)
+ * bytes, or the call is refused with LFFN_ERR_UNSUPPORTED).
  * lffn_lookup_gather_ws_planned_rows is the same for any row format (row_format 0 fp32,
- * 1 bfloat16, 2 half; tables typed accordingly): 16-bit rows take form 3 with 1024
+ * 1 bfloat16, 2 half; tables typed accordingly): 16-bit rows take form 3 with 784 to 1024
  * tokens per workgroup and Do a multiple of 64; half rows take forms 0 and 3 only.
  * No counterpart in the reference.
  */

@@ -352,7 +352,7 @@ struct GatherPlan {
 
 // The four-lanes-per-token kernel: microseconds per table pair of a workgroup = a fixed part (the 64 KB
 // copy, the records, the barrier) + a part per pass of 256 tokens.  Measured on MI355X at 4, 6, 7 and 8
-// passes of fp32 rows: 1.40, 1.74, 1.93, 2.18 us, the same for 128 x 256 x 768 fp32 tables (in the memory-side
+// passes of fp32 rows (5 passes were added later and lie on the same line): 1.40, 1.74, 1.93, 2.18 us, the same for 128 x 256 x 768 fp32 tables (in the memory-side
 // cache) and 512 x 256 x 1024 (537 MB, beyond it: the touch by turns hides the difference).  A pass over
 // 16-bit rows covers twice the columns and is bound by the vector ALU: QUAD_US_PER_PAIR_PASS_16[format].
 constexpr double QUAD_MARGIN = 0.92;      // the form must promise this much to be worth its workspace
@@ -405,7 +405,7 @@ GatherPlan plan_quad(int fmt, int64_t B, int64_t T, int64_t S, int64_t Do, bool 
     const int64_t nslices = Do / cols;
     if (((B + 1023) / 1024) * nslices < 192 || B * nslices > (int64_t(1) << 30)) return best;
     const double per_pass = fmt == LFFN_ROWS_F32 ? QUAD_US_PER_PAIR_PASS : QUAD_US_PER_PAIR_PASS_16[fmt];
-    for (int np : {4, 6, 7, 8}) {
+    for (int np : {4, 5, 6, 7, 8}) {
         if (!lffn_internal_quad_np_built(fmt, np)) continue;
         // Tiles of np passes, the tokens spread evenly over them in groups of 16: from as few tiles as np full
         // passes allow up to as many as still need np passes.  The last pass is then short for some of a

@@ -467,7 +467,7 @@ int64_t lffn_internal_quad_stream_bytes(int64_t B, int64_t T) {
 // pass and lane for fp32 rows and 16 for 16-bit rows, must fit the 128 registers a lane of a 1024-lane
 // workgroup can have.
 bool lffn_internal_quad_np_built(int fmt, int np) {
-    if (fmt == FMT_F32) return np == 4 || np == 6 || np == 7 || np == 8;
+    if (fmt == FMT_F32) return np >= 4 && np <= 8;
     return (fmt == FMT_BF16 || fmt == FMT_F16) && np == 4;
 }
 
@@ -521,6 +521,7 @@ int lffn_internal_lookup_gather_quad_records(const uint32_t *records, int64_t re
         case 8: return launch_quad<FMT_F32, 8, true>(a, st);
         case 7: return launch_quad<FMT_F32, 7, true>(a, st);
         case 6: return launch_quad<FMT_F32, 6, true>(a, st);
+        case 5: return launch_quad<FMT_F32, 5, true>(a, st);
         default: return launch_quad<FMT_F32, 4, true>(a, st);
     }
 }

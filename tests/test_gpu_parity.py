@@ -612,11 +612,11 @@ def test_record_stream_plan_and_refusals():
     # (records, stride, tables, bias, residual, out, B, T, S, Do, tokens): refused before any launch
     bad = lambda *a: lib.lffn_lookup_gather_records_f32(256, *a, None)
     assert bad(4096, 256, None, None, 256, 3000, 20, 256, 256, 1000) == _lib.LFFN_ERR_BAD_ARG            # not whole passes
-    assert bad(4096, 256, None, None, 256, 3000, 20, 256, 256, 1280) == _lib.LFFN_ERR_UNSUPPORTED        # 5 passes: not built
+    assert bad(4096, 256, None, None, 256, 3000, 20, 256, 256, 512) == _lib.LFFN_ERR_UNSUPPORTED         # two passes: not built
     assert bad(4096, 256, None, None, 256, 3000, 21, 256, 256, 1024) == _lib.LFFN_ERR_UNSUPPORTED        # odd T
     assert bad(3008, 256, None, None, 256, 3000, 20, 256, 256, 1024) == _lib.LFFN_ERR_BAD_ARG            # stride short of the last tile's passes
     assert bad(4096, 256, None, None, 256, 3000, 20, 256, 256, 1032) == _lib.LFFN_ERR_BAD_ARG            # not whole groups of 16
-    assert bad(4096, 256, None, None, 256, 3000, 20, 256, 256, 1040) == _lib.LFFN_ERR_UNSUPPORTED        # 5 passes: not built
+    assert bad(8192, 256, None, None, 256, 3000, 20, 256, 256, 2304) == _lib.LFFN_ERR_UNSUPPORTED        # nine passes: not built
     assert bad(2048, 256, None, None, 256, 3000, 20, 256, 256, 1024) == _lib.LFFN_ERR_BAD_ARG            # stride < B
     assert lib.lffn_ln_project_hash_records_f32(256, 256, 256, 1e-5, 256, None, 256, 100, 300, 64, 64, 1, 4, 6, 0.7, 0.3, None) \
         == _lib.LFFN_ERR_BAD_ARG                                                                         # stride < B
@@ -936,7 +936,7 @@ def test_lookup_gather_workspace_query_is_zero_where_the_plain_form_is_as_fast()
 # table pairs; one column slice and several.
 QUAD_PLANS = [(3, 1024), (3, 1536), (3, 1792), (3, 2048),
               # tiles whose last pass is short for some or most of a workgroup's wavefronts
-              (3, 1648), (3, 784), (3, 2032), (3, 1296)]
+              (3, 1648), (3, 784), (3, 2032), (3, 1296), (3, 1280), (3, 1200)]
 QUAD_SHAPES = [(3000, 20, 256, 256), (4133, 6, 256, 384), (1793, 34, 256, 128), (1, 2, 256, 64), (2050, 8, 256, 192)]
 
 
@@ -1007,7 +1007,7 @@ def test_lookup_gather_quad_refusals():
     from lookupffn_amd import _lib
     rng = np.random.RandomState(3)
     tables, code, idx, w = _rand_gather(rng, 300, 20, 256, 64)
-    assert cabi.lookup_gather_ws_planned(code, w, tables, (3, 1280))[0] == _lib.LFFN_ERR_UNSUPPORTED      # 5 passes: not built
+    assert cabi.lookup_gather_ws_planned(code, w, tables, (3, 512))[0] == _lib.LFFN_ERR_UNSUPPORTED       # two passes: not built
     assert cabi.lookup_gather_ws_planned(code, w, tables, (3, 1000))[0] == _lib.LFFN_ERR_BAD_ARG
     assert cabi.lookup_gather_ws_planned(code, w, tables, (3, 1024), ws_bytes=0)[0] == _lib.LFFN_ERR_UNSUPPORTED   # no room for the records
     assert cabi.lookup_gather_ws_planned(code, w, tables, (3, 1024), ws_bytes=6 * 20 * 300)[0] == _lib.LFFN_ERR_UNSUPPORTED
