@@ -412,7 +412,8 @@ GatherPlan plan_quad(int fmt, int64_t B, int64_t T, int64_t S, int64_t Do, bool 
         // workgroup's wavefronts, which leave it out; what a short pass costs was measured as about half a pass
         // plus its share of the reads.  More, shorter tiles can fill workgroup slots that fewer, fuller ones leave
         // idle (16384 tokens x 12 slices of 16-bit rows: 21 tiles of 784 tokens = 252 workgroups, not 16 x 12 = 192).
-        for (int64_t tiles = (B + 256 * np - 1) / (256 * np);; ++tiles) {
+        const int64_t tiles_min = (B + 256 * np - 1) / (256 * np);
+        for (int64_t tiles = tiles_min; tiles <= tiles_min + 32; ++tiles) {       // (filling a round of 256 workgroups never takes more)
             const int64_t tile = (((B + tiles - 1) / tiles) + 15) & ~int64_t(15);
             if (tile <= 256 * (np - 1)) break;
             const int64_t rem = tile - 256 * (np - 1);                                 // tokens in the last pass: 16 .. 256
