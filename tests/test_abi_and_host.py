@@ -227,6 +227,59 @@ def test_workspace_queries_are_host_side_plans():
         assert scatter_ws(*shape) == 0, shape
 
 
+def test_gather_plans_are_consistent_over_a_grid_of_shapes():
+    """Host-side sweep of the three gather queries over 15 000 shapes (ragged token counts, odd table
+    counts, every row format).  Whenever the workspace entry point would run the four-lanes-per-token
+    kernel, the record stream its plan describes fits the workspace the size query asked for, the tile
+    is one the kernel is built for and the planes cover every token slot of every tile; the stand-alone
+    record plan obeys the same rules (it may choose the form for more shapes: its records come from the
+    projection kernel, so it does not count a packing kernel)."""
+    lib = _lib.load()
+    passes_built = {0: (4, 5, 6, 7, 8), 1: (4,), 2: (4,)}
+    seen = {}
+
+    def check_tile(fmt, B, T, S, tokens, stride, nbytes):
+        assert S == 256 and T % 2 == 0
+        assert tokens % 16 == 0 and 16 <= tokens <= 2048
+        np_ = -(-tokens // 256)
+        assert np_ in passes_built[fmt], (fmt, tokens)
+        ntiles = -(-B // tokens)
+        assert stride == (ntiles - 1) * tokens + 256 * np_          # the last tile's slots are whole passes
+        assert B <= stride < B + 2048
+        assert nbytes == 6 * T * stride
+
+    for B in (1, 15, 16, 255, 256, 1000, 2047, 2048, 3000, 4096, 5000, 8192, 10000, 12000, 16383, 16384,
+              16385, 20000, 32768, 50000, 65536, 100000, 262144):
+        for T in (2, 3, 16, 32, 128, 130, 512):
+            for S in (16, 64, 128, 256):
+                for Do in (64, 128, 192, 256, 512, 768, 1024, 2048):
+                    for fmt in (0, 1, 2):
+                        shape = (B, T, S, Do, fmt)
+                        nb = ctypes.c_int64(-1)
+                        assert lib.lffn_lookup_gather_workspace_bytes(B, T, S, Do, fmt, ctypes.byref(nb)) == 0, shape
+                        assert nb.value >= 0
+                        form = ctypes.c_int32(-1)
+                        tokens = lib.lffn_lookup_gather_ws_plan(B, T, S, Do, fmt, nb.value, ctypes.byref(form))
+                        assert form.value in (0, 1, 2, 3, 4) and tokens >= 0, shape
+                        seen[form.value] = seen.get(form.value, 0) + 1
+                        tpw, rs, by = ctypes.c_int32(-1), ctypes.c_int64(-1), ctypes.c_int64(-1)
+                        assert lib.lffn_lookup_gather_records_plan_rows(B, T, S, Do, fmt, ctypes.byref(tpw),
+                                                                        ctypes.byref(rs), ctypes.byref(by)) == 0, shape
+                        if form.value == 3:
+                            # the workspace form packs the same stream: same tile, and it fits what was asked for
+                            assert tpw.value == tokens, shape
+                            assert by.value <= nb.value, shape
+                        if tpw.value:
+                            check_tile(fmt, B, T, S, tpw.value, rs.value, by.value)
+                        else:
+                            assert rs.value == 0 and by.value == 0 and form.value != 3, shape
+                        if form.value == 0:
+                            assert tokens == 0, shape
+                        if nb.value == 0:
+                            assert form.value in (0, 1, 2), shape       # nothing that needs a workspace
+    assert all(seen.get(f, 0) > 100 for f in (0, 1, 2, 3, 4)), seen    # the grid reaches every form
+
+
 def test_module_surface_matches_reference_names_and_shapes():
     m = lookupffn_amd.LookupFFN(_config(hidden_size=768, ffn_num_table=128, block_size=64), 768)
     sd = m.state_dict()
