@@ -17,7 +17,7 @@
  *     results between calls (it remembers, per device, which kernels were granted
  *     large LDS sizes and where its one static scratch array lives).
  *   - Forward outputs are fully overwritten (no zero-initialisation needed).
- *     Only lffn_scatter_add_f32 accumulates into its output.
+ *     Only lffn_scatter_add_f32 / _f16 accumulate into their output.
  *   - Calls are asynchronous on `stream` (NULL = the legacy default stream) and
  *     may be issued from any host thread.
  *   - Return value: LFFN_OK, or a negative LFFN_ERR_* code.  Nothing throws or
@@ -41,7 +41,7 @@ extern "C" {
 #define LFFN_ERR_LAUNCH      -3   /* hipGetLastError() after the launch was not hipSuccess */
 #define LFFN_ERR_SCRATCH     -4   /* an entry point that allocates nothing: the shape exceeds its static scratch */
 
-#define LFFN_ABI_VERSION 6
+#define LFFN_ABI_VERSION 7
 
 /* ABI version of the loaded library (LFFN_ABI_VERSION at build time). */
 int lffn_version(void);
@@ -602,6 +602,25 @@ int lffn_indexed_inner_product_f32(const int32_t *idx, const float *g, const flo
  * Replaces gather_add.weighted_vector_scatter_add_fp32 (gather_fp32.cu:38-67).
  */
 int lffn_scatter_add_f32(const int32_t *idx, const float *g, const float *w, float *out,
+                         int64_t B, int64_t I, int64_t out_size, int64_t Dv, void *stream);
+
+/*
+ * The two backward operators with half (IEEE binary16) inputs, the rest of the reference's
+ * reduced-precision trio beside lffn_gather_add_f16:
+ *   lffn_indexed_inner_product_f16: g [B, Dv] and src [source_size, Dv] half, out [B, I] fp32: every
+ *     product exact, the sum fp32.  Replaces gather_add.indexed_inner_product_fp16
+ *     (PL/gather/cuda/extension/gather_kernel_fp16.cu:121-184), which rounds each product to half
+ *     (__hmul, :165) before its fp32 sum and the result to half (:181).
+ *   lffn_scatter_add_f16: g [B, Dv] half, w [B, I] fp32, out [out_size, Dv] fp32, ACCUMULATED INTO
+ *     with fp32 atomics.  Replaces gather_add.weighted_vector_scatter_add_fp16 (:64-119), which
+ *     multiplies and accumulates in half (__hmul2 and a half2 atomicAdd, :112-115).
+ * The caller rounds the fp32 results to half where it wants the reference's dtypes; they are the
+ * fp32 sums of the exact products, closer to the exact result than the reference's, not
+ * bit-identical to it.
+ */
+int lffn_indexed_inner_product_f16(const int32_t *idx, const uint16_t *g, const uint16_t *src, float *out,
+                                   int64_t B, int64_t I, int64_t source_size, int64_t Dv, void *stream);
+int lffn_scatter_add_f16(const int32_t *idx, const uint16_t *g, const float *w, float *out,
                          int64_t B, int64_t I, int64_t out_size, int64_t Dv, void *stream);
 
 /*

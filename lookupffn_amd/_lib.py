@@ -15,7 +15,7 @@ _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 # LOOKUPFFN_HIP_LIB points at another build of the same ABI (e.g. a tuning build)
 LIB_PATH = os.environ.get("LOOKUPFFN_HIP_LIB") or os.path.join(_PKG_DIR, "liblookupffn_hip.so")
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 LFFN_OK = 0
 LFFN_ERR_BAD_ARG = -1
@@ -91,6 +91,8 @@ SIGNATURES = {
     "lffn_lookup_gather_plan": [_i64, _i64, _i64, _i64, ctypes.c_int32, ctypes.POINTER(ctypes.c_int32)],
     "lffn_indexed_inner_product_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "lffn_scatter_add_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
+    "lffn_indexed_inner_product_f16": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
+    "lffn_scatter_add_f16": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "lffn_lookup_scatter_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, ctypes.c_int32, _vp],
     "lffn_lookup_scatter_workspace_bytes": [_i64, _i64, _i64, _i64, ctypes.POINTER(ctypes.c_int64)],
     "lffn_lookup_scatter_sorted_f32": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, ctypes.c_int32, _vp],

@@ -62,11 +62,57 @@ __device__ __forceinline__ void axpy_vec(float (&acc)[Row<FMT>::EPV], const uint
     }
 }
 
+// d + <g, r> over one 16-byte vector, element ascending; g has the rows' format
+template <int FMT>
+__device__ __forceinline__ float dot_vec(const uint4 &gq, const uint4 &r, float d) {
+    if constexpr (FMT == LFFN_ROWS_F16) {
+        // (float)half * (float)half + float: one v_fma_mix_f32 per value, the product exact
+        const unsigned a[4] = {gq.x, gq.y, gq.z, gq.w}, b[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const half2_t ha = __builtin_bit_cast(half2_t, a[i]), hb = __builtin_bit_cast(half2_t, b[i]);
+            d = fmaf((float)ha.x, (float)hb.x, d);
+            d = fmaf((float)ha.y, (float)hb.y, d);
+        }
+    } else if constexpr (FMT == LFFN_ROWS_BF16) {
+        d = fmaf(bf16_lo(gq.x), bf16_lo(r.x), d); d = fmaf(bf16_hi(gq.x), bf16_hi(r.x), d);
+        d = fmaf(bf16_lo(gq.y), bf16_lo(r.y), d); d = fmaf(bf16_hi(gq.y), bf16_hi(r.y), d);
+        d = fmaf(bf16_lo(gq.z), bf16_lo(r.z), d); d = fmaf(bf16_hi(gq.z), bf16_hi(r.z), d);
+        d = fmaf(bf16_lo(gq.w), bf16_lo(r.w), d); d = fmaf(bf16_hi(gq.w), bf16_hi(r.w), d);
+    } else {
+        d = fmaf(__uint_as_float(gq.x), __uint_as_float(r.x), d);
+        d = fmaf(__uint_as_float(gq.y), __uint_as_float(r.y), d);
+        d = fmaf(__uint_as_float(gq.z), __uint_as_float(r.z), d);
+        d = fmaf(__uint_as_float(gq.w), __uint_as_float(r.w), d);
+    }
+    return d;
+}
+
+// the EPV values of one 16-byte vector as fp32
+template <int FMT>
+__device__ __forceinline__ void widen_vec(float (&v)[Row<FMT>::EPV], const uint4 &r) {
+    if constexpr (FMT == LFFN_ROWS_F16) {
+        const unsigned q[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const half2_t h = __builtin_bit_cast(half2_t, q[i]);
+            v[2 * i] = (float)h.x;
+            v[2 * i + 1] = (float)h.y;
+        }
+    } else if constexpr (FMT == LFFN_ROWS_BF16) {
+        v[0] = bf16_lo(r.x); v[1] = bf16_hi(r.x); v[2] = bf16_lo(r.y); v[3] = bf16_hi(r.y);
+        v[4] = bf16_lo(r.z); v[5] = bf16_hi(r.z); v[6] = bf16_lo(r.w); v[7] = bf16_hi(r.w);
+    } else {
+        v[0] = __uint_as_float(r.x); v[1] = __uint_as_float(r.y);
+        v[2] = __uint_as_float(r.z); v[3] = __uint_as_float(r.w);
+    }
+}
+
 struct GatherArgs {
     const int32_t *idx;   // [B, I]  (codes when structured)
     const void *src;      // [source_size, Dv]
     const float *w;       // [B, I]
-    const float *g;       // [B, Dv]   (backward kernels)
+    const void *g;        // [B, Dv]   (backward kernels; fp32, or the rows' 16-bit format in the 16-bit forms)
     const float *bias;    // [Dv] or null (structured forward)
     const float *residual;// [B, Dv] or null (structured forward): added to the result
     float *out;
@@ -201,7 +247,8 @@ __device__ __forceinline__ float group_sum(float v) {
 
 // out[b,i] = <g[b,:], src[idx[b,i],:]>.  Column chunks are walked inside the
 // block; the per-chunk partial dot products are summed in LDS in chunk order.
-template <int LPT, int NV>
+// 16-bit forms: g and the rows in the same 16-bit format, products and sums in fp32.
+template <int FMT, int LPT, int NV>
 __global__ __launch_bounds__(256) void inner_product_kernel(GatherArgs a, int chunks) {
     constexpr int TPB = 256 / LPT;
     __shared__ int s_row[TPB][IC];
@@ -211,7 +258,8 @@ __global__ __launch_bounds__(256) void inner_product_kernel(GatherArgs a, int ch
     const int ll = threadIdx.x % LPT;
     const int64_t tok0 = int64_t(blockIdx.x) * TPB;
     const int64_t tok = tok0 + tl;
-    const size_t row_bytes = size_t(a.Dv) * 4;
+    const size_t row_bytes = size_t(a.Dv) * Row<FMT>::ESZ;
+    const char *grow = static_cast<const char *>(a.g) + size_t(tok) * row_bytes;
 
     for (int i0 = 0; i0 < a.I; i0 += IC) {
         __syncthreads();
@@ -221,18 +269,18 @@ __global__ __launch_bounds__(256) void inner_product_kernel(GatherArgs a, int ch
         const int n = min(IC, a.I - i0);
         for (int ch = 0; ch < chunks; ++ch) {
             const int vec0 = ch * (LPT * NV) + ll;
-            float4 gv[NV];
+            uint4 gv[NV];
 #pragma unroll
             for (int v = 0; v < NV; ++v)
-                gv[v] = tok < a.B ? *reinterpret_cast<const float4 *>(a.g + tok * a.Dv + (size_t)(vec0 + v * LPT) * 4)
-                                  : make_float4(0.f, 0.f, 0.f, 0.f);
+                gv[v] = tok < a.B ? *reinterpret_cast<const uint4 *>(grow + (size_t)(vec0 + v * LPT) * 16)
+                                  : make_uint4(0u, 0u, 0u, 0u);
             const char *base = static_cast<const char *>(a.src) + size_t(vec0) * 16;
             int ii = 0;
             for (; ii + 4 <= n; ii += 4) {
-                float4 r[4][NV];
+                uint4 r[4][NV];
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
-                    const float4 *p = reinterpret_cast<const float4 *>(base + size_t(s_row[tl][ii + u]) * row_bytes);
+                    const uint4 *p = reinterpret_cast<const uint4 *>(base + size_t(s_row[tl][ii + u]) * row_bytes);
 #pragma unroll
                     for (int v = 0; v < NV; ++v) r[u][v] = p[v * LPT];
                 }
@@ -240,27 +288,16 @@ __global__ __launch_bounds__(256) void inner_product_kernel(GatherArgs a, int ch
                 for (int u = 0; u < 4; ++u) {
                     float d = 0.f;
 #pragma unroll
-                    for (int v = 0; v < NV; ++v) {
-                        d = fmaf(gv[v].x, r[u][v].x, d);
-                        d = fmaf(gv[v].y, r[u][v].y, d);
-                        d = fmaf(gv[v].z, r[u][v].z, d);
-                        d = fmaf(gv[v].w, r[u][v].w, d);
-                    }
+                    for (int v = 0; v < NV; ++v) d = dot_vec<FMT>(gv[v], r[u][v], d);
                     d = group_sum<LPT>(d);
                     if (ll == 0) s_dot[tl][ii + u] += d;
                 }
             }
             for (; ii < n; ++ii) {
-                const float4 *p = reinterpret_cast<const float4 *>(base + size_t(s_row[tl][ii]) * row_bytes);
+                const uint4 *p = reinterpret_cast<const uint4 *>(base + size_t(s_row[tl][ii]) * row_bytes);
                 float d = 0.f;
 #pragma unroll
-                for (int v = 0; v < NV; ++v) {
-                    const float4 r = p[v * LPT];
-                    d = fmaf(gv[v].x, r.x, d);
-                    d = fmaf(gv[v].y, r.y, d);
-                    d = fmaf(gv[v].z, r.z, d);
-                    d = fmaf(gv[v].w, r.w, d);
-                }
+                for (int v = 0; v < NV; ++v) d = dot_vec<FMT>(gv[v], p[v * LPT], d);
                 d = group_sum<LPT>(d);
                 if (ll == 0) s_dot[tl][ii] += d;
             }
@@ -273,10 +310,12 @@ __global__ __launch_bounds__(256) void inner_product_kernel(GatherArgs a, int ch
     }
 }
 
-// out[idx[b,i],:] += w[b,i] * g[b,:] with hardware fp32 atomics.
-template <int LPT, int NV>
+// out[idx[b,i],:] += w[b,i] * g[b,:] with hardware fp32 atomics.  16-bit forms: g in the
+// 16-bit format, widened once; the products and the sums (out) are fp32.
+template <int FMT, int LPT, int NV>
 __global__ __launch_bounds__(256) void scatter_add_kernel(GatherArgs a) {
     constexpr int TPB = 256 / LPT;
+    constexpr int EPV = Row<FMT>::EPV;
     __shared__ int s_row[TPB][IC];
     __shared__ float s_w[TPB][IC];
 
@@ -286,11 +325,15 @@ __global__ __launch_bounds__(256) void scatter_add_kernel(GatherArgs a) {
     const int64_t tok = tok0 + tl;
     const int vec0 = blockIdx.y * (LPT * NV) + ll;
 
-    float4 gv[NV];
+    float gv[NV][EPV];
 #pragma unroll
-    for (int v = 0; v < NV; ++v)
-        gv[v] = tok < a.B ? *reinterpret_cast<const float4 *>(a.g + tok * a.Dv + (size_t)(vec0 + v * LPT) * 4)
-                          : make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int v = 0; v < NV; ++v) {
+        uint4 q = make_uint4(0u, 0u, 0u, 0u);
+        if (tok < a.B)
+            q = *reinterpret_cast<const uint4 *>(static_cast<const char *>(a.g) + size_t(tok) * a.Dv * Row<FMT>::ESZ +
+                                                 (size_t)(vec0 + v * LPT) * 16);
+        widen_vec<FMT>(gv[v], q);
+    }
 
     for (int i0 = 0; i0 < a.I; i0 += IC) {
         __syncthreads();
@@ -300,14 +343,11 @@ __global__ __launch_bounds__(256) void scatter_add_kernel(GatherArgs a) {
         const int n = min(IC, a.I - i0);
         for (int ii = 0; ii < n; ++ii) {
             const float wt = s_w[tl][ii];
-            float *o = a.out + size_t(s_row[tl][ii]) * a.Dv + size_t(vec0) * 4;
+            float *o = a.out + size_t(s_row[tl][ii]) * a.Dv + size_t(vec0) * EPV;
 #pragma unroll
-            for (int v = 0; v < NV; ++v) {
-                unsafeAtomicAdd(o + v * LPT * 4 + 0, wt * gv[v].x);
-                unsafeAtomicAdd(o + v * LPT * 4 + 1, wt * gv[v].y);
-                unsafeAtomicAdd(o + v * LPT * 4 + 2, wt * gv[v].z);
-                unsafeAtomicAdd(o + v * LPT * 4 + 3, wt * gv[v].w);
-            }
+            for (int v = 0; v < NV; ++v)
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) unsafeAtomicAdd(o + v * LPT * EPV + e, wt * gv[v][e]);
         }
     }
 }
@@ -336,9 +376,9 @@ void launch_one(const GatherArgs &a, const Tiling &t, hipStream_t s) {
     if constexpr (OP == Op::Gather)
         hipLaunchKernelGGL((gather_add_kernel<FMT, LPT, NV>), dim3(gx, t.chunks), dim3(256), 0, s, a);
     else if constexpr (OP == Op::Inner)
-        hipLaunchKernelGGL((inner_product_kernel<LPT, NV>), dim3(gx), dim3(256), 0, s, a, t.chunks);
+        hipLaunchKernelGGL((inner_product_kernel<FMT, LPT, NV>), dim3(gx), dim3(256), 0, s, a, t.chunks);
     else
-        hipLaunchKernelGGL((scatter_add_kernel<LPT, NV>), dim3(gx, t.chunks), dim3(256), 0, s, a);
+        hipLaunchKernelGGL((scatter_add_kernel<FMT, LPT, NV>), dim3(gx, t.chunks), dim3(256), 0, s, a);
 }
 
 template <int FMT, Op OP, int LPT>
@@ -461,6 +501,31 @@ extern "C" int lffn_scatter_add_f32(const int32_t *idx, const float *g, const fl
     a.idx = idx; a.src = nullptr; a.w = w; a.g = g; a.bias = nullptr; a.out = out;
     a.B = B; a.I = (int)I; a.source_size = out_size; a.Dv = (int)Dv; a.S = 0;
     return launch<LFFN_ROWS_F32, Op::Scatter>(a, static_cast<hipStream_t>(stream));
+}
+
+// The reduced-precision calls of the backward: g and the rows are half, the results fp32.
+extern "C" int lffn_indexed_inner_product_f16(const int32_t *idx, const uint16_t *g, const uint16_t *src, float *out,
+                                              int64_t B, int64_t I, int64_t source_size, int64_t Dv, void *stream) {
+    int rc = check_common(idx, B, I, source_size, Dv);
+    if (rc != LFFN_OK) return rc;
+    LFFN_REQUIRE(g && src && (out || B * I == 0), LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_aligned16(src) && lffn_aligned16(g), LFFN_ERR_BAD_ARG);
+    GatherArgs a{};
+    a.idx = idx; a.src = src; a.w = nullptr; a.g = g; a.bias = nullptr; a.out = out;
+    a.B = B; a.I = (int)I; a.source_size = source_size; a.Dv = (int)Dv; a.S = 0;
+    return launch<LFFN_ROWS_F16, Op::Inner>(a, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int lffn_scatter_add_f16(const int32_t *idx, const uint16_t *g, const float *w, float *out,
+                                    int64_t B, int64_t I, int64_t out_size, int64_t Dv, void *stream) {
+    int rc = check_common(idx, B, I, out_size, Dv);
+    if (rc != LFFN_OK) return rc;
+    LFFN_REQUIRE(g && out && (w || B * I == 0), LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_aligned16(g) && lffn_aligned16(out), LFFN_ERR_BAD_ARG);
+    GatherArgs a{};
+    a.idx = idx; a.src = nullptr; a.w = w; a.g = g; a.bias = nullptr; a.out = out;
+    a.B = B; a.I = (int)I; a.source_size = out_size; a.Dv = (int)Dv; a.S = 0;
+    return launch<LFFN_ROWS_F16, Op::Scatter>(a, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int lffn_version(void) { return LFFN_ABI_VERSION; }

@@ -1,7 +1,8 @@
 """Weighted gather-add operators: the reference's ``gather`` /
 ``weighted_gather_add`` surface (PL/gather/kernel.py, PL/gather/cuda/kernel.py) on the
-gfx950 kernels.  Rows may be float32, bfloat16 or float16; weights, accumulation and
-outputs are float32."""
+gfx950 kernels.  Rows may be float32, bfloat16 or float16; accumulation is float32.  The
+reference's half-precision calls (every tensor half) are taken as well, forward and backward:
+their sums are formed in float32 and rounded to half once."""
 from __future__ import annotations
 
 import math
@@ -62,7 +63,9 @@ def weighted_vector_gather_add(indexes, source, weights, use_torch=False):
 def indexed_inner_product(indexes, source_1, source_2, use_torch=False):
     """outputs[b,i] = <source_1[b], source_2[indexes[b,i]]>   (PL/gather/cuda/kernel.py:72-122)."""
     _check(indexes, source_1, source_2, "inner")
-    assert source_1.dtype == torch.float32 and source_2.dtype == torch.float32
+    assert source_2.dtype in [torch.float32, torch.float16], source_2.dtype
+    assert source_1.dtype == source_2.dtype, (source_1.dtype, source_2.dtype)
+    half_call = source_2.dtype == torch.float16       # PL/gather/cuda/kernel.py:113-116: half in, half out
     batch_size, index_size = indexes.shape
     source_size, vector_dim = source_2.shape
     assert source_1.shape[0] == batch_size and source_1.shape[1] == vector_dim
@@ -76,13 +79,16 @@ def indexed_inner_product(indexes, source_1, source_2, use_torch=False):
             rows = source_2[indexes[batch_idx, :], :].reshape(index_size, vector_dim)
             out.append((source_1[batch_idx, None, :] * rows).sum(dim=-1))
         return torch.stack(out, dim=0)
-    return ops.indexed_inner_product(indexes, source_1, source_2)
+    out = ops.indexed_inner_product(indexes, source_1, source_2)      # fp32 sums of exact products
+    return out.half() if half_call else out
 
 
 def weighted_vector_scatter_add(indexes, source, weights, output_size, use_torch=False):
     """outputs[indexes[b,i]] += weights[b,i] * source[b]   (PL/gather/cuda/kernel.py:124-173)."""
     _check(indexes, source, weights, "scatter")
-    assert source.dtype == torch.float32 and weights.dtype == torch.float32
+    assert source.dtype in [torch.float32, torch.float16], source.dtype
+    assert weights.dtype == source.dtype, (source.dtype, weights.dtype)
+    half_call = source.dtype == torch.float16         # PL/gather/cuda/kernel.py:164-167: half in, half out
     batch_size, index_size = indexes.shape
     _, vector_dim = source.shape
     assert weights.shape[0] == batch_size and weights.shape[1] == index_size
@@ -98,6 +104,9 @@ def weighted_vector_scatter_add(indexes, source, weights, output_size, use_torch
             inst_indexes = indexes[batch_idx, :, None].repeat(1, vector_dim).reshape(index_size, -1)
             outputs.scatter_add_(0, inst_indexes, inst_source)
         return outputs
+    if half_call:
+        # fp32 products and sums (the reference multiplies and accumulates in half), one rounding at the end
+        return ops.scatter_add(indexes, source, weights.float(), output_size).half()
     return ops.scatter_add(indexes, source, weights, output_size)
 
 
@@ -114,8 +123,11 @@ class WeightedVectorGatherAdd(Function):
     def backward(ctx, grad_outputs):
         grad_outputs = grad_outputs.contiguous()
         indexes, source, weights = ctx.saved_tensors
-        if source.dtype != torch.float32:
-            raise NotImplementedError("backward through 16-bit rows is not built (inference formats)")
+        if source.dtype != weights.dtype or source.dtype == torch.bfloat16:
+            # 16-bit rows under fp32 weights are inference formats; the reference's half call (rows, weights
+            # and gradients all half, PL/gather/cuda/kernel.py:64-67,113-116,164-167) has its backward below
+            raise NotImplementedError("backward through 16-bit rows with fp32 weights is not built (inference formats)")
+        grad_outputs = grad_outputs.to(source.dtype)
         grad_weights = indexed_inner_product(indexes, grad_outputs, source)
         grad_source = weighted_vector_scatter_add(indexes, grad_outputs, weights, source.shape[0])
         return None, grad_source, grad_weights

@@ -965,20 +965,25 @@ _L.define("indexed_inner_product(Tensor indexes, Tensor source_1, Tensor source_
 
 
 def _inner_impl(indexes, source_1, source_2):
+    """fp32 inputs, or both half (the reference's reduced-precision call): the result is fp32 either way."""
     _lib.require_gpu(indexes, source_1, source_2)
     assert source_1.dim() == 2 and source_2.dim() == 2
-    assert source_1.dtype == torch.float32 and source_2.dtype == torch.float32
+    assert source_1.dtype == source_2.dtype and source_2.dtype in (torch.float32, torch.float16), \
+        (source_1.dtype, source_2.dtype)
     assert source_1.is_contiguous() and source_2.is_contiguous()
     B, I = indexes.shape
     S, Dv = source_2.shape
     assert source_1.shape[0] == B and source_1.shape[1] == Dv
     _check_gather_args(indexes, S, Dv)
     out = torch.empty(B, I, dtype=torch.float32, device=source_2.device)
+    lib = _lib.load()
+    fn, name = ((lib.lffn_indexed_inner_product_f16, "lffn_indexed_inner_product_f16")
+                if source_2.dtype == torch.float16 else
+                (lib.lffn_indexed_inner_product_f32, "lffn_indexed_inner_product_f32"))
     with _dev_guard(source_2):
-        rc = _lib.load().lffn_indexed_inner_product_f32(
-            _lib.ptr(indexes), _lib.ptr(source_1), _lib.ptr(source_2), _lib.ptr(out), B, I, S, Dv,
-            _lib.stream_of(source_2))
-    _lib.check(rc, f"lffn_indexed_inner_product_f32(B={B}, I={I}, S={S}, Dv={Dv})")
+        rc = fn(_lib.ptr(indexes), _lib.ptr(source_1), _lib.ptr(source_2), _lib.ptr(out), B, I, S, Dv,
+                _lib.stream_of(source_2))
+    _lib.check(rc, f"{name}(B={B}, I={I}, S={S}, Dv={Dv})")
     return out
 
 
@@ -987,15 +992,16 @@ _L.impl("indexed_inner_product", _inner_impl, "CUDA")
 
 @torch.library.register_fake("lookupffn::indexed_inner_product")
 def _(indexes, source_1, source_2):
-    return source_1.new_empty(indexes.shape)
+    return source_1.new_empty(indexes.shape, dtype=torch.float32)
 
 
 _L.define("scatter_add(Tensor indexes, Tensor source, Tensor weights, int output_size) -> Tensor")
 
 
 def _scatter_impl(indexes, source, weights, output_size):
+    """source fp32 or half (the reference's reduced-precision call); weights and the result fp32."""
     _lib.require_gpu(indexes, source, weights)
-    assert source.dim() == 2 and source.dtype == torch.float32 and source.is_contiguous()
+    assert source.dim() == 2 and source.dtype in (torch.float32, torch.float16) and source.is_contiguous()
     assert weights.dtype == torch.float32 and weights.is_contiguous()
     assert tuple(weights.shape) == tuple(indexes.shape)
     B, I = indexes.shape
@@ -1003,11 +1009,13 @@ def _scatter_impl(indexes, source, weights, output_size):
     assert source.shape[0] == B
     _check_gather_args(indexes, output_size, Dv)
     out = torch.zeros(output_size, Dv, dtype=torch.float32, device=source.device)
+    lib = _lib.load()
+    fn, name = ((lib.lffn_scatter_add_f16, "lffn_scatter_add_f16") if source.dtype == torch.float16 else
+                (lib.lffn_scatter_add_f32, "lffn_scatter_add_f32"))
     with _dev_guard(source):
-        rc = _lib.load().lffn_scatter_add_f32(
-            _lib.ptr(indexes), _lib.ptr(source), _lib.ptr(weights), _lib.ptr(out), B, I, output_size, Dv,
-            _lib.stream_of(source))
-    _lib.check(rc, f"lffn_scatter_add_f32(B={B}, I={I}, out={output_size}, Dv={Dv})")
+        rc = fn(_lib.ptr(indexes), _lib.ptr(source), _lib.ptr(weights), _lib.ptr(out), B, I, output_size, Dv,
+                _lib.stream_of(source))
+    _lib.check(rc, f"{name}(B={B}, I={I}, out={output_size}, Dv={Dv})")
     return out
 
 
@@ -1016,7 +1024,7 @@ _L.impl("scatter_add", _scatter_impl, "CUDA")
 
 @torch.library.register_fake("lookupffn::scatter_add")
 def _(indexes, source, weights, output_size):
-    return source.new_empty(output_size, source.shape[1])
+    return source.new_empty(output_size, source.shape[1], dtype=torch.float32)
 
 
 # Below this many multiply-adds (B * T * Do) the LDS-accumulating scatter is the faster one

@@ -427,7 +427,10 @@ def indexed_inner_product(idx, g, src):
     B, I = idx.shape
     S, Dv = src.shape
     out = torch.full((B, I), float("nan"), dtype=torch.float32, device=DEV)
-    _call("lffn_indexed_inner_product_f32", p(idd), p(gd), p(sd), p(out), B, I, S, Dv)
+    half = src.dtype == np.uint16              # half bit patterns for g and src: the reduced-precision call
+    assert (g.dtype == np.uint16) == half
+    _call("lffn_indexed_inner_product_f16" if half else "lffn_indexed_inner_product_f32",
+          p(idd), p(gd), p(sd), p(out), B, I, S, Dv)
     return host(out)
 
 
@@ -436,7 +439,8 @@ def scatter_add(idx, g, w, out_size, init=None):
     B, I = idx.shape
     Dv = g.shape[1]
     out = torch.zeros(out_size, Dv, dtype=torch.float32, device=DEV) if init is None else dev(init)
-    _call("lffn_scatter_add_f32", p(idd), p(gd), p(wd), p(out), B, I, out_size, Dv)
+    _call("lffn_scatter_add_f16" if g.dtype == np.uint16 else "lffn_scatter_add_f32",     # uint16: half bit patterns
+          p(idd), p(gd), p(wd), p(out), B, I, out_size, Dv)
     return host(out)
 
 

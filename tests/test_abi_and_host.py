@@ -45,6 +45,11 @@ def test_argument_validation_needs_no_gpu():
     # null pointers
     assert lib.lffn_fht_f32(None, None, 4, 8, None) == _lib.LFFN_ERR_BAD_ARG
     assert lib.lffn_gather_add_f32(None, None, None, None, 4, 2, 8, 64, None) == _lib.LFFN_ERR_BAD_ARG
+    assert lib.lffn_indexed_inner_product_f16(256, None, 256, 256, 4, 2, 8, 64, None) == _lib.LFFN_ERR_BAD_ARG
+    assert lib.lffn_scatter_add_f16(256, 256, 256, None, 4, 2, 8, 64, None) == _lib.LFFN_ERR_BAD_ARG
+    assert lib.lffn_indexed_inner_product_f16(256, 256, 256, 256, 4, 2, 8, 96, None) == _lib.LFFN_ERR_UNSUPPORTED  # Dv % 64
+    assert lib.lffn_scatter_add_f16(256, 258, 256, 256, 4, 2, 8, 64, None) == _lib.LFFN_ERR_BAD_ARG          # misaligned g
+    assert lib.lffn_scatter_add_f16(None, None, None, None, 0, 2, 8, 64, None) == _lib.LFFN_ERR_BAD_ARG      # null g, out
     # unsupported shapes (pointers are never dereferenced on the host)
     assert lib.lffn_fht_f32(256, 256, 4, 2048, None) == _lib.LFFN_ERR_UNSUPPORTED
     assert lib.lffn_fht_f32(256, 256, 4, 48, None) == _lib.LFFN_ERR_UNSUPPORTED      # not a power of two

@@ -307,6 +307,37 @@ def test_f16_tables_inference_and_general_gather():
     assert got16.dtype == torch.float16 and relmax(npf(got16), want16) <= 2 ** -10
 
 
+def test_half_precision_call_trains_through_weighted_gather_add():
+    """The reference's half-precision call with gradients (PL/gather/cuda/kernel.py:175-202 with half tensors,
+    kernels gather_kernel_fp16.cu:6-184): rows, weights and the incoming gradient half; the gradients come back
+    half, rounded once from fp32 sums.  Checked against the float64 oracle on the same half values."""
+    rng = np.random.RandomState(12)
+    rows, Dv, B, I = 300, 192, 77, 6
+    src = torch.tensor((0.1 * rng.randn(rows, Dv)).astype(np.float16), device=DEV, requires_grad=True)
+    w = torch.tensor((1 - rng.rand(B, I)).astype(np.float16), device=DEV, requires_grad=True)
+    idx_np = rng.randint(0, rows, size=(B, I)).astype(np.int32)
+    idx = torch.tensor(idx_np, device=DEV)
+    out = lookupffn_amd.weighted_gather_add(idx, src, w)
+    assert out.dtype == torch.float16
+    g = torch.tensor(rng.randn(B, Dv).astype(np.float16), device=DEV)
+    out.backward(g)
+    assert src.grad.dtype == torch.float16 and w.grad.dtype == torch.float16
+    f64 = lambda t: npf(t.detach().float()).astype(np.float64)
+    want_w = oracle.indexed_inner_product(idx_np, f64(g), f64(src))
+    want_s = oracle.scatter_add(idx_np, f64(g), f64(w), rows)
+    assert relmax(f64(w.grad), want_w) <= 2 ** -10            # one rounding to half
+    assert relmax(f64(src.grad), want_s) <= 2 ** -10
+    # the operators on their own take the half call as well, and return half
+    gw = lookupffn_amd.indexed_inner_product(idx, g, src.detach())
+    gs = lookupffn_amd.weighted_vector_scatter_add(idx, g, w.detach(), rows)
+    assert gw.dtype == torch.float16 and torch.equal(gw, w.grad)
+    assert gs.dtype == torch.float16 and relmax(f64(gs), want_s) <= 2 ** -10
+    # half rows under fp32 weights stay an inference format
+    w32 = w.detach().float().requires_grad_(True)
+    with pytest.raises(NotImplementedError):
+        lookupffn_amd.weighted_gather_add(idx, src, w32).sum().backward()
+
+
 def test_reference_call_sequence_of_lookup_gather():
     # LookupFFN.gather keeps the reference's flat-index form (PL/lookup.py:120-130)
     torch.manual_seed(7)

@@ -1266,6 +1266,37 @@ def test_backward_matches_oracle(B, T, S, Do):
     assert relmax(cabi.scatter_add(idx, g, w, T * S, init=init), want_t + init) <= 1e-5
 
 
+@pytest.mark.parametrize("B,T,S,Do", [(256, 32, 256, 256), (5, 6, 16, 128), (67, 10, 8, 192), (33, 130, 4, 768),
+                                      (9, 4, 8, 320), (3, 2, 2, 1920), (19, 64, 256, 1024), (70, 2, 4, 64)])
+def test_backward_half_inputs_match_oracle(B, T, S, Do):
+    """The reduced-precision calls of the backward (gradient rows and table rows in half, the place of
+    gather_kernel_fp16.cu:64-184): every product is exact and the sums are fp32, so the results sit within
+    1e-5 of the float64 oracle on the same half values (the reference rounds products and sums to half:
+    bit parity with it is not defined, its atomics run in no fixed order)."""
+    rng = np.random.RandomState(B + T + Do + 5)
+    tables, code, idx, w = _rand_gather(rng, B, T, S, Do)
+    flat_h = tables.reshape(T * S, Do).astype(np.float16)
+    g_h = rng.randn(B, Do).astype(np.float16)
+    want_w = oracle.indexed_inner_product(idx, g_h.astype(np.float64), flat_h.astype(np.float64))
+    got_w = cabi.indexed_inner_product(idx, g_h.view(np.uint16), flat_h.view(np.uint16))
+    assert relmax(got_w, want_w) <= 1e-5
+    # the same numbers through the fp32 kernel: the two differ by fp32 summation order at most
+    assert relmax(got_w, cabi.indexed_inner_product(idx, g_h.astype(np.float32), flat_h.astype(np.float32))) <= 2e-6
+    want_t = oracle.scatter_add(idx, g_h.astype(np.float64), w.astype(np.float64), T * S)
+    got_t = cabi.scatter_add(idx, g_h.view(np.uint16), w, T * S)
+    assert relmax(got_t, want_t) <= 1e-5
+    init = rng.randn(T * S, Do).astype(np.float32)
+    assert relmax(cabi.scatter_add(idx, g_h.view(np.uint16), w, T * S, init=init), want_t + init) <= 1e-5
+    # small integers: products and sums are exact in fp32 whatever the order, so equality is exact
+    gi = rng.randint(-4, 5, size=(B, Do)).astype(np.float16)
+    ri = rng.randint(-4, 5, size=(T * S, Do)).astype(np.float16)
+    wi = rng.randint(-3, 4, size=(B, T)).astype(np.float32)
+    assert np.array_equal(cabi.indexed_inner_product(idx, gi.view(np.uint16), ri.view(np.uint16)),
+                          oracle.indexed_inner_product(idx, gi.astype(np.float64), ri.astype(np.float64)))
+    assert np.array_equal(cabi.scatter_add(idx, gi.view(np.uint16), wi, T * S),
+                          oracle.scatter_add(idx, gi.astype(np.float64), wi.astype(np.float64), T * S))
+
+
 # (B, T, S, Do): odd table counts, tables smaller than the LDS
 # slice, ragged token counts around the 64-token batches and 1024-token strides, and a
 # table size (512) that takes the zero-fill + global-atomics path
