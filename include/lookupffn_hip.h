@@ -358,23 +358,26 @@ int lffn_ln_project_hash_f32(const float *x, const float *ln_weight, const float
  * (fp32 rows, S = 256, an even number of tables, enough tokens: the conditions under which
  * lffn_lookup_gather_workspace_bytes asks for a record stream, without the cost of the packing kernel)
  * it sets *tokens_per_workgroup (a multiple of 16 up to 2048: the tokens are spread evenly over the
- * workgroups of a slice), *record_stride (words per plane: the token slots of all tiles, fewer than
- * B + 2048) and *bytes (the size of the stream: 6 * T * record_stride); otherwise all three are 0 and
- * the caller uses the other entry points.
+ * workgroups of a slice), *record_stride (12-byte record slots per table pair: whole workgroups' worth,
+ * a multiple of 16, fewer than B + 2048) and *bytes (the size of the stream: 6 * T * record_stride);
+ * otherwise all three are 0 and the caller uses the other entry points.
  *
  * lffn_ln_project_hash_records_f32: lffn_ln_project_hash_f32 (ln_weight and ln_bias both NULL: no
- * LayerNorm, as lffn_project_hash_f32) with its codes and scores written as records: 4-byte aligned
- * device memory of `bytes`, three planes of record_stride words per table pair k:
+ * LayerNorm, as lffn_project_hash_f32) with its codes and scores written as records for a gather of
+ * tokens_per_workgroup tokens per workgroup (the plan's): 16-byte aligned device memory of `bytes`,
+ * record_stride records of three words per table pair k:
  *   word 0: score of the pair's first table, word 1: score of its second, word 2: row of the first |
  *   row of the second << 8, where token b takes the tables in the order (2k, 2k+1) when bit 1 of b is
- *   clear and (2k+1, 2k) when it is set (the order its lanes read them in the gather kernel).
- * Words of tokens from B up to record_stride are left as they are: the gather ignores them.  T even,
- * D >= 16.  The layout is private to these entry points: write it with this call only.
+ *   clear and (2k+1, 2k) when it is set (the order its lanes read them in the gather kernel);
+ *   a pair's records are kept in the order the gather's wavefronts copy them, which depends on
+ *   tokens_per_workgroup: writer and reader must be given the same value.
+ * Records of tokens from B up to record_stride are left as they are: the gather ignores them.  T even,
+ * D >= 16.  The layout is private to these entry points: write it with these calls only.
  *
  * lffn_lookup_gather_records_f32: out[b,:] = residual[b,:] + bias + sum_t score[b,t] * tables[t, code[b,t], :]
- * from such a stream, with the tokens_per_workgroup the plan gave and a record_stride of at least the
- * plan's.  Results are bit-identical to lffn_lookup_gather_ws_f32's for the same shape.  bias and
- * residual may be NULL.
+ * from such a stream, with the tokens_per_workgroup it was written for and a record_stride of at least the
+ * plan's (a multiple of 4).  Results are bit-identical to lffn_lookup_gather_ws_f32's for the same shape.
+ * bias and residual may be NULL.
  *
  * lffn_lookup_gather_records_plan_rows / lffn_lookup_gather_records_rows: the same two calls for any
  * row format (row_format 0 fp32, 1 bfloat16, 2 half; tables typed accordingly).  16-bit rows run 1024
@@ -388,14 +391,15 @@ int lffn_lookup_gather_records_plan(int64_t B, int64_t T, int64_t S, int64_t Do,
                                     int64_t *record_stride, int64_t *bytes);
 int lffn_ln_project_hash_records_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
                                      const float *diag, const float *proj_bias, uint32_t *records,
-                                     int64_t record_stride, int64_t B, int64_t H, int64_t D, int64_t R,
-                                     int64_t J, int64_t T, float decay, float residual, void *stream);
+                                     int64_t record_stride, int32_t tokens_per_workgroup, int64_t B, int64_t H,
+                                     int64_t D, int64_t R, int64_t J, int64_t T, float decay, float residual,
+                                     void *stream);
 /* lffn_ln_bh4_block_hash_f32 (below) with its codes and scores written as records in the same way. */
 int lffn_ln_bh4_block_hash_records_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
                                        const float *w_folded, const float *proj_bias, uint32_t *records,
-                                       int64_t record_stride, int64_t B, int64_t H, int64_t D, int64_t R,
-                                       int64_t J, int64_t T, int64_t block_size, float decay, float residual,
-                                       void *stream);
+                                       int64_t record_stride, int32_t tokens_per_workgroup, int64_t B, int64_t H,
+                                       int64_t D, int64_t R, int64_t J, int64_t T, int64_t block_size, float decay,
+                                       float residual, void *stream);
 int lffn_lookup_gather_records_f32(const uint32_t *records, int64_t record_stride, const float *tables,
                                    const float *bias, const float *residual, float *out, int64_t B, int64_t T,
                                    int64_t S, int64_t Do, int32_t tokens_per_workgroup, void *stream);

@@ -26,6 +26,7 @@ LFFN_ERR_SCRATCH = -4
 _vp = ctypes.c_void_p
 _i64 = ctypes.c_int64
 _f32 = ctypes.c_float
+_i32 = ctypes.c_int32
 
 # name -> argument types (every entry point returns int except the two below)
 SIGNATURES = {
@@ -81,8 +82,8 @@ SIGNATURES = {
     "lffn_lookup_gather_ws_planned_rows": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, ctypes.c_int32,
                                            ctypes.c_int32, ctypes.c_int32, _vp],
     "lffn_lookup_gather_ws_planned_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, ctypes.c_int32, ctypes.c_int32, _vp],
-    "lffn_ln_project_hash_records_f32": [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _vp],
-    "lffn_ln_bh4_block_hash_records_f32": [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _vp],
+    "lffn_ln_project_hash_records_f32": [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _i64, _i32, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _vp],
+    "lffn_ln_bh4_block_hash_records_f32": [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _i64, _i32, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _vp],
     "lffn_lookup_gather_records_plan": [_i64, _i64, _i64, _i64, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64)],
     "lffn_lookup_gather_records_f32": [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, ctypes.c_int32, _vp],
     "lffn_lookup_gather_records_plan_rows": [_i64, _i64, _i64, _i64, ctypes.c_int32, ctypes.POINTER(ctypes.c_int32),

@@ -102,7 +102,8 @@ struct BlockArgs {
     int32_t *codes;        // [B, T]              (hash form)
     float *scores;         // [B, T]              (hash form)
     uint32_t *records;     // hash form, instead of codes and scores: the record stream of the
-    int64_t rec_stride;    // four-lanes-per-token gather, [T/2][3][rec_stride] (see lookup_gather_quad.hip)
+    int64_t rec_stride;    // four-lanes-per-token gather, [T/2][rec_stride][3] (lffn_quad_record_slot)
+    int rec_tile;          // tokens per workgroup of the gather the records are written for
     float *z_out;          // [B, T*8] or null    (hash form: z kept for the backward)
     float *row_stats;      // [B, 2] or null: LayerNorm's mean and 1/sigma of every row, kept for the backward
     float *stage_save;     // forward: [R, J-1, B, D] inputs of stages 1..J-1, or null;
@@ -560,21 +561,23 @@ __global__ __launch_bounds__(256 * HV / NH, HV == 1 ? 2 : 1) void bh4_block_kern
                 }
                 __syncthreads();
                 if (a.records) {
-                    // records: per table pair three words per token, the workgroup's TOK tokens side by
-                    // side in each plane (whole 128-byte lines for 32 tokens); a token whose index has bit
-                    // 1 set takes the pair's tables in the order (2k+1, 2k)
-                    for (int item = tid; item < TOK * (D / 16); item += 64 * NWAVE) {
-                        const int row = item % TOK, kk = item / TOK;
-                        const int64_t tok = tok_base + row;
+                    // records: per table pair three words per token, the workgroup's TOK tokens (whole
+                    // groups of 16: 192 contiguous bytes each) side by side; a token whose index has bit 1
+                    // set takes the pair's tables in the order (2k+1, 2k)
+                    static_assert((64 * NWAVE) % TOK == 0, "a thread stays on one token");
+                    const int row = tid % TOK;
+                    const int64_t tok = tok_base + row;
+                    const int64_t slot = tok < B ? lffn_quad_record_slot(tok, a.rec_tile) : 0;
+                    for (int kk = tid / TOK; kk < D / 16; kk += 64 * NWAVE / TOK) {
                         const int pair = r * (D / 16) + kk;
                         if (tok < B && 2 * pair + 1 < a.T) {
                             const int ca = cs[row * CROW + 2 * kk], cb = cs[row * CROW + 2 * kk + 1];
                             const float sa = ss[row * CROW + 2 * kk], sb = ss[row * CROW + 2 * kk + 1];
                             const bool second_first = (tok & 2) != 0;
-                            uint32_t *dst = a.records + (size_t)pair * 3 * a.rec_stride + tok;
+                            uint32_t *dst = a.records + ((size_t)pair * a.rec_stride + slot) * LFFN_RECORD_WORDS;
                             dst[0] = __float_as_uint(second_first ? sb : sa);
-                            dst[a.rec_stride] = __float_as_uint(second_first ? sa : sb);
-                            dst[2 * a.rec_stride] = second_first ? (unsigned)(cb | (ca << 8)) : (unsigned)(ca | (cb << 8));
+                            dst[1] = __float_as_uint(second_first ? sa : sb);
+                            dst[2] = second_first ? (unsigned)(cb | (ca << 8)) : (unsigned)(ca | (cb << 8));
                         }
                     }
                 } else {
@@ -710,14 +713,15 @@ extern "C" int lffn_ln_bh4_block_hash_f32(const float *x, const float *ln_weight
 
 extern "C" int lffn_ln_bh4_block_hash_records_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
                                                   const float *w_folded, const float *proj_bias, uint32_t *records,
-                                                  int64_t record_stride, int64_t B, int64_t H, int64_t D, int64_t R,
-                                                  int64_t J, int64_t T, int64_t block_size, float decay, float residual,
-                                                  void *stream) {
+                                                  int64_t record_stride, int32_t tokens_per_workgroup, int64_t B,
+                                                  int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
+                                                  int64_t block_size, float decay, float residual, void *stream) {
     LFFN_REQUIRE(B >= 0 && R >= 1 && J >= 1 && D >= 1 && H >= 1 && H <= D && T >= 0, LFFN_ERR_BAD_ARG);
     LFFN_REQUIRE(H % 4 == 0 && J <= 64, LFFN_ERR_UNSUPPORTED);
     LFFN_REQUIRE(block_size == BS && lffn_is_pow2(D) && D >= BS && D <= 1024, LFFN_ERR_UNSUPPORTED);
     LFFN_REQUIRE(R <= 4096 && B <= (int64_t(1) << 31) - 1 && T <= (1 << 24), LFFN_ERR_UNSUPPORTED);
-    LFFN_REQUIRE(T * 8 <= R * D && T % 2 == 0 && record_stride >= B, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(T * 8 <= R * D && T % 2 == 0 && lffn_record_layout_ok(B, record_stride, tokens_per_workgroup),
+                 LFFN_ERR_BAD_ARG);
     LFFN_REQUIRE(!ln_weight || (ln_bias && ln_eps >= 0.f), LFFN_ERR_BAD_ARG);
     if (B == 0 || T == 0) return LFFN_OK;
     LFFN_REQUIRE(x && w_folded && records, LFFN_ERR_BAD_ARG);
@@ -726,7 +730,7 @@ extern "C" int lffn_ln_bh4_block_hash_records_f32(const float *x, const float *l
                  LFFN_ERR_BAD_ARG);
     BlockArgs a{};
     a.x = x; a.ln_w = ln_weight; a.ln_b = ln_bias; a.ln_eps = ln_eps; a.wf = w_folded; a.pbias = proj_bias;
-    a.records = records; a.rec_stride = record_stride; a.B = B; a.H = (int)H; a.R = (int)R; a.J = (int)J; a.T = (int)T;
+    a.records = records; a.rec_stride = record_stride; a.rec_tile = tokens_per_workgroup; a.B = B; a.H = (int)H; a.R = (int)R; a.J = (int)J; a.T = (int)T;
     a.decay = decay; a.residual = residual;
     return dispatch_block<true>(a, D, static_cast<hipStream_t>(stream));
 }

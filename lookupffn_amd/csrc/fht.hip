@@ -239,11 +239,13 @@ struct ProjectArgs {
     int32_t *codes;       // [B, T] (HASH only)
     float *scores;        // [B, T] (HASH only)
     // HASH only, instead of codes and scores: the record stream of the four-lanes-per-token gather
-    // (lookup_gather_quad.hip), three planes of rec_stride words per table pair: score of the pair's first
+    // (lookup_gather_quad.hip), rec_stride records of three words per table pair: score of the pair's first
     // table, score of its second, row of the first | row of the second << 8, where a token whose index has
-    // bit 1 set takes the pair's tables in the order (2k+1, 2k).  T even, 8-bit codes.
-    uint32_t *records;    // [T/2][3][rec_stride] or null
-    int64_t rec_stride;   // >= B
+    // bit 1 set takes the pair's tables in the order (2k+1, 2k); a token's slot: lffn_quad_record_slot.
+    // T even, 8-bit codes.
+    uint32_t *records;    // [T/2][rec_stride][3] or null
+    int64_t rec_stride;   // record slots per table pair: whole tiles of rec_tile tokens
+    int rec_tile;         // tokens per workgroup of the gather the records are written for
     int blocks_per_xcd;   // records: workgroup b takes rows from the range of XCD b % 8 (see project_kernel)
     int64_t B;
     int H;                // valid input columns (<= D)
@@ -353,14 +355,18 @@ __global__ __launch_bounds__(256) void project_kernel(ProjectArgs a) {
     const int lr = lane % LPR;
     // GATHER: one token per workgroup; its four wavefronts each compute the token's codes (no
     // hand-over needed) and then share the gather, a quarter of the tables each
-    // Records are written a word at a time into planes indexed by token: a 128-byte line holds 32
-    // consecutive tokens' words, and consecutive workgroups run on different XCDs, whose L2s would each
-    // write back a sliver of every line.  So with records every XCD takes a contiguous range of rows
-    // (workgroup b runs on XCD b % 8 and is that XCD's workgroup number b / 8).
+    // Records are written 12 bytes at a time, a token's slot next to its neighbours': a 128-byte line holds
+    // about ten consecutive tokens' records of a table pair, and consecutive workgroups run on different
+    // XCDs, whose L2s would each write back a sliver of every line.  So with records every XCD takes a
+    // contiguous range of rows (workgroup b runs on XCD b % 8 and is that XCD's workgroup number b / 8).
     const int64_t blk = (HASH && !GATHER && a.records)
                             ? int64_t(blockIdx.x % 8) * a.blocks_per_xcd + blockIdx.x / 8 : int64_t(blockIdx.x);
     const int64_t row = GATHER ? int64_t(blockIdx.x) : (blk * 4 + wave) * RPW + lane / LPR;
     const bool live = row < a.B;
+    int64_t rec_slot = 0;                  // where this row's records go within a table pair's
+    if constexpr (HASH && !GATHER) {
+        if (a.records && live) rec_slot = lffn_quad_record_slot(row, a.rec_tile);
+    }
 
     float orig[NJ][4];
 #pragma unroll
@@ -528,11 +534,11 @@ __global__ __launch_bounds__(256) void project_kernel(ProjectArgs a) {
                         __builtin_amdgcn_update_dpp(0, __float_as_int(score_here), 0x55, 0xF, 0xF, true));
                     if (live && (lr & 3) == 3 && t < a.T) {
                         const bool second_first = (row & 2) != 0;
-                        uint32_t *dst = a.records + (size_t)(t >> 1) * 3 * a.rec_stride + row;
+                        uint32_t *dst = a.records + ((size_t)(t >> 1) * a.rec_stride + rec_slot) * LFFN_RECORD_WORDS;
                         dst[0] = __float_as_uint(second_first ? score_here : score_even);
-                        dst[a.rec_stride] = __float_as_uint(second_first ? score_even : score_here);
-                        dst[2 * a.rec_stride] = second_first ? (unsigned)(code_here | (code_even << 8))
-                                                             : (unsigned)(code_even | (code_here << 8));
+                        dst[1] = __float_as_uint(second_first ? score_even : score_here);
+                        dst[2] = second_first ? (unsigned)(code_here | (code_even << 8))
+                                              : (unsigned)(code_even | (code_here << 8));
                     }
                 } else if (live && (lr & 1) && t < a.T) {
                     a.codes[row * a.T + t] = (nib_hi << 4) | nib;
@@ -916,7 +922,7 @@ static int project_hash_impl(const float *x, const float *ln_w, const float *ln_
                              float *z_out, int32_t *codes, float *scores,
                              int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
                              float decay, float residual, void *stream, uint32_t *records = nullptr,
-                             int64_t record_stride = 0);
+                             int64_t record_stride = 0, int record_tile = 0);
 
 extern "C" int lffn_ln_project_hash_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
                                         const float *diag, const float *proj_bias,
@@ -930,13 +936,16 @@ extern "C" int lffn_ln_project_hash_f32(const float *x, const float *ln_weight, 
 
 extern "C" int lffn_ln_project_hash_records_f32(const float *x, const float *ln_weight, const float *ln_bias, float ln_eps,
                                                 const float *diag, const float *proj_bias, uint32_t *records,
-                                                int64_t record_stride, int64_t B, int64_t H, int64_t D, int64_t R,
-                                                int64_t J, int64_t T, float decay, float residual, void *stream) {
+                                                int64_t record_stride, int32_t tokens_per_workgroup, int64_t B,
+                                                int64_t H, int64_t D, int64_t R, int64_t J, int64_t T, float decay,
+                                                float residual, void *stream) {
     LFFN_REQUIRE(ln_eps >= 0.f && ((ln_weight && ln_bias) || (!ln_weight && !ln_bias)), LFFN_ERR_BAD_ARG);
-    LFFN_REQUIRE(records && record_stride >= B && T % 2 == 0, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(records && T % 2 == 0 && B >= 0, LFFN_ERR_BAD_ARG);
+    LFFN_REQUIRE(lffn_record_layout_ok(B, record_stride, tokens_per_workgroup) && (uintptr_t)records % 4 == 0,
+                 LFFN_ERR_BAD_ARG);
     LFFN_REQUIRE(D >= 16, LFFN_ERR_UNSUPPORTED);           // a table pair's 16 values within an aligned lane quad
     return project_hash_impl(x, ln_weight, ln_bias, ln_eps, diag, proj_bias, nullptr, nullptr, nullptr,
-                             B, H, D, R, J, T, decay, residual, stream, records, record_stride);
+                             B, H, D, R, J, T, decay, residual, stream, records, record_stride, tokens_per_workgroup);
 }
 
 extern "C" int lffn_project_hash_f32(const float *x, const float *diag, const float *proj_bias,
@@ -951,7 +960,8 @@ static int project_hash_impl(const float *x, const float *ln_w, const float *ln_
                              const float *diag, const float *proj_bias,
                              float *z_out, int32_t *codes, float *scores,
                              int64_t B, int64_t H, int64_t D, int64_t R, int64_t J, int64_t T,
-                             float decay, float residual, void *stream, uint32_t *records, int64_t record_stride) {
+                             float decay, float residual, void *stream, uint32_t *records, int64_t record_stride,
+                             int record_tile) {
     LFFN_REQUIRE(x && diag && ((codes && scores) || records), LFFN_ERR_BAD_ARG);
     int rc = check_dims(B, H, D, R, J);
     if (rc != LFFN_OK) return rc;
@@ -962,7 +972,7 @@ static int project_hash_impl(const float *x, const float *ln_w, const float *ln_
                  LFFN_ERR_BAD_ARG);
     ProjectArgs a{};
     a.x = x; a.diag = diag; a.pbias = proj_bias; a.out = z_out; a.codes = codes; a.scores = scores;
-    a.records = records; a.rec_stride = record_stride;
+    a.records = records; a.rec_stride = record_stride; a.rec_tile = record_tile;
     a.ln_w = ln_w; a.ln_b = ln_b; a.ln_eps = ln_eps;
     a.B = B; a.H = (int)H; a.R = (int)R; a.J = (int)J;
     a.out_stride = (int)(T * 8); a.out_cols = (int)(T * 8); a.T = (int)T;

@@ -100,6 +100,30 @@ int lffn_internal_lookup_gather_quad_records(const uint32_t *records, int64_t re
                                              const float *bias, const float *residual, float *out, int64_t B,
                                              int64_t T, int64_t S, int64_t Do, int fmt, int tokens, void *stream);
 
+// The record stream of the four-lanes-per-token gather (lookup_gather_quad.hip), as its writers address it.
+// A record is three words: score of the pair's first table, score of its second, row of the first | row of
+// the second << 8, where token b takes the tables of pair k in the order (2k, 2k+1) when bit 1 of b is clear
+// and (2k+1, 2k) when it is set.  Records are kept per table pair, record_stride slots of 12 bytes each, in
+// the order the gather's wavefronts copy them: a tile of tile_tokens tokens (a multiple of 16 in
+// (256 (np-1), 256 np]) is np passes of 16 wavefronts x 16 tokens, group p*16 + w of the tile being pass p of
+// wavefront w; a wavefront's records of all its passes are contiguous (pass-major), the wavefronts follow each
+// other, the tiles follow each other: slot = tile * tile_tokens + first slot of the wavefront + pass * 16 +
+// token within the group.  Wavefronts below n_last = tile_tokens/16 - 16 (np-1) have np passes, the others np-1.
+__host__ __device__ __forceinline__ int64_t lffn_quad_record_slot(int64_t token, int tile_tokens) {
+    const int npm1 = (tile_tokens - 1) >> 8;                  // passes - 1
+    const int n_last = (tile_tokens >> 4) - 16 * npm1;
+    const int64_t tile = token / tile_tokens;
+    const int r = (int)(token - tile * tile_tokens);
+    const int group = r >> 4, wave = group & 15, pass = group >> 4;
+    return tile * tile_tokens + 16 * (npm1 * wave + (wave < n_last ? wave : n_last)) + pass * 16 + (r & 15);
+}
+constexpr int LFFN_RECORD_WORDS = 3;
+// what a writer of records checks: a tile size the slots are defined for and room for every tile
+static inline bool lffn_record_layout_ok(int64_t B, int64_t record_stride, int64_t tile_tokens) {
+    return tile_tokens >= 16 && tile_tokens <= 2048 && tile_tokens % 16 == 0 &&
+           record_stride >= (B + tile_tokens - 1) / tile_tokens * tile_tokens;
+}
+
 // lookup_inner.hip: the four-lanes-per-token score gradient where the shape qualifies (not exported)
 __attribute__((visibility("hidden")))
 bool lffn_internal_lookup_inner_quad_try(const int32_t *code, const float *g, int64_t g_token_stride,

@@ -921,7 +921,8 @@ extern "C" int lffn_lookup_gather_records_rows(const uint32_t *records, int64_t 
                  LFFN_ERR_UNSUPPORTED);
     LFFN_REQUIRE(tables && out && (records || B == 0), LFFN_ERR_BAD_ARG);
     LFFN_REQUIRE(lffn_aligned16(tables) && lffn_aligned16(out) && (!bias || lffn_aligned16(bias)) &&
-                     (!residual || lffn_aligned16(residual)) && (uintptr_t)records % 4 == 0, LFFN_ERR_BAD_ARG);
+                     (!residual || lffn_aligned16(residual)) && lffn_aligned16(records) && record_stride % 4 == 0,
+                 LFFN_ERR_BAD_ARG);
     if (B == 0) return LFFN_OK;
     return lffn_internal_lookup_gather_quad_records(records, record_stride, tables, bias, residual, out, B, T, S, Do,
                                                     row_format, tokens_per_workgroup, stream);

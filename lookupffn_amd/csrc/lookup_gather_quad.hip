@@ -19,17 +19,19 @@
 //     select, and rotate through the four columns over the four reads of a table pair.  So the
 //     order in which a quad adds the pair's two tables depends on the quad (2k then 2k+1, or the
 //     reverse); each token still adds its T rows one at a time in fp32;
-//   * (code, score) pairs come from a stream of records, three words per (table pair, token) kept as
-//     three planes [table pair][word][token], that a small kernel packs first (the caller's [B, T]
-//     arrays have a token's pair 8 bytes wide in rows T*4 bytes apart: sixteen cache lines per
-//     wavefront load).  A wavefront copies the records of its 16*NP tokens for the NEXT table pair
-//     straight from global memory into its own corner of LDS while it works on the current one (no
-//     registers, nothing to wait for), reads them from there at the start of the step, two records
-//     per lane, and hands them round the quad with DPP quad_perm moves.  Six registers hold a lane's
-//     records, against 3*NP when they were loaded a chunk of tables ahead.  (Planes, because a
-//     global -> LDS copy places its lanes' data 4 bytes apart for one word per lane but 16 bytes
-//     apart for three or four: as planes the records take 12 bytes each in LDS, and 2048 tokens'
-//     worth fits beside the two table buffers.)
+//   * (code, score) pairs come from a stream of records, three words per (table pair, token), that a
+//     small kernel packs first (the caller's [B, T] arrays have a token's pair 8 bytes wide in rows
+//     T*4 bytes apart: sixteen cache lines per wavefront load).  The stream keeps, per table pair, the
+//     records in the order the wavefronts use them (lffn_quad_record_slot in lffn_common.h): all the
+//     records a wavefront needs for a pair, 16 tokens x its passes, are one contiguous run of 192
+//     bytes per pass.  A wavefront copies that run for the NEXT table pair straight from global
+//     memory into its own corner of LDS while it works on the current one (one or two 16-byte-per-
+//     lane copy instructions, no registers, nothing to wait for), reads its records from there at the
+//     start of the step, two per lane, and hands them round the quad with DPP quad_perm moves.  Six
+//     registers hold a lane's records, against 3*NP when they were loaded a chunk of tables ahead.
+//     (As three planes indexed by token, which is how the stream was laid out first, the same copy
+//     took six one-word-per-lane instructions, and the vector memory path is as busy as the LDS:
+//     105 -> 100 us at 16384 tokens x 128 tables x 768.)
 //
 // One barrier per table pair; the global -> LDS copy of pair k+1 has the whole of pair k's work to land.
 //
@@ -54,14 +56,14 @@ constexpr int fmt_bytes(int fmt) { return fmt == FMT_F32 ? 4 : 2; }
 constexpr int QUAD_TOUCH_AHEAD = 3;         // pairs between the one being read and the one being touched
 
 // (code, score) of one token and one table pair in the order the token's quad takes the pair's tables
-// (tokens whose index has bit 1 set take table 2k+1 first): three words, stored as three planes of
-// Bpad words per table pair: word 0 = score of the first table, 1 = score of the second, 2 = row of the
-// first table | row of the second << 8.
+// (tokens whose index has bit 1 set take table 2k+1 first): three words, word 0 = score of the first
+// table, 1 = score of the second, 2 = row of the first table | row of the second << 8; where a token's
+// record sits among its pair's: lffn_quad_record_slot.
 struct PairRecord {
     float score_first, score_second;
     uint32_t rows;
 };
-constexpr int REC_WORDS = 3;
+constexpr int REC_WORDS = LFFN_RECORD_WORDS;
 
 struct QuadArgs {
     const char *tables;    // [T, S, Do] fp32, bfloat16 or half
@@ -73,8 +75,8 @@ struct QuadArgs {
     int ntiles, nslices, per_xcd;
     int tile_tokens;       // tokens per tile: a multiple of 16 in ((NP - 1) * 256, NP * 256]
     int row_bytes;         // Do * bytes per element
-    const uint32_t *stream;     // [T/2][3][Bpad] record words written by pack_pairs_kernel
-    int64_t Bpad;               // words per plane: covers every token slot of every tile (lffn_internal_quad_record_stride)
+    const uint32_t *stream;     // [T/2][Bpad][3] record words written by pack_pairs_kernel
+    int64_t Bpad;               // record slots per table pair: every tile's tile_tokens (lffn_internal_quad_record_stride)
 };
 
 // global_load_lds_dwordx4 / _dword with a scalar base and a 32-bit lane offset: lane i of the
@@ -100,13 +102,12 @@ __device__ __forceinline__ void lds_dma4(const char *base, uint32_t lane_offset,
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x3 __attribute__((ext_vector_type(3)));
 typedef __attribute__((address_space(3))) const u32x4 *lds_vec_ptr;
-// a record in LDS: its three words are PLANE words apart
+// a record in LDS: three consecutive words
 struct LdsRecord { unsigned x, y, z; };
 typedef __attribute__((address_space(3))) const unsigned *lds_word_ptr;
-template <int PLANE>
 __device__ __forceinline__ LdsRecord read_record(unsigned lds_byte_addr) {
     lds_word_ptr p = (lds_word_ptr)(uintptr_t)lds_byte_addr;
-    return LdsRecord{p[0], p[PLANE], p[2 * PLANE]};
+    return LdsRecord{p[0], p[1], p[2]};
 }
 
 // Value held by lane N of the caller's quad, in every lane of the quad (one DPP move).
@@ -123,12 +124,13 @@ __device__ __forceinline__ unsigned with_row(unsigned base, unsigned packed) {
     return __builtin_amdgcn_perm(packed, base, 0x03020000u | ((4u + BYTE) << 8));
 }
 
-// Packs the caller's [B, T] codes and scores into the record stream [T/2][3][Bpad].  A workgroup takes 64
+// Packs the caller's [B, T] codes and scores into the record stream [T/2][Bpad][3].  A workgroup takes 64
 // tokens x 32 table pairs: it reads them pair-fastest (a token's 32 pairs are 256 contiguous bytes),
-// turns them round in LDS and writes them token-fastest (64 tokens' words of a plane are 256 contiguous
-// bytes).  Tokens from B up to Bpad (whole tiles of the gather kernel) get all-zero records.
+// turns them round in LDS and writes them token-fastest (16 consecutive tokens' records of a pair are 192
+// contiguous bytes).  Slots of tokens from B on are left as they are: the gather reads them (their row
+// numbers are bytes, always inside the LDS buffer) and does not store their sums.
 __global__ __launch_bounds__(256) void pack_pairs_kernel(const int32_t *code, const float *score, uint32_t *stream,
-                                                         int64_t B, int64_t Bpad, int T, int S) {
+                                                         int64_t B, int64_t Bpad, int T, int S, int tile_tokens) {
     __shared__ PairRecord tile[32][64 + 1];
     const int npairs = T / 2;
     const int64_t tok0 = int64_t(blockIdx.x) * 64;
@@ -151,16 +153,17 @@ __global__ __launch_bounds__(256) void pack_pairs_kernel(const int32_t *code, co
         tile[kk][row] = r;
     }
     __syncthreads();
+    const int row = threadIdx.x & 63;
+    const int64_t slot = tok0 + row < B ? lffn_quad_record_slot(tok0 + row, tile_tokens) : 0;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        const int item = threadIdx.x + 256 * i;
-        const int row = item & 63, kk = item >> 6;
-        if (tok0 + row < Bpad && k0 + kk < npairs) {
-            uint32_t *dst = stream + int64_t(k0 + kk) * REC_WORDS * Bpad + tok0 + row;
+        const int kk = (threadIdx.x >> 6) + 4 * i;
+        if (tok0 + row < B && k0 + kk < npairs) {
+            uint32_t *dst = stream + (int64_t(k0 + kk) * Bpad + slot) * REC_WORDS;
             const PairRecord r = tile[kk][row];
             dst[0] = __float_as_uint(r.score_first);
-            dst[Bpad] = __float_as_uint(r.score_second);
-            dst[2 * Bpad] = r.rows;
+            dst[1] = __float_as_uint(r.score_second);
+            dst[2] = r.rows;
         }
     }
 }
@@ -197,8 +200,7 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
     static_assert(NP >= 4 && NP <= 8, "a lane reads the records of passes l and l + 4");
     constexpr int EPV = 16 / fmt_bytes(FMT);              // columns in a 16-byte piece
     constexpr int SLICE_COLS = SLICE_BYTES / fmt_bytes(FMT);
-    constexpr int WAVE_RECS = 16 * NP;                    // records a wavefront uses per table pair
-    constexpr int REC_LOADS = (WAVE_RECS + 63) / 64;      // one-word-per-lane copy instructions per plane
+    constexpr int WAVE_RECS = 16 * NP;                    // records a wavefront uses per table pair, at most
     extern __shared__ uint4 lds[];                // 2 buffers of BUF_BYTES, the touches' sink, the wavefronts' records
 
     const int xcd = blockIdx.x % XCDS;
@@ -223,7 +225,8 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
     // are 1648 each, six passes and seven of sixteen wavefronts in the seventh, instead of nine full tiles of
     // 1792 and a tenth that is mostly padding).
     const int64_t tok0 = int64_t(tile) * a.tile_tokens + wave * 16 + quad;
-    const bool last_pass = (NP - 1) * 256 + wave * 16 < a.tile_tokens;        // uniform over the wavefront
+    const int n_last = a.tile_tokens / 16 - 16 * (NP - 1);                     // wavefronts that have the last pass
+    const bool last_pass = wave < n_last;                                      // uniform over the wavefront
 
     // acc[p][h][e]: token tok0 + 256 p, column ((half0 ^ h) * 4 + l) * EPV + e of the slice
     float acc[NP][2][EPV];
@@ -284,30 +287,24 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
     int turn = 0;                                   // k mod ntiles, kept without a division
     const uint32_t touch_dst = lds0 + 2u * BUF_BYTES;
 
-    // This wavefront's records: 16*NP per table pair, record r = pass r/16, quad r%16; word w of record r
-    // at rec_lds + 4 (w * WAVE_RECS + r).  Copy instruction (w, n) brings word w of records 64n .. 64n+63
-    // (lane i: record 64n + i), one word per lane.
+    // This wavefront's records of a table pair: 16 per pass, record r = pass r/16, quad r%16, 12 bytes each,
+    // one contiguous run in the stream (lffn_quad_record_slot) and, copied as it is, at rec_lds + 12 r in
+    // LDS.  12 NPW lanes copy 16 bytes each: one instruction up to five passes, two beyond.
     const uint32_t rec_lds = lds0 + 2u * BUF_BYTES + TOUCH_SINK_BYTES + (uint32_t)wave * (WAVE_RECS * REC_WORDS * 4);
-    const char *rec_base = reinterpret_cast<const char *>(a.stream + int64_t(tile) * a.tile_tokens + wave * 16);
-    const size_t plane_bytes = (size_t)a.Bpad * 4;
-    // byte offset of word 0 of record (pass, quad) from rec_base: pass * 256 tokens further on
-    const uint32_t rec_off = (uint32_t)(((lane >> 4) * 256 + (lane & 15)) * 4);
-    auto copy_records_to_lds = [&](int k) {
-        const char *src = rec_base + (size_t)k * REC_WORDS * plane_bytes;
-#pragma unroll
-        for (int n = 0; n < REC_LOADS; ++n) {
-            // passes 4n .. 4n+3: the last instruction of NP = 6, 7 has lanes beyond the tile's passes
-            if (64 * n + 64 <= WAVE_RECS || lane < WAVE_RECS - 64 * n) {
-#pragma unroll
-                for (int w = 0; w < REC_WORDS; ++w)
-                    lds_dma4(src + (size_t)w * plane_bytes + (size_t)n * (4 * 256 * 4), rec_off,
-                             rec_lds + (uint32_t)(w * WAVE_RECS + n * 64) * 4u);
-            }
+    const int wave_slot = 16 * ((NP - 1) * wave + min(wave, n_last));
+    const char *rec_base = reinterpret_cast<const char *>(a.stream + (int64_t(tile) * a.tile_tokens + wave_slot) * REC_WORDS);
+    const size_t pair_rec_bytes = (size_t)a.Bpad * (REC_WORDS * 4);
+    auto copy_records_to_lds = [&](int k, auto npw_c) {
+        constexpr int NV = 12 * decltype(npw_c)::value;         // 16-byte vectors
+        const char *src = rec_base + (size_t)k * pair_rec_bytes;
+        if (NV >= 64 || lane < NV) lds_dma16(src, (uint32_t)lane * 16u, rec_lds);
+        if constexpr (NV > 64) {
+            if (lane < NV - 64) lds_dma16(src + 1024, (uint32_t)lane * 16u, rec_lds + 1024u);
         }
     };
     // lane l of a quad reads the records of passes l and l + 4 (clamped: NP = 4..7 have fewer than 8)
-    const uint32_t rec_read0 = rec_lds + (uint32_t)((l * 16 + quad) * 4);
-    const uint32_t rec_read1 = rec_lds + (uint32_t)((min(l + 4, NP - 1) * 16 + quad) * 4);
+    const uint32_t rec_read0 = rec_lds + (uint32_t)((l * 16 + quad) * (REC_WORDS * 4));
+    const uint32_t rec_read1 = rec_lds + (uint32_t)((min(l + 4, NP - 1) * 16 + quad) * (REC_WORDS * 4));
 
     // LDS byte addresses of this lane's four reads of a pair, row field (byte 1) still empty: read i
     // takes table (i >> 1) of the quad's order, half (i & 1) of its order.  Bit 16 selects the buffer and
@@ -320,7 +317,13 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
         base[i] = lds0 + (unsigned)(table_sel * 128 + half * 64 + l * 16);
     }
 
-    copy_records_to_lds(0);
+    // The loop over the table pairs for a wavefront that takes NPW of the NP passes (NP, or NP - 1 when its group
+    // of the last pass lies beyond the tile): two copies of the loop, chosen once, so that neither has a branch
+    // inside (a conditional in the loop body, even a uniform one, costs this kernel hundreds of spilled
+    // registers).  Both copies meet at the same barriers.
+    auto run_pairs = [&](auto npw_c) {
+    constexpr int NPW = decltype(npw_c)::value;
+    copy_records_to_lds(0, npw_c);
     copy_pair_to_lds(slice_base, lds0);
     __builtin_amdgcn_s_waitcnt(WAIT_VMCNT_0);
     // A pair's records: x, y = the scores and z = the row numbers (first | second << 8), in the order the
@@ -328,18 +331,12 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
     // for its own copies, so they are read BEFORE the barrier: their latency is out of the way when the
     // barrier opens and the first row reads go out at once.  (The copies are inline assembly: the compiler
     // does not know that they write LDS nor that the wait is what completes them, so an ordering point it
-    // does honour keeps the reads below the wait.)
+    // does honour keeps the reads below the wait.)  A lane whose pass l + 4 is beyond NPW reads a record
+    // that is not this step's (or not written at all): it is never used.
     asm volatile("" ::: "memory");
-    LdsRecord rec0 = read_record<WAVE_RECS>(rec_read0);
-    LdsRecord rec1 = read_record<WAVE_RECS>(rec_read1);
+    LdsRecord rec0 = read_record(rec_read0);
+    LdsRecord rec1 = read_record(rec_read1);
     __syncthreads();
-
-    // The loop over the table pairs for a wavefront that takes NPW of the NP passes (NP, or NP - 1 when its group
-    // of the last pass lies beyond the tile): two copies of the loop, chosen once, so that neither has a branch
-    // inside (a conditional in the loop body, even a uniform one, costs this kernel hundreds of spilled
-    // registers).  Both copies meet at the same barriers.
-    auto run_pairs = [&](auto npw_c) {
-    constexpr int NPW = decltype(npw_c)::value;
     for (int k = 0; k < npairs; ++k) {
 
         // Software pipeline over the passes: a pass's four rows are requested while the pass before
@@ -371,7 +368,7 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
         // barrier); the last step copies the last pair's again.
         asm volatile("" : "+v"(rec0.x), "+v"(rec0.y), "+v"(rec0.z), "+v"(rec1.x), "+v"(rec1.y), "+v"(rec1.z));
         const int kn = min(k + 1, npairs - 1);
-        copy_records_to_lds(kn);
+        copy_records_to_lds(kn, npw_c);
         copy_pair_to_lds(slice_base + (size_t)kn * pair_stride, lds0 + (uint32_t)((k + 1) & 1) * BUF_BYTES);
         if constexpr (TOUCH) {
             const bool mine = turn == tile;                              // uniform
@@ -412,8 +409,8 @@ __global__ __launch_bounds__(WG) void lookup_gather_quad_kernel(QuadArgs a) {
         // the next pair's records (this wavefront's own, just landed; kept below the wait by the ordering
         // point), then the barrier for the segments
         asm volatile("" ::: "memory");
-        rec0 = read_record<WAVE_RECS>(rec_read0);
-        rec1 = read_record<WAVE_RECS>(rec_read1);
+        rec0 = read_record(rec_read0);
+        rec1 = read_record(rec_read1);
         __syncthreads();
     }
     };
@@ -481,16 +478,16 @@ int lffn_internal_quad_passes(int fmt, int64_t tokens) {
     return 0;
 }
 
-// Words per plane of the record stream for B tokens in tiles of `tokens`: the last tile's slots run to its
-// last pass's end whatever B is, since the gather copies a workgroup's records by whole passes.
+// Record slots per table pair for B tokens in tiles of `tokens`: whole tiles (a multiple of 16, fewer than
+// B + 2048).
 int64_t lffn_internal_quad_record_stride(int64_t B, int fmt, int64_t tokens) {
-    const int np = lffn_internal_quad_passes(fmt, tokens);
-    const int64_t ntiles = (B + tokens - 1) / tokens;
-    return (ntiles > 0 ? (ntiles - 1) * tokens : 0) + 256 * int64_t(np);      // < B + 2048
+    (void)fmt;
+    return (B + tokens - 1) / tokens * tokens;
 }
 
-// Run the gather from a record stream [T/2][3][record_stride] (pack_pairs_kernel's layout; the projection
-// kernel of fht.hip writes the same) with `tokens` tokens per workgroup.  The caller has checked that the
+// Run the gather from a record stream [T/2][record_stride][3] (pack_pairs_kernel's layout; the projection
+// kernels of fht.hip and bh4_block.hip write the same) with `tokens` tokens per workgroup, the tile size
+// the stream was written for.  The caller has checked that the
 // shape qualifies: S = 256 (a table pair fills an LDS buffer), T even, Do a multiple of the slice's columns
 // (32 for fp32 rows, 64 for 16-bit rows), 2*S*Do*element bytes < 2^32 (32-bit lane offsets from a table
 // pair's base), a tile size the format is built for.  record_stride: at least
@@ -501,7 +498,10 @@ int lffn_internal_lookup_gather_quad_records(const uint32_t *records, int64_t re
                                              int64_t T, int64_t S, int64_t Do, int fmt, int tokens, void *stream) {
     const int np = lffn_internal_quad_passes(fmt, tokens);
     if (!records || S != MAX_S || T % 2 != 0 || np == 0 || tokens <= 256 * (np - 1)) return LFFN_ERR_BAD_ARG;
-    if (record_stride < lffn_internal_quad_record_stride(B, fmt, tokens)) return LFFN_ERR_BAD_ARG;
+    // 16-byte copies: the stream and every table pair's part of it on 16-byte boundaries
+    if (record_stride < lffn_internal_quad_record_stride(B, fmt, tokens) || record_stride % 4 != 0 ||
+        !lffn_aligned16(records))
+        return LFFN_ERR_BAD_ARG;
     const int esz = fmt_bytes(fmt);
     if (Do % (SLICE_BYTES / esz) != 0) return LFFN_ERR_BAD_ARG;
     QuadArgs a{};
@@ -532,11 +532,12 @@ int lffn_internal_lookup_gather_quad(const int32_t *code, const float *score, co
                                      const float *bias, const float *residual, float *out, int64_t B, int64_t T,
                                      int64_t S, int64_t Do, int fmt, int tokens, void *workspace, void *stream) {
     if (!workspace || S != MAX_S || T % 2 != 0 || lffn_internal_quad_passes(fmt, tokens) == 0) return LFFN_ERR_BAD_ARG;
+    if (B == 0) return LFFN_OK;
     uint32_t *recs = static_cast<uint32_t *>(workspace);
     const int64_t stride = lffn_internal_quad_record_stride(B, fmt, tokens);
-    const dim3 grid((unsigned)((stride + 63) / 64), (unsigned)((T / 2 + 31) / 32));
+    const dim3 grid((unsigned)((B + 63) / 64), (unsigned)((T / 2 + 31) / 32));
     hipLaunchKernelGGL(pack_pairs_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), code, score, recs, B,
-                       stride, (int)T, (int)S);
+                       stride, (int)T, (int)S, tokens);
     if (hipGetLastError() != hipSuccess) return LFFN_ERR_LAUNCH;
     return lffn_internal_lookup_gather_quad_records(recs, stride, tables, bias, residual, out, B, T, S, Do, fmt, tokens, stream);
 }

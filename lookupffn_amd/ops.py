@@ -869,7 +869,7 @@ def ln_project_hash_records_direct(x, ln_w, ln_b, eps, diag, pbias, T, decay, re
     with _dev_guard(x):
         rc = _lib.load().lffn_ln_project_hash_records_f32(
             x.data_ptr(), ln_w.data_ptr(), ln_b.data_ptr(), eps, diag.data_ptr(), None if pbias is None else pbias.data_ptr(),
-            records.data_ptr(), plan[1], B, H, D, R, J, T, decay, residual, _lib.stream_of(x))
+            records.data_ptr(), plan[1], plan[0], B, H, D, R, J, T, decay, residual, _lib.stream_of(x))
     if rc != 0:
         _lib.check(rc, f"lffn_ln_project_hash_records_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T})")
     return records
@@ -886,7 +886,7 @@ def ln_bh4_block_hash_records_direct(x, ln_w, ln_b, eps, w_folded, pbias, T, dec
     with _dev_guard(x):
         rc = _lib.load().lffn_ln_bh4_block_hash_records_f32(
             x.data_ptr(), ln_w.data_ptr(), ln_b.data_ptr(), eps, w_folded.data_ptr(), None if pbias is None else pbias.data_ptr(),
-            records.data_ptr(), plan[1], B, H, D, R, J, T, bs, decay, residual, _lib.stream_of(x))
+            records.data_ptr(), plan[1], plan[0], B, H, D, R, J, T, bs, decay, residual, _lib.stream_of(x))
     if rc != 0:
         _lib.check(rc, f"lffn_ln_bh4_block_hash_records_f32(B={B}, H={H}, D={D}, R={R}, J={J}, T={T})")
     return records

@@ -399,6 +399,24 @@ def lookup_gather_records_plan(B, T, S, Do):
     return tokens.value, stride.value, nbytes.value
 
 
+def record_slots(B, tokens):
+    """Where the records of tokens 0..B-1 sit among a table pair's, for a gather of `tokens` tokens per
+    workgroup: a tile is passes of 16 wavefronts x 16 tokens (group p*16 + w of the tile = pass p of wavefront
+    w), a wavefront's records of all its passes are contiguous, wavefronts and tiles follow each other."""
+    npm1 = (tokens - 1) // 256
+    n_last = tokens // 16 - 16 * npm1
+    b = np.arange(B, dtype=np.int64)
+    tile, r = b // tokens, b % tokens
+    group = r // 16
+    wave, pas = group % 16, group // 16
+    return tile * tokens + 16 * (npm1 * wave + np.minimum(wave, n_last)) + pas * 16 + r % 16
+
+
+def records_of_tokens(rec, T, stride, B, tokens):
+    """The record stream as [T/2, B, 3] words (token order)."""
+    return rec.reshape(T // 2, stride, 3)[:, record_slots(B, tokens), :]
+
+
 def layer_through_records(x, ln_w, ln_b, eps, diag, pbias, tables, obias, residual=None, decay=0.7, plan=None):
     """lffn_ln_project_hash_records_f32 followed by lffn_lookup_gather_records_f32; returns (output, records)."""
     B, H = x.shape
@@ -410,7 +428,7 @@ def layer_through_records(x, ln_w, ln_b, eps, diag, pbias, tables, obias, residu
     rd = None if residual is None else dev(residual)
     rec = torch.full((nbytes // 4,), -1, dtype=torch.int32, device=DEV)
     out = torch.full((B, Do), float("nan"), dtype=torch.float32, device=DEV)
-    _call("lffn_ln_project_hash_records_f32", p(xd), p(wd), p(bd), eps, p(dd), p(pd), p(rec), stride, B, H, D, R, J, T,
+    _call("lffn_ln_project_hash_records_f32", p(xd), p(wd), p(bd), eps, p(dd), p(pd), p(rec), stride, tokens, B, H, D, R, J, T,
           decay, 1.0 - decay)
     _call("lffn_lookup_gather_records_f32", p(rec), stride, p(td), p(od), p(rd), p(out), B, T, S, Do, tokens)
     return host(out), rec.cpu().numpy().view(np.uint32)

@@ -236,7 +236,7 @@ def test_gather_plans_are_consistent_over_a_grid_of_shapes():
     """Host-side sweep of the three gather queries over 15 000 shapes (ragged token counts, odd table
     counts, every row format).  Whenever the workspace entry point would run the four-lanes-per-token
     kernel, the record stream its plan describes fits the workspace the size query asked for, the tile
-    is one the kernel is built for and the planes cover every token slot of every tile; the stand-alone
+    is one the kernel is built for and a table pair's records cover every token slot of every tile; the stand-alone
     record plan obeys the same rules (it may choose the form for more shapes: its records come from the
     projection kernel, so it does not count a packing kernel)."""
     lib = _lib.load()
@@ -249,7 +249,7 @@ def test_gather_plans_are_consistent_over_a_grid_of_shapes():
         np_ = -(-tokens // 256)
         assert np_ in passes_built[fmt], (fmt, tokens)
         ntiles = -(-B // tokens)
-        assert stride == (ntiles - 1) * tokens + 256 * np_          # the last tile's slots are whole passes
+        assert stride == ntiles * tokens and stride % 16 == 0       # whole tiles: 16-byte copies stay aligned
         assert B <= stride < B + 2048
         assert nbytes == 6 * T * stride
 

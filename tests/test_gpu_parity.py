@@ -517,7 +517,7 @@ def test_ln_project_hash_matches_oracle(H, D, R, T):
 # workgroup of the projection kernel and a quad; two repeats of a short transform (rows shared by four
 # tokens per wavefront); an odd number of table pairs
 # what lffn_lookup_gather_records_plan picks at configs 2 and 3: (tokens per workgroup, record stride, bytes)
-CONFIG2_RECORD_PLAN = (1648, 16624, 6 * 128 * 16624)        # 10 tiles of 103 groups of 16 tokens x 24 slices
+CONFIG2_RECORD_PLAN = (1648, 16480, 6 * 128 * 16480)        # 10 tiles of 103 groups of 16 tokens x 24 slices
 CONFIG3_RECORD_PLAN = (2048, 16384, 6 * 512 * 16384)        # 8 tiles x 32 slices
 RECORD_LAYERS = [(16384, 768, 1024, 1, 128, 768, None), (4099, 768, 1024, 1, 128, 768, (1024, 5120)),
                  (5000, 100, 128, 2, 30, 128, (1536, 6144)), (2050, 64, 64, 1, 6, 64, (2048, 4096)),
@@ -550,13 +550,13 @@ def test_layer_through_the_record_stream_matches_the_two_kernel_form(B, H, D, R,
     assert not np.isnan(got).any()
     codes, scores, _ = cabi.ln_project_hash(x, ln_w, ln_b, 1e-5, diag, pbias, T)
     # the records, word for word
-    rec = rec.reshape(T // 2, 3, stride)[:, :, :B]
+    rec = cabi.records_of_tokens(rec, T, stride, B, tokens)                      # [T/2, B, 3]
     swap = ((np.arange(B) & 2) != 0)[None, :]
     c0, c1 = codes[:, 0::2].T, codes[:, 1::2].T                                  # [T/2, B]
     s0, s1 = scores[:, 0::2].T, scores[:, 1::2].T
-    assert np.array_equal(rec[:, 0].view(np.float32), np.where(swap, s1, s0))
-    assert np.array_equal(rec[:, 1].view(np.float32), np.where(swap, s0, s1))
-    assert np.array_equal(rec[:, 2], np.where(swap, c1 | (c0 << 8), c0 | (c1 << 8)).astype(np.uint32))
+    assert np.array_equal(np.ascontiguousarray(rec[:, :, 0]).view(np.float32), np.where(swap, s1, s0))
+    assert np.array_equal(np.ascontiguousarray(rec[:, :, 1]).view(np.float32), np.where(swap, s0, s1))
+    assert np.array_equal(rec[:, :, 2], np.where(swap, c1 | (c0 << 8), c0 | (c1 << 8)).astype(np.uint32))
     # the output: the same kernel at the same tile size through the workspace entry point, bit for bit
     rc, want_same = cabi.lookup_gather_ws_planned(codes, scores, tables, (3, tokens), bias=obias, residual=res)
     assert rc == 0 and np.array_equal(got, want_same)
@@ -589,15 +589,15 @@ def test_block_layer_through_the_record_stream(B, H, D, R, T, Do, tokens):
     d = cabi.dev
     xd, lw, lb, wd, pd, td, od = d(x), d(ln_w), d(ln_b), d(wf), d(pbias), d(tables), d(obias)
     cabi._call("lffn_ln_bh4_block_hash_records_f32", cabi.p(xd), cabi.p(lw), cabi.p(lb), float(np.float32(1e-5)), cabi.p(wd),
-               cabi.p(pd), cabi.p(rec), stride, B, H, D, R, J, T, bs, float(np.float32(0.7)), float(np.float32(1 - 0.7)))
+               cabi.p(pd), cabi.p(rec), stride, tokens, B, H, D, R, J, T, bs, float(np.float32(0.7)), float(np.float32(1 - 0.7)))
     cabi._call("lffn_lookup_gather_records_f32", cabi.p(rec), stride, cabi.p(td), cabi.p(od), None, cabi.p(out), B, T, S, Do, tokens)
-    r = rec.cpu().numpy().view(np.uint32).reshape(T // 2, 3, stride)[:, :, :B]
+    r = cabi.records_of_tokens(rec.cpu().numpy().view(np.uint32), T, stride, B, tokens)
     swap = ((np.arange(B) & 2) != 0)[None, :]
     c0, c1 = codes[:, 0::2].T, codes[:, 1::2].T
     s0, s1 = scores[:, 0::2].T, scores[:, 1::2].T
-    assert np.array_equal(r[:, 0].view(np.float32), np.where(swap, s1, s0))
-    assert np.array_equal(r[:, 1].view(np.float32), np.where(swap, s0, s1))
-    assert np.array_equal(r[:, 2], np.where(swap, c1 | (c0 << 8), c0 | (c1 << 8)).astype(np.uint32))
+    assert np.array_equal(np.ascontiguousarray(r[:, :, 0]).view(np.float32), np.where(swap, s1, s0))
+    assert np.array_equal(np.ascontiguousarray(r[:, :, 1]).view(np.float32), np.where(swap, s0, s1))
+    assert np.array_equal(r[:, :, 2], np.where(swap, c1 | (c0 << 8), c0 | (c1 << 8)).astype(np.uint32))
     rc, want = cabi.lookup_gather_ws_planned(codes, scores, tables, (3, tokens), bias=obias)
     assert rc == 0 and np.array_equal(cabi.host(out), want)
 
@@ -614,14 +614,22 @@ def test_record_stream_plan_and_refusals():
     assert bad(4096, 256, None, None, 256, 3000, 20, 256, 256, 1000) == _lib.LFFN_ERR_BAD_ARG            # not whole passes
     assert bad(4096, 256, None, None, 256, 3000, 20, 256, 256, 512) == _lib.LFFN_ERR_UNSUPPORTED         # two passes: not built
     assert bad(4096, 256, None, None, 256, 3000, 21, 256, 256, 1024) == _lib.LFFN_ERR_UNSUPPORTED        # odd T
-    assert bad(3008, 256, None, None, 256, 3000, 20, 256, 256, 1024) == _lib.LFFN_ERR_BAD_ARG            # stride short of the last tile's passes
+    assert bad(3008, 256, None, None, 256, 3000, 20, 256, 256, 1024) == _lib.LFFN_ERR_BAD_ARG            # stride short of the last tile
+    assert bad(3074, 256, None, None, 256, 3000, 20, 256, 256, 1024) == _lib.LFFN_ERR_BAD_ARG            # stride not a multiple of 4
+    assert lib.lffn_lookup_gather_records_f32(260, 4096, 256, None, None, 256, 3000, 20, 256, 256, 1024, None) \
+        == _lib.LFFN_ERR_BAD_ARG                                                                         # records not 16-byte aligned
     assert bad(4096, 256, None, None, 256, 3000, 20, 256, 256, 1032) == _lib.LFFN_ERR_BAD_ARG            # not whole groups of 16
     assert bad(8192, 256, None, None, 256, 3000, 20, 256, 256, 2304) == _lib.LFFN_ERR_UNSUPPORTED        # nine passes: not built
     assert bad(2048, 256, None, None, 256, 3000, 20, 256, 256, 1024) == _lib.LFFN_ERR_BAD_ARG            # stride < B
-    assert lib.lffn_ln_project_hash_records_f32(256, 256, 256, 1e-5, 256, None, 256, 100, 300, 64, 64, 1, 4, 6, 0.7, 0.3, None) \
-        == _lib.LFFN_ERR_BAD_ARG                                                                         # stride < B
-    assert lib.lffn_ln_project_hash_records_f32(256, 256, 256, 1e-5, 256, None, 256, 1024, 300, 64, 64, 1, 4, 5, 0.7, 0.3, None) \
+    # (x, ln_w, ln_b, eps, diag, bias, records, stride, tokens per workgroup, B, H, D, R, J, T, ...)
+    assert lib.lffn_ln_project_hash_records_f32(256, 256, 256, 1e-5, 256, None, 256, 100, 1024, 300, 64, 64, 1, 4, 6, 0.7, 0.3, None) \
+        == _lib.LFFN_ERR_BAD_ARG                                                                         # stride < a tile
+    assert lib.lffn_ln_project_hash_records_f32(256, 256, 256, 1e-5, 256, None, 256, 1024, 1024, 300, 64, 64, 1, 4, 5, 0.7, 0.3, None) \
         == _lib.LFFN_ERR_BAD_ARG                                                                         # odd T
+    assert lib.lffn_ln_project_hash_records_f32(256, 256, 256, 1e-5, 256, None, 256, 4096, 1000, 300, 64, 64, 1, 4, 6, 0.7, 0.3, None) \
+        == _lib.LFFN_ERR_BAD_ARG                                                                         # tile not whole groups of 16
+    assert lib.lffn_ln_bh4_block_hash_records_f32(256, 256, 256, 1e-5, 256, None, 256, 1024, 2064, 300, 64, 64, 1, 4, 6, 64, 0.7, 0.3, None) \
+        == _lib.LFFN_ERR_BAD_ARG                                                                         # tile beyond 2048
 
 
 @pytest.mark.parametrize("P,na,nb", [(1, 4, 0), (7, 64, 100), (512, 768, 768), (512, 4096, 1024), (1000, 260, 4),
