@@ -351,13 +351,16 @@ struct GatherPlan {
 };
 
 // The four-lanes-per-token kernel: microseconds per table pair of a workgroup = a fixed part (the 64 KB
-// copy, the records, the barrier) + a part per pass of 256 tokens.  Measured on MI355X at 4, 6, 7 and 8
-// passes of fp32 rows (5 passes were added later and lie on the same line): 1.40, 1.74, 1.93, 2.18 us, the same for 128 x 256 x 768 fp32 tables (in the memory-side
-// cache) and 512 x 256 x 1024 (537 MB, beyond it: the touch by turns hides the difference).  A pass over
-// 16-bit rows covers twice the columns and is bound by the vector ALU: QUAD_US_PER_PAIR_PASS_16[format].
+// copy, the records, the barrier) + a part per pass of 256 tokens, a short last pass counting by its share
+// of 256 tokens.  Measured on MI355X with 10 tiles x 24 slices of fp32 rows (128 x 256 x 768 tables, in the
+// memory-side cache): 1.23, 1.33, 1.52, 1.68, 1.85 us at 4 .. 8 passes, 1.58 at 6.44, 1.19 at 3.06 (the copies
+// bound the step below about 1.19 us); 512 x 256 x 1024 tables (537 MB, beyond the cache) cost 0.13 to 0.3 us
+// more per pair.  A pass over 16-bit rows covers twice the columns and is bound by the vector ALU.
 constexpr double QUAD_MARGIN = 0.92;      // the form must promise this much to be worth its workspace
-constexpr double QUAD_US_PER_PAIR = 0.62, QUAD_US_PER_PAIR_PASS = 0.195;
-constexpr double QUAD_US_PER_PAIR_PASS_16[3] = {0.0, 0.355, 0.26};     // indexed by LFFN_ROWS_*: bfloat16, half (measured at 4 passes)
+// indexed by LFFN_ROWS_*: fp32, bfloat16, half
+constexpr double QUAD_US_PER_PAIR[3] = {0.53, 0.56, 0.61};
+constexpr double QUAD_US_PER_PAIR_PASS[3] = {0.165, 0.36, 0.275};
+constexpr double QUAD_US_PER_PAIR_MIN = 1.19;
 
 template <bool BF16>
 GatherPlan plan_gather(int64_t B, int64_t T, int64_t S, int64_t Do) {
@@ -404,22 +407,23 @@ GatherPlan plan_quad(int fmt, int64_t B, int64_t T, int64_t S, int64_t Do, bool 
         return best;
     const int64_t nslices = Do / cols;
     if (((B + 1023) / 1024) * nslices < 192 || B * nslices > (int64_t(1) << 30)) return best;
-    const double per_pass = fmt == LFFN_ROWS_F32 ? QUAD_US_PER_PAIR_PASS : QUAD_US_PER_PAIR_PASS_16[fmt];
+    const double per_pass = QUAD_US_PER_PAIR_PASS[fmt], fixed = QUAD_US_PER_PAIR[fmt];
     for (int np : {4, 5, 6, 7, 8}) {
         if (!lffn_internal_quad_np_built(fmt, np)) continue;
         // Tiles of np passes, the tokens spread evenly over them in groups of 16: from as few tiles as np full
         // passes allow up to as many as still need np passes.  The last pass is then short for some of a
-        // workgroup's wavefronts, which leave it out; what a short pass costs was measured as about half a pass
-        // plus its share of the reads.  More, shorter tiles can fill workgroup slots that fewer, fuller ones leave
+        // workgroup's wavefronts, which leave it out: it costs its share of a pass.  More, shorter tiles can
+        // fill workgroup slots that fewer, fuller ones leave
         // idle (16384 tokens x 12 slices of 16-bit rows: 21 tiles of 784 tokens = 252 workgroups, not 16 x 12 = 192).
         const int64_t tiles_min = (B + 256 * np - 1) / (256 * np);
         for (int64_t tiles = tiles_min; tiles <= tiles_min + 32; ++tiles) {       // (filling a round of 256 workgroups never takes more)
             const int64_t tile = (((B + tiles - 1) / tiles) + 15) & ~int64_t(15);
             if (tile <= 256 * (np - 1)) break;
             const int64_t rem = tile - 256 * (np - 1);                                 // tokens in the last pass: 16 .. 256
-            const double passes = double(np - 1) + (rem == 256 ? 1.0 : 0.5 + 0.5 * double(rem) / 256.0);
+            const double passes = double(np - 1) + double(rem) / 256.0;
             const int64_t rounds = (tiles * nslices + 255) / 256;
-            const double us = double(rounds) * double(T / 2) * (QUAD_US_PER_PAIR + passes * per_pass) +
+            const double pair_us = fixed + passes * per_pass;
+            const double us = double(rounds) * double(T / 2) * (pair_us > QUAD_US_PER_PAIR_MIN ? pair_us : QUAD_US_PER_PAIR_MIN) +
                               (pack ? double(B) * double(T) * 14.0 / 3e6 + 4.0 : 0.0);     // packing: 8 bytes read, 6 written per (token, table)
             if (us < best.us) best = GatherPlan{3, np, us, (int)tile};
         }
