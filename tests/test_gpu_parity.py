@@ -1552,6 +1552,38 @@ def test_lookup_inner_full_size_duality():
     assert relmax(cabi.lookup_inner(code, 2.0 * g, tables), 2.0 * got.astype(np.float64)) <= 1e-6
 
 
+def test_half_backward_full_size_duality():
+    """The half-precision backward operators at the config-2 size (16384 tokens x 128 rows each, 768 columns,
+    Zipf(1.1) rows as in config 5): the forward, the inner product and the scatter-add are three views of one
+    trilinear form, sum_bi w[b,i] <g[b], src[idx[b,i]]>, so their totals agree; samples against float64."""
+    rng = np.random.RandomState(44)
+    B, T, S, Do = 16384, 128, 256, 768
+    p = 1.0 / np.arange(1, S + 1) ** 1.1
+    p /= p.sum()
+    code = rng.choice(S, size=(B, T), p=p).astype(np.int32)
+    idx = code + (np.arange(T, dtype=np.int32) * S)[None]
+    w = (1.0 - rng.rand(B, T)).astype(np.float32)
+    src = (0.02 * rng.randn(T * S, Do)).astype(np.float16)
+    g = rng.randn(B, Do).astype(np.float16)
+    fwd = cabi.gather_add(idx, src.view(np.uint16), w, fmt=cabi.ROWS_F16)                       # [B, Do]
+    inner = cabi.indexed_inner_product(idx, g.view(np.uint16), src.view(np.uint16))             # [B, T]
+    scat = cabi.scatter_add(idx, g.view(np.uint16), w, T * S)                                   # [T*S, Do]
+    a = float((fwd.astype(np.float64) * g.astype(np.float64)).sum())
+    b = float((inner.astype(np.float64) * w).sum())
+    c = float((scat.astype(np.float64) * src.astype(np.float64)).sum())
+    scale = float(np.abs(inner.astype(np.float64) * w).sum())
+    assert abs(a - b) <= 1e-5 * scale and abs(c - b) <= 1e-5 * scale
+    sub = slice(7000, 7100)
+    want = oracle.indexed_inner_product(idx[sub], g[sub].astype(np.float64), src.astype(np.float64))
+    assert relmax(inner[sub], want) <= 1e-5
+    # the hottest rows of a few tables against float64 sums over every token
+    for t in (0, 77, 127):
+        for c_ in (0, 1):
+            hit = code[:, t] == c_
+            want_row = (w[hit, t].astype(np.float64)[:, None] * g[hit].astype(np.float64)).sum(0)
+            assert relmax(scat[t * S + c_], want_row) <= 1e-5
+
+
 def test_scatter_duplicates_zipf():
     # heavy duplication of rows (BASELINE.json config 5 draws codes Zipf(1.1))
     rng = np.random.RandomState(40)
