@@ -349,7 +349,7 @@ def main_backward(args):
                            "derivative, transposed BH4(block 1)x4, grad of diagonals and bias"},
         # the sorted scatter reads every (token, table)'s 3 KB gradient row from L2 into registers (the
         # gradient matrix stays in the L2s) and writes each table row once: its bound is the L2 read path
-        "roofline": {"bound": "l2", "kernel": "lookup_scatter (three launches: transpose/pack, sort, sorted accumulate)",
+        "roofline": {"bound": "l2", "kernel": "lookup_scatter (three launches: transpose, sort + slice-major copy, sorted accumulate)",
                      "achieved": row_bytes / (scatter_ms * 1e-3) / 1e9, "peak": L2_READ_PEAK_GBS, "unit": "GB/s",
                      "frac": row_bytes / (scatter_ms * 1e-3) / 1e9 / L2_READ_PEAK_GBS,
                      "peak_basis": "16 channels x 128 B/clk per XCD x 8 XCDs x 2.4 GHz",

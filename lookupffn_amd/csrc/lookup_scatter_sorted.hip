@@ -3,19 +3,25 @@
 //   grad_tables[t][code[b][t]][:] += score[b][t] * g[b][:]        (PL/gather/cuda/kernel.py:190-202,
 //                                                                   PL/gather/cuda/extension/gather_kernel_fp32.cu:49)
 //
-// Three kernels and a workspace.
+// Three launches and a workspace.
 //
-// lookup_prep_kernel: lays the inputs out for the other two.  code and score are [B, T]; a
-// table's column is one value per 4*T bytes, and 64 lanes reading it are 64 separate
-// requests, which made the sort four times slower than it is.  The kernel writes them
-// transposed, [T, B] (codes masked, as 16-bit values), and copies g to a slice-major
-// layout [Do/32][B][32], in which the 128-byte row pieces of a slice are contiguous:
-// with rows 4*Do bytes apart the pieces of one slice fall on a quarter of the L2 channels.
+// lookup_prep_kernel: code and score are [B, T]; a table's column is one value per 4*T bytes,
+// and 64 lanes reading it are 64 separate requests, which made the sort four times slower
+// than it is.  The kernel writes them transposed, [T, B] (codes masked, as 16-bit values).
 //
-// lookup_sort_kernel: one workgroup per table sorts the tokens by their code for that
+// lookup_sort_pack_kernel: two jobs in one launch, by workgroup number.  The sort occupies one
+// workgroup per table (128 of the 256 compute units at 128 tables) and is bound by latency; the
+// copy of g to a slice-major layout [Do/32][B][32] (in which the 128-byte row pieces of a slice
+// are contiguous: with rows 4*Do bytes apart the pieces of one slice fall on a quarter of the L2
+// channels) is pure memory traffic and depends on nothing: its workgroups fill the rest of the
+// chip while the sort runs (23 + 25 us as two launches at 16384 tokens x 128 tables x 768).
+//
+// The sort: one workgroup per table sorts the tokens by their code for that
 // table (a stable counting sort: per-wavefront histograms over contiguous token ranges,
 // ranks inside a 64-token batch from ballots over the code bits) and writes (token, score)
-// pairs bucket by bucket.  Every bucket is padded to a multiple of eight entries with
+// pairs bucket by bucket: into LDS first (a 16-bit token and a score per entry: at most 18432
+// entries, 108 KB), from where the list goes to memory in whole lines; written straight
+// from the ranks, every wavefront store was 64 separate 8-byte requests.  Every bucket is padded to a multiple of eight entries with
 // (first token of the bucket, 0.0f), so that eight consecutive entries always belong to
 // one code, and the bucket boundaries are stored in units of eight entries.
 //
@@ -53,46 +59,48 @@ struct PrepArgs {
     float *score_t;        // [T, Bp]
     float *g_packed;       // [Do / SC][B][SC]
     int64_t B, Bp;
-    int T, S, Do, tiles_t, transpose_blocks;
+    int T, S, Do, tiles_t;
 };
 
-constexpr int PACK_TOKENS = 8;       // tokens per workgroup of the copy of g
-
+// one 64 x 64 tile of code and score per workgroup
 __global__ __launch_bounds__(256) void lookup_prep_kernel(PrepArgs a) {
     __shared__ int sc[64][65];
     __shared__ float ss[64][65];
     const int tid = threadIdx.x, lane = tid & 63, row0 = tid >> 6;
-    if ((int)blockIdx.x < a.transpose_blocks) {               // one 64 x 64 tile of code and score
-        const int64_t b0 = int64_t(blockIdx.x / a.tiles_t) * 64;
-        const int t0 = (blockIdx.x % a.tiles_t) * 64;
-        const int mask = a.S - 1;
-        for (int r = row0; r < 64; r += 4) {
-            const int64_t b = b0 + r;
-            const int t = t0 + lane;
-            if (b < a.B && t < a.T) {
-                sc[r][lane] = a.code[b * a.T + t] & mask;
-                ss[r][lane] = a.score[b * a.T + t];
-            }
+    const int64_t b0 = int64_t(blockIdx.x / a.tiles_t) * 64;
+    const int t0 = (blockIdx.x % a.tiles_t) * 64;
+    const int mask = a.S - 1;
+    for (int r = row0; r < 64; r += 4) {
+        const int64_t b = b0 + r;
+        const int t = t0 + lane;
+        if (b < a.B && t < a.T) {
+            sc[r][lane] = a.code[b * a.T + t] & mask;
+            ss[r][lane] = a.score[b * a.T + t];
         }
-        __syncthreads();
-        for (int r = row0; r < 64; r += 4) {
-            const int t = t0 + r;
-            const int64_t b = b0 + lane;
-            if (b < a.B && t < a.T) {
-                a.code_t[(size_t)t * a.Bp + b] = (uint16_t)sc[lane][r];
-                a.score_t[(size_t)t * a.Bp + b] = ss[lane][r];
-            }
+    }
+    __syncthreads();
+    for (int r = row0; r < 64; r += 4) {
+        const int t = t0 + r;
+        const int64_t b = b0 + lane;
+        if (b < a.B && t < a.T) {
+            a.code_t[(size_t)t * a.Bp + b] = (uint16_t)sc[lane][r];
+            a.score_t[(size_t)t * a.Bp + b] = ss[lane][r];
         }
-    } else {                                                  // PACK_TOKENS rows of g
-        const int64_t b0 = int64_t(blockIdx.x - a.transpose_blocks) * PACK_TOKENS;
-        const int q = a.Do / 4;
-        for (int e = tid; e < PACK_TOKENS * q; e += 256) {
-            const int64_t b = b0 + e / q;
-            const int col = (e % q) * 4;
-            if (b < a.B)
-                *reinterpret_cast<float4 *>(a.g_packed + ((size_t)(col / SC) * a.B + b) * SC + col % SC) =
-                    *reinterpret_cast<const float4 *>(a.g + (size_t)b * a.Do + col);
-        }
+    }
+}
+
+constexpr int PACK_TOKENS = 32;      // rows of g per workgroup of the slice-major copy
+
+// PACK_TOKENS rows of g, copied to the slice-major layout (workgroup `blk` of the copy)
+__device__ __forceinline__ void pack_rows(const PrepArgs &a, int64_t blk) {
+    const int64_t b0 = blk * PACK_TOKENS;
+    const int q = a.Do / 4;
+    for (int e = threadIdx.x; e < PACK_TOKENS * q; e += SORT_WG) {
+        const int64_t b = b0 + e / q;
+        const int col = (e % q) * 4;
+        if (b < a.B)
+            *reinterpret_cast<float4 *>(a.g_packed + ((size_t)(col / SC) * a.B + b) * SC + col % SC) =
+                *reinterpret_cast<const float4 *>(a.g + (size_t)b * a.Do + col);
     }
 }
 
@@ -103,9 +111,10 @@ struct SortArgs {
     int32_t *off8;         // [T, S + 1] bucket starts, in units of eight entries
     int64_t B, Bp, stride;
     int T, S, nbits;
+    int stage;             // the sorted list is collected in LDS and written out in whole lines (it fits: S <= 256)
 };
 
-__global__ __launch_bounds__(SORT_WG) void lookup_sort_kernel(SortArgs a) {
+__device__ __forceinline__ void sort_table(const SortArgs &a, const int t) {
     extern __shared__ int sm[];
     const int S = a.S;
     int *hist = sm;                    // [SORT_WAVES][S]: counts, then running write positions
@@ -113,8 +122,9 @@ __global__ __launch_bounds__(SORT_WG) void lookup_sort_kernel(SortArgs a) {
     int *start = count + S;            // padded bucket starts (entries)
     int *first = start + S;            // lowest token of the bucket
     int *total = first + S;
+    float *sc_s = reinterpret_cast<float *>(total + 4);                       // [stride] scores of the sorted list
+    unsigned short *tok_s = reinterpret_cast<unsigned short *>(sc_s + a.stride);   // [stride] tokens
 
-    const int t = blockIdx.x;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint16_t *code = a.code + (size_t)t * a.Bp;
     const float *score = a.score + (size_t)t * a.Bp;
@@ -122,24 +132,44 @@ __global__ __launch_bounds__(SORT_WG) void lookup_sort_kernel(SortArgs a) {
     for (int q = tid; q < S; q += SORT_WG) first[q] = 0x7fffffff;
     __syncthreads();
 
+    // A wavefront takes up to SORT_DEPTH batches of 64 consecutive tokens (the launch keeps B within 1024 * SORT_DEPTH).
+    // Their codes and scores are loaded once, all loads in flight together, and stay in registers through both
+    // passes, as does every token's rank among the tokens of its batch with the same code (from ballots over
+    // the code bits): the first pass counts a batch's codes once per code (the lowest lane of each adds the
+    // whole count: no two lanes of an instruction touch one counter, however skewed the codes are), the
+    // second turns ranks into positions.
     const int64_t per = ((a.B + SORT_WG - 1) / SORT_WG) * 64;       // tokens per wavefront, whole batches
     const int64_t lo = min<int64_t>(a.B, wave * per), hi = min<int64_t>(a.B, lo + per);
     int *myh = hist + wave * S;
-    // SORT_DEPTH batches of loads are issued together so that their latencies overlap
-    for (int64_t b0 = lo; b0 < hi; b0 += 64 * SORT_DEPTH) {
-        int cv[SORT_DEPTH];
+    int cv[SORT_DEPTH], rk[SORT_DEPTH];
+    float sv[SORT_DEPTH];
 #pragma unroll
-        for (int k = 0; k < SORT_DEPTH; ++k) {
-            const int64_t b = b0 + 64 * k + lane;                // loads are unconditional (clamped), so none waits for another
-            const int c = code[min<int64_t>(b, a.B - 1)];
-            cv[k] = b < hi ? c : -1;
+    for (int k = 0; k < SORT_DEPTH; ++k) {
+        const int64_t b = lo + 64 * k + lane;                    // loads are unconditional (clamped), so none waits for another
+        const int64_t bc = min<int64_t>(b, a.B - 1);
+        const int c = code[bc];
+        sv[k] = score[bc];
+        cv[k] = b < hi ? c : -1;
+    }
+#pragma unroll
+    for (int k = 0; k < SORT_DEPTH; ++k) {
+        rk[k] = 0;
+        if (lo + 64 * k >= hi) continue;                         // uniform
+        const bool live = cv[k] >= 0;
+        const int c = live ? cv[k] : 0;
+        unsigned long long m = __ballot(live);
+        for (int bit = 0; bit < a.nbits; ++bit) {
+            const bool mine = (c >> bit) & 1;
+            const unsigned long long bb = __ballot(mine);
+            m &= mine ? bb : ~bb;
         }
-#pragma unroll
-        for (int k = 0; k < SORT_DEPTH; ++k)
-            if (cv[k] >= 0) {
-                atomicAdd(&myh[cv[k]], 1);
-                atomicMin(&first[cv[k]], (int)(b0 + 64 * k + lane));
-            }
+        const int rank = __popcll(m & ((1ull << lane) - 1ull));
+        const int cnt = __popcll(m);
+        rk[k] = rank | (cnt << 8);
+        if (live && rank == 0) {
+            myh[c] += cnt;
+            atomicMin(&first[c], (int)(lo + 64 * k + lane));
+        }
     }
     __syncthreads();
     for (int c = tid; c < S; c += SORT_WG) {
@@ -186,42 +216,43 @@ __global__ __launch_bounds__(SORT_WG) void lookup_sort_kernel(SortArgs a) {
     __syncthreads();
 
     uint2 *out = a.pairs + (size_t)t * a.stride;
-    for (int64_t b0 = lo; b0 < hi; b0 += 64 * SORT_DEPTH) {
-        int cv[SORT_DEPTH];
-        float sv[SORT_DEPTH];
 #pragma unroll
-        for (int k = 0; k < SORT_DEPTH; ++k) {
-            const int64_t b = b0 + 64 * k + lane;
-            const int64_t bc = min<int64_t>(b, a.B - 1);
-            const int c = code[bc];
-            sv[k] = score[bc];
-            cv[k] = b < hi ? c : -1;
-        }
-#pragma unroll
-        for (int k = 0; k < SORT_DEPTH; ++k) {
-            if (b0 + 64 * k >= hi) break;                     // uniform
-            const bool live = cv[k] >= 0;
-            const int c = live ? cv[k] : 0;
-            unsigned long long m = __ballot(live);
-            for (int bit = 0; bit < a.nbits; ++bit) {
-                const bool mine = (c >> bit) & 1;
-                const unsigned long long bb = __ballot(mine);
-                m &= mine ? bb : ~bb;
+    for (int k = 0; k < SORT_DEPTH; ++k) {
+        if (lo + 64 * k >= hi) continue;                         // uniform
+        if (cv[k] >= 0) {
+            const int c = cv[k], rank = rk[k] & 0xff, cnt = rk[k] >> 8;
+            const int base = myh[c];                              // all lanes of a code read before its last lane writes
+            if (a.stage) {                                        // uniform
+                tok_s[base + rank] = (unsigned short)(lo + 64 * k + lane);
+                sc_s[base + rank] = sv[k];
+            } else {
+                out[base + rank] = make_uint2((unsigned)(lo + 64 * k + lane), __float_as_uint(sv[k]));
             }
-            const int rank = __popcll(m & ((1ull << lane) - 1ull));
-            const int cnt = __popcll(m);
-            if (live) {
-                const int base = myh[c];                      // all lanes of a code read before its last lane writes
-                out[base + rank] = make_uint2((unsigned)(b0 + 64 * k + lane), __float_as_uint(sv[k]));
-                if (rank == cnt - 1) myh[c] = base + cnt;
-            }
+            if (rank == cnt - 1) myh[c] = base + cnt;
         }
     }
     __syncthreads();
     for (int c = tid; c < S; c += SORT_WG) {
         const int n = count[c], o = start[c];
-        for (int p = n; p < ((n + 7) & ~7); ++p) out[o + p] = make_uint2((unsigned)first[c], 0u);
+        for (int p = n; p < ((n + 7) & ~7); ++p) {
+            if (a.stage) {
+                tok_s[o + p] = (unsigned short)first[c];
+                sc_s[o + p] = 0.f;
+            } else {
+                out[o + p] = make_uint2((unsigned)first[c], 0u);
+            }
+        }
     }
+    if (!a.stage) return;                                     // uniform
+    __syncthreads();
+    const int n_out = *total;
+    for (int i = tid; i < n_out; i += SORT_WG) out[i] = make_uint2((unsigned)tok_s[i], __float_as_uint(sc_s[i]));
+}
+
+// workgroups [0, nsort): the sort of one table each; the others: PACK_TOKENS rows of the copy of g each
+__global__ __launch_bounds__(SORT_WG) void lookup_sort_pack_kernel(SortArgs sa, PrepArgs pa, int nsort) {
+    if ((int)blockIdx.x < nsort) sort_table(sa, (int)blockIdx.x);      // uniform over the workgroup
+    else pack_rows(pa, int64_t(blockIdx.x) - nsort);
 }
 
 struct SortedArgs {
@@ -436,13 +467,33 @@ int sorted_backward(const int32_t *code, const float *score, const float *g, con
         pa.g_packed = reinterpret_cast<float *>(base + w.g_packed);
         pa.B = Bc; pa.Bp = Bp; pa.T = (int)T; pa.S = (int)S; pa.Do = (int)Do;
         pa.tiles_t = (int)((T + 63) / 64);
-        // (score gradient only: the codes and scores need no transposing, only g its slice-major copy)
+        // (score gradient only: the codes and scores need no transposing or sorting, only g its slice-major copy)
         const int64_t transpose_blocks = grad_tables ? (Bp / 64) * pa.tiles_t : 0;
         const int64_t pack_blocks = (Bc + PACK_TOKENS - 1) / PACK_TOKENS;
-        LFFN_REQUIRE(transpose_blocks + pack_blocks <= 0x7fffffff, LFFN_ERR_UNSUPPORTED);
-        pa.transpose_blocks = (int)transpose_blocks;
-        hipLaunchKernelGGL(lookup_prep_kernel, dim3((unsigned)(transpose_blocks + pack_blocks)), dim3(256), 0, st, pa);
-        int rc = lffn_launch_status();
+        const int64_t nsort = grad_tables ? T : 0;
+        LFFN_REQUIRE(transpose_blocks <= 0x7fffffff && nsort + pack_blocks <= 0x7fffffff, LFFN_ERR_UNSUPPORTED);
+        int rc = LFFN_OK;
+        if (transpose_blocks > 0) {
+            hipLaunchKernelGGL(lookup_prep_kernel, dim3((unsigned)transpose_blocks), dim3(256), 0, st, pa);
+            rc = lffn_launch_status();
+            if (rc != LFFN_OK) return rc;
+        }
+        SortArgs sa{};
+        sa.code = pa.code_t; sa.score = pa.score_t; sa.pairs = pairs; sa.off8 = off8;
+        sa.B = Bc; sa.Bp = Bp; sa.stride = stride; sa.T = (int)T; sa.S = (int)S; sa.nbits = lffn_log2(S);
+        // histograms and bucket tables, then the sorted list itself (4 + 2 bytes per entry; tokens of a chunk fit 16 bits)
+        static_assert(CHUNK <= 65536, "tokens of a chunk are staged as 16-bit values");
+        static_assert(CHUNK <= int64_t(SORT_WG) * SORT_DEPTH, "a wavefront of the sort holds its tokens in registers");
+        const size_t tables_lds = (size_t(SORT_WAVES) * S + 3 * S + 4 + 4) * sizeof(int);
+        const size_t staged_lds = tables_lds + size_t(stride) * 6 + 16;
+        sa.stage = staged_lds <= 160 * 1024 ? 1 : 0;            // 512-row tables: the list goes straight to memory
+        const size_t sort_lds = nsort ? (sa.stage ? staged_lds : tables_lds) : 0;
+        static LdsGrant granted;
+        if (!lffn_grant_dynamic_lds(reinterpret_cast<const void *>(lookup_sort_pack_kernel), sort_lds, granted))
+            return LFFN_ERR_LAUNCH;
+        hipLaunchKernelGGL(lookup_sort_pack_kernel, dim3((unsigned)(nsort + pack_blocks)), dim3(SORT_WG), sort_lds, st, sa, pa,
+                           (int)nsort);
+        rc = lffn_launch_status();
         if (rc != LFFN_OK) return rc;
 
         if (grad_score) {
@@ -453,14 +504,6 @@ int sorted_backward(const int32_t *code, const float *score, const float *g, con
             if (rc != LFFN_OK) return rc;
         }
         if (!grad_tables) continue;
-
-        SortArgs sa{};
-        sa.code = pa.code_t; sa.score = pa.score_t; sa.pairs = pairs; sa.off8 = off8;
-        sa.B = Bc; sa.Bp = Bp; sa.stride = stride; sa.T = (int)T; sa.S = (int)S; sa.nbits = lffn_log2(S);
-        const size_t sort_lds = (size_t(SORT_WAVES) * S + 3 * S + 4) * sizeof(int);
-        hipLaunchKernelGGL(lookup_sort_kernel, dim3((unsigned)T), dim3(SORT_WG), sort_lds, st, sa);
-        rc = lffn_launch_status();
-        if (rc != LFFN_OK) return rc;
 
         SortedArgs ma{};
         ma.pairs = pairs; ma.off8 = off8; ma.g = pa.g_packed; ma.out = grad_tables; ma.stride = stride;
