@@ -70,21 +70,30 @@ __global__ __launch_bounds__(256) void lookup_prep_kernel(PrepArgs a) {
     const int64_t b0 = int64_t(blockIdx.x / a.tiles_t) * 64;
     const int t0 = (blockIdx.x % a.tiles_t) * 64;
     const int mask = a.S - 1;
-    for (int r = row0; r < 64; r += 4) {
-        const int64_t b = b0 + r;
-        const int t = t0 + lane;
-        if (b < a.B && t < a.T) {
-            sc[r][lane] = a.code[b * a.T + t] & mask;
-            ss[r][lane] = a.score[b * a.T + t];
-        }
+    // all sixteen rows of a thread are requested before the first is used
+    int cv[16];
+    float sv[16];
+    const int t_in = t0 + lane;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int64_t b = b0 + row0 + 4 * i;
+        const bool live = b < a.B && t_in < a.T;
+        cv[i] = live ? a.code[b * a.T + t_in] : 0;
+        sv[i] = live ? a.score[b * a.T + t_in] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        sc[row0 + 4 * i][lane] = cv[i] & mask;
+        ss[row0 + 4 * i][lane] = sv[i];
     }
     __syncthreads();
-    for (int r = row0; r < 64; r += 4) {
-        const int t = t0 + r;
-        const int64_t b = b0 + lane;
-        if (b < a.B && t < a.T) {
-            a.code_t[(size_t)t * a.Bp + b] = (uint16_t)sc[lane][r];
-            a.score_t[(size_t)t * a.Bp + b] = ss[lane][r];
+    const int64_t b_out = b0 + lane;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int r = row0 + 4 * i, t = t0 + r;
+        if (b_out < a.B && t < a.T) {
+            a.code_t[(size_t)t * a.Bp + b_out] = (uint16_t)sc[lane][r];
+            a.score_t[(size_t)t * a.Bp + b_out] = ss[lane][r];
         }
     }
 }
@@ -95,12 +104,26 @@ constexpr int PACK_TOKENS = 32;      // rows of g per workgroup of the slice-maj
 __device__ __forceinline__ void pack_rows(const PrepArgs &a, int64_t blk) {
     const int64_t b0 = blk * PACK_TOKENS;
     const int q = a.Do / 4;
-    for (int e = threadIdx.x; e < PACK_TOKENS * q; e += SORT_WG) {
-        const int64_t b = b0 + e / q;
-        const int col = (e % q) * 4;
-        if (b < a.B)
-            *reinterpret_cast<float4 *>(a.g_packed + ((size_t)(col / SC) * a.B + b) * SC + col % SC) =
-                *reinterpret_cast<const float4 *>(a.g + (size_t)b * a.Do + col);
+    // eight loads per thread in flight before the first store (a store must not overtake a load the compiler
+    // cannot prove independent of it, so load-store pairs one after the other would each wait out a round trip)
+    constexpr int DEPTH = 8;
+    for (int e0 = threadIdx.x; e0 < PACK_TOKENS * q; e0 += SORT_WG * DEPTH) {
+        float4 v[DEPTH];
+#pragma unroll
+        for (int i = 0; i < DEPTH; ++i) {
+            const int e = e0 + i * SORT_WG;
+            const int64_t b = b0 + e / q;
+            v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (e < PACK_TOKENS * q && b < a.B) v[i] = *reinterpret_cast<const float4 *>(a.g + (size_t)b * a.Do + (e % q) * 4);
+        }
+#pragma unroll
+        for (int i = 0; i < DEPTH; ++i) {
+            const int e = e0 + i * SORT_WG;
+            const int64_t b = b0 + e / q;
+            const int col = (e % q) * 4;
+            if (e < PACK_TOKENS * q && b < a.B)
+                *reinterpret_cast<float4 *>(a.g_packed + ((size_t)(col / SC) * a.B + b) * SC + col % SC) = v[i];
+        }
     }
 }
 
